@@ -1,0 +1,198 @@
+// Quantised matmul for prefill (any M): y[M,N] = x[M,K] @ dq(W)[N,K]^T.
+//
+// Matrix-core design for gfx950: a 128x128 output tile per 256-thread workgroup, one
+// 64-wide K step per iteration = exactly one quantisation group, so every packed row
+// segment needs a single (scale, bias).  Each thread dequantises 32 (4-bit) or
+// 2x16 (8-bit) codes to bf16 in registers - bf16(fma(s, q, b)), codes converted with
+// v_cvt_f32_ubyteN - and stores them to LDS next to the activation tile; the four
+// waves (2x2) then issue v_mfma_f32_32x32x16_bf16 on 64x64 sub-tiles with float32
+// accumulators.  Global loads of the next K step are issued before the MFMAs of the
+// current one.  LDS rows are padded by 16 bytes to keep ds_read_b128 conflict-free.
+#include "../../include/exo_mi355x.h"
+#include "common.h"
+
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row
+constexpr int kThreads = 256;
+
+struct QmmParams {
+  const bf16_t* x;
+  const uint32_t* w;
+  const bf16_t* s;
+  const bf16_t* b;
+  const bf16_t* residual;
+  bf16_t* y;
+  int M, N, K;
+};
+
+template <int BITS>
+struct WFrag {  // one thread's share of the packed W tile for one K step
+  uint4 q[BITS / 4];  // 4-bit: 16 B = 32 codes; 8-bit: 2 x 16 B = 2 x 16 codes
+  float s, b;
+};
+
+__device__ __forceinline__ float ubyte_f(uint32_t v, int i) {
+  return (float)((v >> (8 * i)) & 0xffu);  // v_cvt_f32_ubyteN
+}
+
+template <int BITS>
+__global__ __launch_bounds__(kThreads) void qmm_kernel(const QmmParams p) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t ws[BN * LDS_STRIDE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int G = p.K >> 6;
+  const int wpr = p.K * BITS / 32;
+
+  // W: thread -> (row, part).  4-bit: 2 parts of 32 codes; 8-bit: 2 parts of 32 codes
+  // (two 16-byte loads each).
+  const int w_row = tid >> 1, w_part = tid & 1;
+  const bool w_ok = (n0 + w_row) < p.N;
+  const uint32_t* wsrc = p.w + (size_t)(n0 + (w_ok ? w_row : 0)) * wpr + w_part * (BITS);
+  const bf16_t* ssrc = p.s + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
+  const bf16_t* bsrc = p.b + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
+
+  uint4 xa[4];
+  WFrag<BITS> wf;
+
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int id = tid + kThreads * r;
+      const int row = id >> 3, kp = id & 7;
+      if (m0 + row < p.M)
+        xa[r] = *reinterpret_cast<const uint4*>(p.x + (size_t)(m0 + row) * p.K + k0 + kp * 8);
+      else
+        xa[r] = make_uint4(0, 0, 0, 0);
+    }
+    const int kw = k0 * BITS / 32;  // word offset of this K step
+#pragma unroll
+    for (int i = 0; i < BITS / 4; ++i)
+      wf.q[i] = *reinterpret_cast<const uint4*>(wsrc + kw + i * 4);
+    wf.s = bf2f(ssrc[k0 >> 6]);
+    wf.b = bf2f(bsrc[k0 >> 6]);
+    if (!w_ok) {
+      wf.s = 0.f;
+      wf.b = 0.f;
+    }
+  };
+
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int id = tid + kThreads * r;
+      const int row = id >> 3, kp = id & 7;
+      *reinterpret_cast<uint4*>(&xs[row * LDS_STRIDE + kp * 8]) = xa[r];
+    }
+    bf16_t* dst = &ws[w_row * LDS_STRIDE + w_part * 32];
+    const float s = wf.s, b = wf.b;
+    if (BITS == 4) {
+      const uint32_t* qw = reinterpret_cast<const uint32_t*>(&wf.q[0]);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {  // two 16-byte LDS stores of 8 codes... x2 words each
+        uint4 o[2];
+        uint32_t* o4 = reinterpret_cast<uint32_t*>(o);
+#pragma unroll
+        for (int wi = 0; wi < 2; ++wi) {
+          const uint32_t v = qw[h * 2 + wi];
+          const uint32_t ev = v & 0x0f0f0f0fu, od = (v >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o4[wi * 4 + e] = pack_bf2(fmaf(s, ubyte_f(ev, e), b), fmaf(s, ubyte_f(od, e), b));
+        }
+        *reinterpret_cast<uint4*>(dst + h * 16) = o[0];
+        *reinterpret_cast<uint4*>(dst + h * 16 + 8) = o[1];
+      }
+    } else {
+      const uint32_t* qw = reinterpret_cast<const uint32_t*>(&wf.q[0]);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {  // 8 codes (2 words) per 16-byte LDS store
+        uint4 o;
+        uint32_t* o4 = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int wi = 0; wi < 2; ++wi) {
+          const uint32_t v = qw[h * 2 + wi];
+          o4[wi * 2] = pack_bf2(fmaf(s, ubyte_f(v, 0), b), fmaf(s, ubyte_f(v, 1), b));
+          o4[wi * 2 + 1] = pack_bf2(fmaf(s, ubyte_f(v, 2), b), fmaf(s, ubyte_f(v, 3), b));
+        }
+        *reinterpret_cast<uint4*>(dst + h * 8) = o;
+      }
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int frow = lane & 31, fk = (lane >> 5) * 8;
+  load_global(0);
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    __syncthreads();  // previous step's LDS reads are done
+    store_lds();
+    __syncthreads();
+    if (k0 + BK < p.K) load_global(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      bf16x8_t a[2], bq[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const bf16x8_t*>(&xs[(wm + i * 32 + frow) * LDS_STRIDE + ks + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        bq[j] = *reinterpret_cast<const bf16x8_t*>(&ws[(wn + j * 32 + frow) * LDS_STRIDE + ks + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], bq[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // D[i][j]: column j = lane%32 (W row n), rows 8*(r/4) + 4*(lane/32) + r%4 (token m)
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < p.M && n < p.N) {
+          const size_t o = (size_t)m * p.N + n;
+          float v = acc[i][j][r];
+          if (p.residual) v = bf2f(f2bf(v)) + bf2f(p.residual[o]);
+          p.y[o] = f2bf(v);
+        }
+      }
+    }
+}
+
+}  // namespace
+
+extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M,
+                       int N, int K, int bits, int group_size, exo_stream_t stream) {
+  EXO_REQUIRE(bits == 4 || bits == 8, "exo_qmm: bits must be 4 or 8, got %d", bits);
+  EXO_REQUIRE(group_size == 64, "exo_qmm: group_size must be 64, got %d", group_size);
+  EXO_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 64 == 0, "exo_qmm: bad shape M=%d N=%d K=%d", M, N,
+              K);
+  EXO_REQUIRE(x && w && scales && biases && y, "exo_qmm: null pointer");
+  if (M == 0) return EXO_OK;
+  QmmParams p{x, w, scales, biases, residual, y, M, N, K};
+  dim3 grid(exo_ceil_div(N, BN), exo_ceil_div(M, BM));
+  EXO_REQUIRE(grid.y <= 65535, "exo_qmm: M=%d too large", M);
+  if (bits == 4)
+    qmm_kernel<4><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+  else
+    qmm_kernel<8><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+  EXO_CHECK_LAUNCH("exo_qmm");
+  return EXO_OK;
+}

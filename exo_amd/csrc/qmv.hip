@@ -1,0 +1,514 @@
+// Fused dequant-GEMV for decode (M <= 16): y = x @ dq(W)^T on MLX affine-packed W.
+//
+// HBM-bound design for gfx950:
+//  * every lane streams 16-byte pieces ("chunks") of a packed row with
+//    global_load_dwordx4; a row is covered by LPR lanes (power of two, 64 when the
+//    row is long enough) so that each load instruction of a wave reads 1 KiB that is
+//    contiguous per row; 8 such loads are in flight per lane before any is consumed.
+//  * codes are never converted one by one: a 4-bit word w gives four bf16x2 registers
+//    (w >> 4t) & 0x000F000F | 0x43004300 = (128+q_t, 128+q_{t+4}); v_dot2_f32_bf16
+//    multiplies them with the matching activation pair in float32.  The +128 is
+//    removed with the per-chunk activation sum: sum x*q = D - 128*sum(x).
+//    8-bit codes are treated as two nibbles against (x, 16x).
+//  * per chunk (half / quarter of a 64-group):  acc += s*(D - 128*Sx) + b*Sx.
+//  * activations sit in LDS, pre-permuted to the register order above and laid out
+//    so a wave's ds_read_b128 is conflict-free; per-chunk sums are precomputed once
+//    per workgroup.
+#include "../../include/exo_mi355x.h"
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr int kUnits = 8;  // 16-byte loads in flight per lane
+
+struct QmvParams {
+  const bf16_t* x;         // [M,K]
+  const uint32_t* w[2];    // packed [N, WPR]   ([1] only for the swiglu pair)
+  const bf16_t* s[2];      // [N, K/64]
+  const bf16_t* b[2];
+  const bf16_t* residual;  // [M,N] or null
+  bf16_t* y;               // [M,N]
+  int M, N, K;
+  int wpr;       // words per row
+  int lpr_log2;  // lanes per row
+  int iters;     // chunks per lane per row
+  int slots;     // ceil(N / (64/LPR)): wave-wide row sets
+  int spw;       // slots per wave
+  int ragged;    // N is not a multiple of 64/LPR: the last slot has rows >= N
+  // gather (MoE) mode: blockIdx.y = (token, slot) pair; expert = idx[pair]
+  const int32_t* idx;  // [T*topk] or null
+  int E, topk, x_rows;
+};
+
+// Stage x (rows m0..m0+MT) into LDS in dot2 register order; compute chunk sums.
+// xs layout per m: uint4[(j*4 + t) * LPR + sl]  for chunk c = sl + j*LPR, word t.
+// sx layout per m: float2[c] = (128 * sum(stored), sum(x)).
+template <int BITS, int MT>
+__device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uint4* xs,
+                                        float2* sx) {
+  const int cpr = p.wpr >> 2;
+  const int lpr_mask = (1 << p.lpr_log2) - 1;
+  for (int wi = threadIdx.x; wi < p.wpr; wi += kThreads) {
+    const int c = wi >> 2, t = wi & 3;
+    const int j = c >> p.lpr_log2, sl = c & lpr_mask;
+    const int dst = (((j << 2) + t) << p.lpr_log2) + sl;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      uint4 o = make_uint4(0, 0, 0, 0);
+      float stored = 0.f, truesum = 0.f;
+      if (m < p.M) {
+        if (BITS == 4) {
+          uint4 xv = *reinterpret_cast<const uint4*>(x + (size_t)m * p.K + (size_t)wi * 8);
+          o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
+          o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
+          o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
+          o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
+          truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
+                    (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
+          stored = truesum;
+        } else {
+          uint2 xv = *reinterpret_cast<const uint2*>(x + (size_t)m * p.K + (size_t)wi * 4);
+          uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);  // (x0,x2)
+          uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u); // (x1,x3)
+          o.x = a;
+          o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
+          o.z = c2;
+          o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
+          truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
+          stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
+        }
+      }
+      xs[(size_t)m * p.wpr + dst] = o;
+      stored += __shfl_xor(stored, 1, 64);
+      truesum += __shfl_xor(truesum, 1, 64);
+      stored += __shfl_xor(stored, 2, 64);
+      truesum += __shfl_xor(truesum, 2, 64);
+      if (t == 0) sx[(size_t)m * cpr + c] = make_float2(128.f * stored, truesum);
+    }
+  }
+}
+
+template <int BITS>
+__device__ __forceinline__ void unpack_word(uint32_t w, uint32_t (&pr)[4]) {
+  // nibble t and nibble t+4 of the word as (128+n_t, 128+n_{t+4}) in bf16
+  pr[0] = (w & 0x000F000Fu) | 0x43004300u;
+  pr[1] = ((w >> 4) & 0x000F000Fu) | 0x43004300u;
+  pr[2] = ((w >> 8) & 0x000F000Fu) | 0x43004300u;
+  pr[3] = ((w >> 12) & 0x000F000Fu) | 0x43004300u;
+}
+
+// NMAT == 2: the pair (gate, up) with the SwiGLU epilogue.
+template <int BITS, int MT, int NMAT>
+__global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
+  extern __shared__ uint4 smem[];
+  uint4* xs = smem;
+  float2* sx = reinterpret_cast<float2*>(smem + (size_t)MT * p.wpr);
+  constexpr int U = kUnits / NMAT;
+  constexpr int GSHIFT = (BITS == 4) ? 1 : 2;  // chunks per group, log2
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int lpr = 1 << p.lpr_log2;
+  const int rpwi = 64 >> p.lpr_log2;  // rows per wave instruction
+  const int sl = lane & (lpr - 1);
+  const int sub = lane >> p.lpr_log2;
+  const int G = p.K >> 6;
+  const int cpr = p.wpr >> 2;
+
+  const int gw = blockIdx.x * kWaves + wave;
+  const int s_begin = min(gw * p.spw, p.slots);
+  const int s_end = min(s_begin + p.spw, p.slots);
+  const int total = (s_end - s_begin) * p.iters;
+
+  // gather mode: this workgroup's (token, slot) pair selects expert, x row and y row
+  const bf16_t* xin = p.x;
+  bf16_t* yout = p.y;
+  size_t ew = 0, eg = 0;
+  if (p.idx) {
+    const int pair = blockIdx.y;
+    int e = p.idx[pair];
+    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+    ew = (size_t)e * p.N * p.wpr;
+    eg = (size_t)e * p.N * G;
+    xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
+    yout += (size_t)pair * p.N;
+  }
+
+  const int row0 = s_begin * rpwi + sub;
+  const size_t slot_words = (size_t)rpwi * p.wpr;  // words between slots
+  const int j_words = lpr * 4;
+  const uint32_t* wl[NMAT];
+  const bf16_t* sl_s[NMAT];
+  const bf16_t* sl_b[NMAT];
+#pragma unroll
+  for (int a = 0; a < NMAT; ++a) {
+    wl[a] = p.w[a] + ew + (size_t)row0 * p.wpr + sl * 4;
+    sl_s[a] = p.s[a] + eg + (size_t)row0 * G + (sl >> GSHIFT);
+    sl_b[a] = p.b[a] + eg + (size_t)row0 * G + (sl >> GSHIFT);
+  }
+  const int slot_groups = rpwi * G;
+  const int j_groups = lpr >> GSHIFT;
+
+  uint4 wv[NMAT][U];
+  bf16_t sc[NMAT][U], bi[NMAT][U];
+
+  // unit u -> (slot, j); issue the first batch of weight loads before staging x so
+  // the HBM latency overlaps the prologue.
+  auto issue = [&](int u0) {
+    int slot = u0 / p.iters;  // once per batch
+    int j = u0 - slot * p.iters;
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int last = (u0 + i >= total);  // clamp: re-read the final unit
+      size_t wo = (size_t)slot * slot_words + (size_t)j * j_words;
+      size_t so = (size_t)slot * slot_groups + (size_t)j * j_groups;
+      if (p.ragged) {  // rows past N re-read row N-1 (their results are not stored)
+        const int over = (s_begin + slot) * rpwi + sub - (p.N - 1);
+        if (over > 0) {
+          wo -= (size_t)over * p.wpr;
+          so -= (size_t)over * G;
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a) {
+        wv[a][i] = *reinterpret_cast<const uint4*>(wl[a] + wo);
+        sc[a][i] = sl_s[a][so];
+        bi[a][i] = sl_b[a][so];
+      }
+      if (!last && u0 + i + 1 < total) {
+        if (++j == p.iters) {
+          j = 0;
+          ++slot;
+        }
+      }
+    }
+  };
+
+  if (total > 0) issue(0);
+  stage_x<BITS, MT>(p, xin, xs, sx);
+  __syncthreads();
+  if (total <= 0) return;
+
+  float acc[NMAT][MT];
+#pragma unroll
+  for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[a][m] = 0.f;
+
+  int slot = 0, j = 0;  // of the unit being consumed
+  for (int u0 = 0; u0 < total; u0 += U) {
+    // registers of this batch -> locals, then prefetch the next batch
+    uint4 cw[NMAT][U];
+    float cs[NMAT][U], cb[NMAT][U];
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        cw[a][i] = wv[a][i];
+        cs[a][i] = bf2f(sc[a][i]);
+        cb[a][i] = bf2f(bi[a][i]);
+      }
+    if (u0 + U < total) issue(u0 + U);
+
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      if (u0 + i < total) {
+        const int c = sl + (j << p.lpr_log2);
+        float d[NMAT][MT];
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+          for (int m = 0; m < MT; ++m) d[a][m] = 0.f;
+        const uint32_t* cwi[NMAT];
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a) cwi[a] = reinterpret_cast<const uint32_t*>(&cw[a][i]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          uint32_t pr[NMAT][4];
+#pragma unroll
+          for (int a = 0; a < NMAT; ++a) unpack_word<BITS>(cwi[a][t], pr[a]);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const uint4 xv = xs[(size_t)m * p.wpr + ((((j << 2) + t) << p.lpr_log2) + sl)];
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) {
+              d[a][m] = dot2_bf16(pr[a][0], xv.x, d[a][m]);
+              d[a][m] = dot2_bf16(pr[a][1], xv.y, d[a][m]);
+              d[a][m] = dot2_bf16(pr[a][2], xv.z, d[a][m]);
+              d[a][m] = dot2_bf16(pr[a][3], xv.w, d[a][m]);
+            }
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float2 sm = sx[(size_t)m * cpr + c];
+#pragma unroll
+          for (int a = 0; a < NMAT; ++a) {
+            acc[a][m] = fmaf(cs[a][i], d[a][m] - sm.x, acc[a][m]);
+            acc[a][m] = fmaf(cb[a][i], sm.y, acc[a][m]);
+          }
+        }
+        if (++j == p.iters) {  // row finished: reduce over its lanes and store
+          const int row = (s_begin + slot) * rpwi + sub;
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            float r[NMAT];
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) {
+              float v = acc[a][m];
+              v += __shfl_xor(v, 1, 64);
+              if (p.lpr_log2 > 1) v += __shfl_xor(v, 2, 64);
+              if (p.lpr_log2 > 2) v += __shfl_xor(v, 4, 64);
+              if (p.lpr_log2 > 3) v += __shfl_xor(v, 8, 64);
+              if (p.lpr_log2 > 4) v += __shfl_xor(v, 16, 64);
+              if (p.lpr_log2 > 5) v += __shfl_xor(v, 32, 64);
+              r[a] = v;
+              acc[a][m] = 0.f;
+            }
+            if (sl == 0 && m < p.M && row < p.N) {
+              const size_t o = (size_t)m * p.N + row;
+              float out;
+              if (NMAT == 2) {
+                const float g = bf2f(f2bf(r[0])), up = bf2f(f2bf(r[NMAT - 1]));
+                out = g / (1.f + __expf(-g)) * up;
+              } else {
+                out = r[0];
+                if (p.residual) out = bf2f(f2bf(out)) + bf2f(p.residual[o]);
+              }
+              yout[o] = f2bf(out);
+            }
+          }
+          j = 0;
+          ++slot;
+        }
+      }
+    }
+  }
+}
+
+struct Plan {
+  int lpr_log2, iters, slots, spw, grid, ragged;
+  size_t lds;
+};
+
+bool make_plan(int N, int K, int bits, int mt, Plan* pl) {
+  const int wpr = K * bits / 32;
+  const int cpr = wpr / 4;  // 16-byte chunks per row
+  if (cpr * 4 != wpr || cpr == 0) return false;
+  const int lmin = bits == 4 ? 1 : 2;  // a lane group must span whole 64-groups
+  int l = 6;
+  while (l > lmin && (cpr % (1 << l)) != 0) --l;
+  if ((cpr % (1 << l)) != 0) return false;
+  const int rpwi = 64 >> l;
+  if ((int64_t)N * wpr >= (int64_t)1 << 31) return false;
+  pl->lpr_log2 = l;
+  pl->iters = cpr >> l;
+  pl->slots = (N + rpwi - 1) / rpwi;
+  pl->ragged = (N % rpwi) != 0;
+  pl->lds = (size_t)mt * ((size_t)wpr * 16 + (size_t)cpr * 8);
+  const int wg_per_cu = pl->lds <= 40 * 1024 ? 2 : 1;
+  int max_waves = 256 * wg_per_cu * kWaves;
+  // at least ~4 units of work per wave so the x staging is amortised
+  int min_spw = (4 + pl->iters - 1) / pl->iters;
+  int spw = (pl->slots + max_waves - 1) / max_waves;
+  if (spw < min_spw) spw = min_spw;
+  pl->spw = spw;
+  pl->grid = (pl->slots + spw * kWaves - 1) / (spw * kWaves);
+  return true;
+}
+
+template <int BITS, int MT, int NMAT>
+int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
+  auto kern = qmv_kernel<BITS, MT, NMAT>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+      return EXO_ERR_HIP;
+    }
+    attr_done = true;
+  }
+  kern<<<dim3(pl.grid, pairs), dim3(kThreads), pl.lds, st>>>(p);
+  return EXO_OK;
+}
+
+struct Gather {
+  const int32_t* idx = nullptr;
+  int pairs = 1, E = 0, topk = 1, x_rows = 1;
+};
+
+template <int NMAT>
+int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const* s,
+                 const bf16_t* const* b, const bf16_t* residual, bf16_t* y, int M, int N,
+                 int K, int bits, hipStream_t st, const char* name,
+                 const Gather& ga = Gather()) {
+  // M is processed in tiles of at most 4 rows (bounded by LDS: the whole K of every
+  // row of the tile is resident); each tile re-streams W.
+  int m0 = 0;
+  while (m0 < M) {
+    int mt = (M - m0 >= 4) ? 4 : ((M - m0 >= 2) ? 2 : 1);
+    if (ga.idx) mt = 1;
+    Plan pl;
+    for (;;) {
+      if (!make_plan(N, K, bits, mt, &pl)) {
+        exo_set_error("%s: unsupported shape N=%d K=%d bits=%d", name, N, K, bits);
+        return EXO_ERR_ARG;
+      }
+      if (pl.lds <= 150 * 1024 || mt == 1) break;
+      mt >>= 1;
+    }
+    if (pl.lds > 150 * 1024) {
+      exo_set_error("%s: K=%d too large for the LDS-resident activation tile", name, K);
+      return EXO_ERR_ARG;
+    }
+    QmvParams p;
+    p.x = x + (size_t)m0 * K;
+    for (int a = 0; a < 2; ++a) {
+      p.w[a] = w[a < NMAT ? a : 0];
+      p.s[a] = s[a < NMAT ? a : 0];
+      p.b[a] = b[a < NMAT ? a : 0];
+    }
+    p.residual = residual ? residual + (size_t)m0 * N : nullptr;
+    p.y = y + (size_t)m0 * N;
+    p.M = (M - m0 < mt) ? (M - m0) : mt;
+    p.N = N;
+    p.K = K;
+    p.wpr = K * bits / 32;
+    p.lpr_log2 = pl.lpr_log2;
+    p.iters = pl.iters;
+    p.slots = pl.slots;
+    p.spw = pl.spw;
+    p.ragged = pl.ragged;
+    p.idx = ga.idx;
+    p.E = ga.E;
+    p.topk = ga.topk;
+    p.x_rows = ga.x_rows;
+    const int pairs = ga.idx ? ga.pairs : 1;
+    int rc;
+    if (bits == 4) {
+      rc = mt == 4   ? launch_one<4, 4, NMAT>(p, pl, pairs, st)
+           : mt == 2 ? launch_one<4, 2, NMAT>(p, pl, pairs, st)
+                     : launch_one<4, 1, NMAT>(p, pl, pairs, st);
+    } else {
+      rc = mt == 4   ? launch_one<8, 4, NMAT>(p, pl, pairs, st)
+           : mt == 2 ? launch_one<8, 2, NMAT>(p, pl, pairs, st)
+                     : launch_one<8, 1, NMAT>(p, pl, pairs, st);
+    }
+    if (rc != EXO_OK) return rc;
+    m0 += mt;
+  }
+  return EXO_OK;
+}
+
+int check_gather(const char* name, int T, int topk, int x_rows, int E) {
+  EXO_REQUIRE(T >= 0 && topk > 0 && E > 0, "%s: bad T=%d topk=%d E=%d", name, T, topk, E);
+  EXO_REQUIRE(x_rows == 1 || x_rows == topk, "%s: x_rows=%d must be 1 or topk=%d", name, x_rows,
+              topk);
+  EXO_REQUIRE((int64_t)T * topk <= 65535, "%s: T*topk=%lld exceeds the decode-sized limit 65535",
+              name, (long long)T * topk);
+  return EXO_OK;
+}
+
+int check_common(const char* name, int M, int N, int K, int bits, int group_size) {
+  EXO_REQUIRE(bits == 4 || bits == 8, "%s: bits must be 4 or 8, got %d", name, bits);
+  EXO_REQUIRE(group_size == 64, "%s: group_size must be 64, got %d", name, group_size);
+  EXO_REQUIRE(M >= 0 && M <= 16, "%s: M=%d outside [0,16]; use exo_qmm", name, M);
+  EXO_REQUIRE(N > 0 && K > 0 && K % 64 == 0, "%s: bad shape N=%d K=%d (K %% 64 != 0?)", name,
+              N, K);
+  return EXO_OK;
+}
+
+}  // namespace
+
+extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M,
+                       int N, int K, int bits, int group_size, exo_stream_t stream) {
+  int rc = check_common("exo_qmv", M, N, K, bits, group_size);
+  if (rc) return rc;
+  EXO_REQUIRE(x && w && scales && biases && y, "exo_qmv: null pointer");
+  if (M == 0) return EXO_OK;
+  const uint32_t* ws[1] = {w};
+  const bf16_t* ss[1] = {scales};
+  const bf16_t* bs[1] = {biases};
+  rc = qmv_dispatch<1>(x, ws, ss, bs, residual, y, M, N, K, bits, (hipStream_t)stream,
+                       "exo_qmv");
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_qmv");
+  return EXO_OK;
+}
+
+extern "C" int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
+                              const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
+                              const uint16_t* bu, uint16_t* y, int M, int N, int K, int bits,
+                              int group_size, exo_stream_t stream) {
+  int rc = check_common("exo_qmv_swiglu", M, N, K, bits, group_size);
+  if (rc) return rc;
+  EXO_REQUIRE(x && wg && sg && bg && wu && su && bu && y, "exo_qmv_swiglu: null pointer");
+  if (M == 0) return EXO_OK;
+  const uint32_t* ws[2] = {wg, wu};
+  const bf16_t* ss[2] = {sg, su};
+  const bf16_t* bs[2] = {bg, bu};
+  rc = qmv_dispatch<2>(x, ws, ss, bs, nullptr, y, M, N, K, bits, (hipStream_t)stream,
+                       "exo_qmv_swiglu");
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_qmv_swiglu");
+  return EXO_OK;
+}
+
+extern "C" int exo_gather_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const int32_t* idx, uint16_t* y, int T,
+                              int topk, int x_rows, int E, int N, int K, int bits,
+                              int group_size, exo_stream_t stream) {
+  int rc = check_common("exo_gather_qmv", 1, N, K, bits, group_size);
+  if (rc) return rc;
+  rc = check_gather("exo_gather_qmv", T, topk, x_rows, E);
+  if (rc) return rc;
+  EXO_REQUIRE(x && w && scales && biases && idx && y, "exo_gather_qmv: null pointer");
+  if (T == 0) return EXO_OK;
+  const uint32_t* ws[1] = {w};
+  const bf16_t* ss[1] = {scales};
+  const bf16_t* bs[1] = {biases};
+  Gather ga;
+  ga.idx = idx;
+  ga.pairs = T * topk;
+  ga.E = E;
+  ga.topk = topk;
+  ga.x_rows = x_rows;
+  rc = qmv_dispatch<1>(x, ws, ss, bs, nullptr, y, 1, N, K, bits, (hipStream_t)stream,
+                       "exo_gather_qmv", ga);
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_gather_qmv");
+  return EXO_OK;
+}
+
+extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
+                                     const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
+                                     const uint16_t* bu, const int32_t* idx, uint16_t* y, int T,
+                                     int topk, int E, int N, int K, int bits, int group_size,
+                                     exo_stream_t stream) {
+  int rc = check_common("exo_gather_qmv_swiglu", 1, N, K, bits, group_size);
+  if (rc) return rc;
+  rc = check_gather("exo_gather_qmv_swiglu", T, topk, 1, E);
+  if (rc) return rc;
+  EXO_REQUIRE(x && wg && sg && bg && wu && su && bu && idx && y,
+              "exo_gather_qmv_swiglu: null pointer");
+  if (T == 0) return EXO_OK;
+  const uint32_t* ws[2] = {wg, wu};
+  const bf16_t* ss[2] = {sg, su};
+  const bf16_t* bs[2] = {bg, bu};
+  Gather ga;
+  ga.idx = idx;
+  ga.pairs = T * topk;
+  ga.E = E;
+  ga.topk = topk;
+  ga.x_rows = 1;
+  rc = qmv_dispatch<2>(x, ws, ss, bs, nullptr, y, 1, N, K, bits, (hipStream_t)stream,
+                       "exo_gather_qmv_swiglu", ga);
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_gather_qmv_swiglu");
+  return EXO_OK;
+}

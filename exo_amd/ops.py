@@ -1,0 +1,349 @@
+"""Operator layer: MLX-named operators on torch device tensors, executed by the HIP
+kernels of libexo_mi355x.so through its C ABI.
+
+Names and argument meaning follow the MLX operators the reference calls
+(.typings/mlx/core/__init__.pyi: quantized_matmul :4198-4234, gather_qmm :2957-3006,
+dequantize :2413-2451; mx.fast.rms_norm / rope / scaled_dot_product_attention).
+torch is used for device memory and streams only; every function launches on torch's
+current stream and never synchronises.  Errors: ValueError for bad arguments (the C
+ABI's -1), NativeError for HIP failures or a missing library.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import native
+from .native import check
+
+GROUP_SIZE = 64
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+@dataclass
+class QuantizedWeight:
+    """MLX affine-quantised matrix: ``weight`` uint32 words viewed as int32
+    [..., N, K*bits/32], ``scales`` / ``biases`` bf16 [..., N, K/64]."""
+
+    weight: torch.Tensor
+    scales: torch.Tensor
+    biases: torch.Tensor
+    bits: int
+    group_size: int = GROUP_SIZE
+
+    def __post_init__(self):
+        if self.weight.dtype == torch.uint32:
+            self.weight = self.weight.view(torch.int32)
+        assert self.weight.dtype == torch.int32
+        assert self.scales.dtype == torch.bfloat16 and self.biases.dtype == torch.bfloat16
+        assert self.bits in (4, 8) and self.group_size == GROUP_SIZE
+
+    @property
+    def N(self) -> int:
+        return self.weight.shape[-2]
+
+    @property
+    def K(self) -> int:
+        return self.weight.shape[-1] * 32 // self.bits
+
+    @property
+    def nbytes(self) -> int:
+        return (
+            self.weight.numel() * 4 + self.scales.numel() * 2 + self.biases.numel() * 2
+        )
+
+    def to(self, device) -> "QuantizedWeight":
+        return QuantizedWeight(
+            self.weight.to(device).contiguous(),
+            self.scales.to(device).contiguous(),
+            self.biases.to(device).contiguous(),
+            self.bits,
+            self.group_size,
+        )
+
+    def __getitem__(self, rows: slice) -> "QuantizedWeight":
+        return QuantizedWeight(
+            self.weight[rows], self.scales[rows], self.biases[rows], self.bits, self.group_size
+        )
+
+
+# ------------------------------------------------------------------ format ops
+
+
+def unpack_codes(weight: torch.Tensor, bits: int) -> torch.Tensor:
+    """uint32 words [..., W] -> uint8 codes [..., W*32/bits]."""
+    lib = native.load()
+    w = weight.view(torch.int32) if weight.dtype == torch.uint32 else weight
+    out = torch.empty(
+        *w.shape[:-1], w.shape[-1] * (32 // bits), dtype=torch.uint8, device=w.device
+    )
+    check(lib.exo_unpack_codes(_ptr(w), _ptr(out), w.numel(), bits, _stream()), "unpack_codes")
+    return out
+
+
+def dequantize(qw: QuantizedWeight) -> torch.Tensor:
+    """mx.dequantize -> bf16 [..., N, K]."""
+    lib = native.load()
+    rows = qw.weight.numel() // qw.weight.shape[-1]
+    out = torch.empty(*qw.weight.shape[:-1], qw.K, dtype=torch.bfloat16, device=qw.weight.device)
+    check(
+        lib.exo_dequantize(
+            _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(out), rows, qw.K, qw.bits,
+            qw.group_size, _stream(),
+        ),
+        "dequantize",
+    )
+    return out
+
+
+def embed(ids: torch.Tensor, qw: QuantizedWeight, out: torch.Tensor | None = None) -> torch.Tensor:
+    """QuantizedEmbedding.__call__: ids int32 [n] -> bf16 [n, K]."""
+    lib = native.load()
+    assert ids.dtype == torch.int32
+    n = ids.numel()
+    if out is None:
+        out = torch.empty(n, qw.K, dtype=torch.bfloat16, device=ids.device)
+    check(
+        lib.exo_embed_dequant(
+            _ptr(ids), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(out), n, qw.N,
+            qw.K, qw.bits, qw.group_size, _stream(),
+        ),
+        "embed",
+    )
+    return out
+
+
+# ------------------------------------------------------------------ matmuls
+
+QMV_MAX_M = 16
+
+
+def quantized_matmul(
+    x: torch.Tensor,
+    qw: QuantizedWeight,
+    residual: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """mx.quantized_matmul(x, w, scales, biases, transpose=True): x bf16 [M,K] ->
+    bf16 [M,N].  M <= 16 runs the fused dequant-GEMV, larger M the MFMA GEMM.
+    ``residual`` (bf16 [M,N]) fuses the block's ``h + r``."""
+    lib = native.load()
+    assert x.dtype == torch.bfloat16 and x.dim() == 2
+    M, K = x.shape
+    if K != qw.K:
+        raise ValueError(f"quantized_matmul: x has K={K}, weight has K={qw.K}")
+    if out is None:
+        out = torch.empty(M, qw.N, dtype=torch.bfloat16, device=x.device)
+    fn = lib.exo_qmv if M <= QMV_MAX_M else lib.exo_qmm
+    check(
+        fn(
+            _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(residual), _ptr(out),
+            M, qw.N, K, qw.bits, qw.group_size, _stream(),
+        ),
+        "quantized_matmul",
+    )
+    return out
+
+
+def qmm(x, qw: QuantizedWeight, residual=None, out=None) -> torch.Tensor:
+    """Force the matrix-core path (any M)."""
+    lib = native.load()
+    M, K = x.shape
+    if out is None:
+        out = torch.empty(M, qw.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_qmm(
+            _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(residual), _ptr(out),
+            M, qw.N, K, qw.bits, qw.group_size, _stream(),
+        ),
+        "qmm",
+    )
+    return out
+
+
+def qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) for M <= 16."""
+    lib = native.load()
+    M, K = x.shape
+    assert gate.N == up.N and gate.K == up.K == K and gate.bits == up.bits
+    if out is None:
+        out = torch.empty(M, gate.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_qmv_swiglu(
+            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+            _ptr(up.scales), _ptr(up.biases), _ptr(out), M, gate.N, K, gate.bits,
+            gate.group_size, _stream(),
+        ),
+        "qmv_swiglu",
+    )
+    return out
+
+
+def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, out=None):
+    """mx.gather_qmm(x, w, s, b, rhs_indices=idx, transpose=True) for decode-sized
+    inputs: x bf16 [T, R, K] (R == 1 or topk), idx int32 [T, topk] -> bf16 [T, topk, N]."""
+    lib = native.load()
+    T, R, K = x.shape
+    topk = rhs_indices.shape[1]
+    assert rhs_indices.dtype == torch.int32 and rhs_indices.shape[0] == T
+    E = qw.weight.shape[0]
+    if out is None:
+        out = torch.empty(T, topk, qw.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_gather_qmv(
+            _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(rhs_indices),
+            _ptr(out), T, topk, R, E, qw.N, K, qw.bits, qw.group_size, _stream(),
+        ),
+        "gather_qmm",
+    )
+    return out
+
+
+def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None):
+    """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N]."""
+    lib = native.load()
+    T, K = x.shape
+    topk = idx.shape[1]
+    E = gate.weight.shape[0]
+    if out is None:
+        out = torch.empty(T, topk, gate.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_gather_qmv_swiglu(
+            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+            _ptr(up.scales), _ptr(up.biases), _ptr(idx), _ptr(out), T, topk, E, gate.N, K,
+            gate.bits, gate.group_size, _stream(),
+        ),
+        "gather_qmv_swiglu",
+    )
+    return out
+
+
+# ------------------------------------------------------------------ small ops
+
+
+def add_rms_norm(x, residual, weight, eps: float, h_out=None, n_out=None):
+    """h = x (+ residual, bf16 add); returns (h, rms_norm(h) * weight)."""
+    lib = native.load()
+    rows, H = x.shape
+    if n_out is None:
+        n_out = torch.empty_like(x)
+    if residual is not None and h_out is None:
+        h_out = torch.empty_like(x)
+    check(
+        lib.exo_add_rmsnorm(
+            _ptr(x), _ptr(residual), _ptr(weight), _ptr(h_out), _ptr(n_out), rows, H, eps,
+            _stream(),
+        ),
+        "add_rms_norm",
+    )
+    return (h_out if residual is not None else x), n_out
+
+
+def rms_norm(x, weight, eps: float, out=None):
+    """mx.fast.rms_norm over the last axis of x [rows, H]."""
+    return add_rms_norm(x, None, weight, eps, None, out)[1]
+
+
+def rope_kv_append(qkv, q_out, k_cache, v_cache, pos, inv_freq, B, T, Hq, Hkv, D,
+                   q_norm_w=None, k_norm_w=None, eps: float = 0.0):
+    """Split fused qkv [B*T,(Hq+2Hkv)*D]; (q/k head norm;) RoPE at pos[b]+t; q -> q_out
+    [B*T,Hq*D]; k,v -> caches [B,Hkv,S_max,D]."""
+    lib = native.load()
+    S_max = k_cache.shape[2]
+    check(
+        lib.exo_rope_kv_append(
+            _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq),
+            _ptr(q_norm_w), _ptr(k_norm_w), eps, B, T, Hq, Hkv, D, S_max, _stream(),
+        ),
+        "rope_kv_append",
+    )
+
+
+def sdpa_decode_workspace(B: int, Hq: int, D: int, device) -> torch.Tensor:
+    n = native.load().exo_sdpa_decode_workspace(B, Hq, D)
+    return torch.empty(n // 4, dtype=torch.float32, device=device)
+
+
+def sdpa_decode(q, k_cache, v_cache, pos, out, workspace, scale, B, Hq, Hkv, D):
+    lib = native.load()
+    check(
+        lib.exo_sdpa_decode(
+            _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(out), _ptr(workspace), scale,
+            B, Hq, Hkv, D, k_cache.shape[2], _stream(),
+        ),
+        "sdpa_decode",
+    )
+
+
+def sdpa_prefill(q, k_cache, v_cache, pos, out, scale, B, T, Hq, Hkv, D):
+    lib = native.load()
+    check(
+        lib.exo_sdpa_prefill(
+            _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(out), scale, B, T, Hq, Hkv,
+            D, k_cache.shape[2], _stream(),
+        ),
+        "sdpa_prefill",
+    )
+
+
+def swiglu(gate, up, out=None):
+    lib = native.load()
+    if out is None:
+        out = torch.empty_like(gate)
+    check(lib.exo_swiglu(_ptr(gate), _ptr(up), _ptr(out), gate.numel(), _stream()), "swiglu")
+    return out
+
+
+def router_topk(logits, k: int, renorm: bool):
+    """-> (idx int32 [rows,k], scores bf16 [rows,k])."""
+    lib = native.load()
+    rows, E = logits.shape
+    idx = torch.empty(rows, k, dtype=torch.int32, device=logits.device)
+    sc = torch.empty(rows, k, dtype=torch.bfloat16, device=logits.device)
+    check(
+        lib.exo_router_topk(_ptr(logits), _ptr(idx), _ptr(sc), rows, E, k, int(renorm), _stream()),
+        "router_topk",
+    )
+    return idx, sc
+
+
+def moe_combine(y, scores, residual=None, out=None):
+    lib = native.load()
+    T, topk, H = y.shape
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=y.device)
+    check(
+        lib.exo_moe_combine(_ptr(y), _ptr(scores), _ptr(residual), _ptr(out), T, topk, H, _stream()),
+        "moe_combine",
+    )
+    return out
+
+
+def argmax_workspace(rows: int, device) -> torch.Tensor:
+    n = native.load().exo_argmax_workspace(rows)
+    return torch.empty(n // 4, dtype=torch.float32, device=device)
+
+
+def argmax_logsumexp(logits, token, lse, logprob, workspace, pos_inc=None):
+    """Greedy sampler + log-normaliser over bf16 logits [rows, V]."""
+    lib = native.load()
+    rows, V = logits.shape
+    check(
+        lib.exo_argmax_logsumexp(
+            _ptr(logits), _ptr(token), _ptr(lse), _ptr(logprob), _ptr(workspace), _ptr(pos_inc),
+            rows, V, _stream(),
+        ),
+        "argmax_logsumexp",
+    )

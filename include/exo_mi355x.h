@@ -1,0 +1,159 @@
+/* libexo_mi355x.so - C ABI of the MI355X (gfx950) kernels for exo's per-shard
+ * transformer forward on MLX affine-quantised weights.
+ *
+ * The reference has no FFI on this path: its engine calls mlx / mlx_lm Python
+ * operators.  Each entry point below replaces one of those operators and cites
+ * the place the reference states or calls it (paths relative to the reference
+ * tree).  All pointers are DEVICE pointers unless noted; `stream` is a
+ * hipStream_t passed as void*.  No entry point allocates, frees or synchronises;
+ * all are asynchronous on `stream`.  Return value: 0 ok, -1 bad argument,
+ * -2 HIP launch error; exo_last_error() gives the message (thread-local).
+ *
+ * Tensor conventions (MLX checkpoint layout, untouched):
+ *   packed weight  uint32 [N, K*bits/32], element i of a row in word i/(32/bits),
+ *                  bits [bits*(i mod 32/bits), +bits)     (.typings/mlx/core/__init__.pyi:4180-4184)
+ *   scales/biases  bf16   [N, K/group_size]               (src/exo/worker/engines/mlx/auto_parallel.py:880-881)
+ *   activations    bf16 row-major
+ * group_size must be 64 and bits 4 or 8.
+ */
+#ifndef EXO_MI355X_H
+#define EXO_MI355X_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* exo_stream_t;
+
+int exo_abi_version(void);
+const char* exo_last_error(void);
+/* 1 if dequantised bf16 weights are formed as bf16(bf16(s*q)+b), 0 if bf16(fma(s,q,b)). */
+int exo_dequant_two_roundings(void);
+
+/* K0: packed words -> one uint8 code per element.  (.typings/mlx/core/__init__.pyi:4180-4184) */
+int exo_unpack_codes(const uint32_t* w, uint8_t* out, int64_t n_words, int bits,
+                     exo_stream_t stream);
+
+/* mx.dequantize(w, scales, biases, group_size, bits) -> bf16 [rows, K].
+ * (.typings/mlx/core/__init__.pyi:2413-2451) */
+int exo_dequantize(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   uint16_t* out, int64_t rows, int K, int bits, int group_size,
+                   exo_stream_t stream);
+
+/* K4: nn.QuantizedEmbedding.__call__: out[i,:] = dequantize(row ids[i]).
+ * ids int32 [n_ids] on device.  (.typings/mlx/nn/layers/quantized.pyi:42-85) */
+int exo_embed_dequant(const int32_t* ids, const uint32_t* w, const uint16_t* scales,
+                      const uint16_t* biases, uint16_t* out, int n_ids, int vocab, int K,
+                      int bits, int group_size, exo_stream_t stream);
+
+/* K1: mx.quantized_matmul(x, w, scales, biases, transpose=True) for M <= 16 rows of
+ * x (decode): y[M,N] = x[M,K] @ dq(w)[N,K]^T, float32 accumulation, bf16 out.
+ * Optional fused epilogue: if `residual` is non-null, y = bf16(residual + bf16(acc))
+ * (the `h + r` of a transformer block).  (.typings/mlx/core/__init__.pyi:4198-4234,
+ * reached through nn.QuantizedLinear.__call__ .typings/mlx/nn/layers/quantized.pyi:87-118) */
+int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+            const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
+            int K, int bits, int group_size, exo_stream_t stream);
+
+/* K1+K8: fused gate/up projection and SwiGLU for M <= 16:
+ * y[M,N] = silu(x @ dq(wg)^T) * (x @ dq(wu)^T), each projection rounded to bf16
+ * first, as two QuantizedLinear calls followed by swiglu would.
+ * (.typings/mlx_lm/models/switch_layers.pyi:52-57) */
+int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
+                   const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
+                   const uint16_t* bu, uint16_t* y, int M, int N, int K, int bits,
+                   int group_size, exo_stream_t stream);
+
+/* K2: the same operator for any M (prefill): weights are dequantised to bf16 in
+ * LDS and multiplied on the matrix cores, float32 accumulation, bf16 out. */
+int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+            const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
+            int K, int bits, int group_size, exo_stream_t stream);
+
+/* K3: mx.gather_qmm(x, w, scales, biases, rhs_indices=idx, transpose=True) as
+ * QuantizedSwitchLinear calls it: w uint32 [E,N,K*bits/32]; idx int32 [T,topk];
+ * x bf16 [T, x_rows, K] with x_rows == 1 (same row for every slot) or topk;
+ * y bf16 [T, topk, N].  Decode-sized T (grouped GEMV).
+ * (.typings/mlx/core/__init__.pyi:2957-3006; .typings/mlx_lm/models/switch_layers.pyi:10-31) */
+int exo_gather_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                   const uint16_t* biases, const int32_t* idx, uint16_t* y, int T, int topk,
+                   int x_rows, int E, int N, int K, int bits, int group_size,
+                   exo_stream_t stream);
+
+/* K3+K8: SwitchGLU gate/up + swiglu in one pass: y[T,topk,N] =
+ * silu(x @ dq(wg[e])^T) * (x @ dq(wu[e])^T), x bf16 [T,K].
+ * (.typings/mlx_lm/models/switch_layers.pyi:59-73) */
+int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
+                          const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
+                          const uint16_t* bu, const int32_t* idx, uint16_t* y, int T,
+                          int topk, int E, int N, int K, int bits, int group_size,
+                          exo_stream_t stream);
+
+/* K5: mx.fast.rms_norm with the preceding residual add fused:
+ *   h = residual ? bf16(x + residual) : x ;  h_out = h (may be null) ;
+ *   n_out = bf16(h * rsqrt(mean(h^2)+eps) * weight).
+ * rows x H bf16.  (called by mlx_lm llama/qwen3_moe blocks; no stub in the reference) */
+int exo_add_rmsnorm(const uint16_t* x, const uint16_t* residual, const uint16_t* weight,
+                    uint16_t* h_out, uint16_t* n_out, int rows, int H, float eps,
+                    exo_stream_t stream);
+
+/* K6+K10 (+ Qwen3 q/k-norm): split a fused qkv row into heads, optionally RMS-normalise
+ * each q/k head (q_norm_w/k_norm_w bf16 [D] or null), rotate q and k (rotate-half
+ * RoPE, angle (pos[b]+t)*inv_freq[i]) and append k,v to the cache at pos[b]+t.
+ *   qkv      bf16 [B*T, (Hq+2*Hkv)*D]
+ *   q_out    bf16 [B*T, Hq*D]
+ *   k_cache/v_cache bf16 [B, Hkv, S_max, D]
+ *   pos      int32 [B] on device: tokens already cached per sequence
+ *   inv_freq float [D/2]
+ * (mx.fast.rope, KVCache.update_and_fetch .typings/mlx_lm/models/cache.pyi:150-169,
+ *  rope_utils .typings/mlx_lm/models/rope_utils.pyi:20-51) */
+int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
+                       uint16_t* v_cache, const int32_t* pos, const float* inv_freq,
+                       const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps, int B,
+                       int T, int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
+
+/* K7 decode: scaled_dot_product_attention for one new token per sequence over the
+ * cache, grouped-query: q bf16 [B, Hq*D]; lens int32 [B] = pos[b]+1 valid keys;
+ * out bf16 [B, Hq*D].  `workspace` float, exo_sdpa_decode_workspace(B,Hq,D) bytes.
+ * (.typings/mlx_lm/models/base.pyi:39-47) */
+int64_t exo_sdpa_decode_workspace(int B, int Hq, int D);
+int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                    const int32_t* pos, uint16_t* out, float* workspace, float scale, int B,
+                    int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
+
+/* K7 prefill: causal attention of T new tokens per sequence (already appended to the
+ * cache) over pos[b]+T keys.  q bf16 [B*T, Hq*D] -> out same shape. */
+int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                     const int32_t* pos, uint16_t* out, float scale, int B, int T, int Hq,
+                     int Hkv, int D, int S_max, exo_stream_t stream);
+
+/* K8: swiglu(gate, up) = silu(gate)*up elementwise, n elements.
+ * (.typings/mlx_lm/models/switch_layers.pyi:52-57) */
+int exo_swiglu(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n,
+               exo_stream_t stream);
+
+/* K9: Qwen3-MoE routing: softmax over E experts (float32, rounded to bf16), the k
+ * largest (ties to the lower id, slots in descending score), optional renormalisation.
+ * logits bf16 [rows,E] -> idx int32 [rows,k], scores bf16 [rows,k].  E <= 256, k <= 16. */
+int exo_router_topk(const uint16_t* logits, int32_t* idx, uint16_t* scores, int rows, int E,
+                    int k, int renorm, exo_stream_t stream);
+
+/* MoE combine: out[t,:] = bf16( sum_j bf16(y[t,j,:] * scores[t,j]) ) (+ residual[t,:]
+ * added in bf16 when non-null).  y bf16 [T,topk,H]. */
+int exo_moe_combine(const uint16_t* y, const uint16_t* scores, const uint16_t* residual,
+                    uint16_t* out, int T, int topk, int H, exo_stream_t stream);
+
+/* A9 (src/exo/worker/engines/mlx/patches/opt_batch_gen.py:67-88, greedy sampler):
+ * per row of bf16 logits [rows,V]: token = argmax (lowest index on ties),
+ * lse = logsumexp (float32), logprob of the token.  `workspace` float,
+ * exo_argmax_workspace(rows) bytes.  If pos_inc is non-null, pos_inc[r] += 1 for
+ * every row (advances the per-sequence cache position for the next graph replay). */
+int64_t exo_argmax_workspace(int rows);
+int exo_argmax_logsumexp(const uint16_t* logits, int32_t* token, float* lse, float* logprob,
+                         float* workspace, int32_t* pos_inc, int rows, int V,
+                         exo_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

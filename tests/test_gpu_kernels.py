@@ -1,0 +1,304 @@
+"""Parity of every HIP kernel, called through the C ABI, against the CPU oracle.
+
+Bar: bit-exact for codes / dequantised weights / indices; rtol 2e-2 (+ atol =
+rtol*rms) for bf16 activations.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import affine
+from oracle import ops as O
+from tests.util import (
+    assert_close, n_bits, n_f32, rand_bf16, rand_quantized, rng, t_bf16, t_qw, t_u32,
+)
+
+pytestmark = pytest.mark.gpu
+
+from exo_amd import native, ops  # noqa: E402
+
+
+def test_library_loads_and_reports_mode():
+    lib = native.load()
+    assert lib.exo_abi_version() == 1
+    assert lib.exo_dequant_two_roundings() in (0, 1)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_unpack_codes_bit_exact(device, bits):
+    w = rng(1).integers(0, 2**32, size=(37, 96), dtype=np.uint64).astype(np.uint32)
+    got = ops.unpack_codes(t_u32(w, device), bits).cpu().numpy()
+    np.testing.assert_array_equal(got, affine.unpack_codes(w, bits))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_dequantize_bit_exact(device, bits):
+    trip = rand_quantized(50, 512, bits, seed=3)
+    got = n_bits(ops.dequantize(t_qw(trip, bits, device)))
+    mode = "M1" if native.load().exo_dequant_two_roundings() else "M2"
+    want = affine.dequantize(*trip, 64, bits, mode)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_dequantize_all_codes_extreme_scales(device, bits):
+    # every code value at every slot, with scales/biases spanning magnitudes
+    K = 256 if bits == 8 else 64
+    per = 1 << bits
+    codes = (np.arange(per * K).reshape(per, K) // 1 + np.arange(per)[:, None]) % per
+    codes = np.tile(codes.astype(np.uint8), (1, 1))
+    w = affine.pack_codes(codes, bits)
+    G = K // 64
+    s = affine.f32_to_bf16_bits((rng(5).standard_normal((per, G)) * 10.0 ** rng(6).integers(-6, 3, (per, G))).astype(np.float32))
+    b = affine.f32_to_bf16_bits((rng(7).standard_normal((per, G)) * 10.0 ** rng(8).integers(-6, 3, (per, G))).astype(np.float32))
+    got = n_bits(ops.dequantize(t_qw((w, s, b), bits, device)))
+    mode = "M1" if native.load().exo_dequant_two_roundings() else "M2"
+    np.testing.assert_array_equal(got, affine.dequantize(w, s, b, 64, bits, mode))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_embed_bit_exact(device, bits):
+    trip = rand_quantized(300, 256, bits, seed=9)
+    ids = np.array([0, 299, 5, 5, 17, 128], np.int32)
+    got = n_bits(ops.embed(torch.from_numpy(ids).to(device), t_qw(trip, bits, device)))
+    mode = "M1" if native.load().exo_dequant_two_roundings() else "M2"
+    want = affine.dequantize(trip[0][ids], trip[1][ids], trip[2][ids], 64, bits, mode)
+    np.testing.assert_array_equal(got, want)
+
+
+QMV_SHAPES = [  # (N, K)
+    (256, 4096), (64, 2048), (128, 14336), (96, 768), (64, 1536), (200, 8192), (128, 64),
+    (72, 192),
+]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("N,K", QMV_SHAPES)
+@pytest.mark.parametrize("M", [1, 2, 3, 7, 16])
+def test_qmv(device, bits, N, K, M):
+    trip = rand_quantized(N, K, bits, seed=N + K + bits)
+    x = rand_bf16((M, K), seed=M + K)
+    got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device)))
+    want = affine.qmm(x, *trip, 64, bits)
+    assert_close(got, want, what=f"qmv {M}x{N}x{K} b{bits}")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qmv_is_accurate_beyond_bf16(device, bits):
+    # float32 accumulation: before the final rounding the result should sit within
+    # about one bf16 ulp of the float64 value.
+    N, K, M = 512, 4096, 1
+    trip = rand_quantized(N, K, bits, seed=77)
+    x = rand_bf16((M, K), seed=78)
+    got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device)))
+    wd = affine.dequantize_f32(*trip, 64, bits).astype(np.float64)
+    exact = x.astype(np.float64) @ wd.T
+    err = np.abs(got - exact)
+    assert np.all(err <= np.abs(exact) * 2.0**-8 + 1e-4), err.max()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qmv_residual(device, bits):
+    N, K, M = 192, 2048, 3
+    trip = rand_quantized(N, K, bits, seed=21)
+    x = rand_bf16((M, K), seed=22)
+    r = rand_bf16((M, N), seed=23)
+    got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device), residual=t_bf16(r, device)))
+    want = affine.bf16_round(affine.qmm(x, *trip, 64, bits) + r)
+    assert_close(got, want, what="qmv+residual")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [1, 4])
+def test_qmv_swiglu(device, bits, M):
+    N, K = 320, 2048
+    g = rand_quantized(N, K, bits, seed=31)
+    u = rand_quantized(N, K, bits, seed=32)
+    x = rand_bf16((M, K), seed=33)
+    got = n_f32(ops.qmv_swiglu(t_bf16(x, device), t_qw(g, bits, device), t_qw(u, bits, device)))
+    want = O.swiglu(affine.qmm(x, *g, 64, bits), affine.qmm(x, *u, 64, bits))
+    assert_close(got, want, what="qmv_swiglu")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (33, 130, 192), (257, 128, 1024), (17, 64, 64)])
+def test_qmm_mfma(device, bits, M, N, K):
+    trip = rand_quantized(N, K, bits, seed=M + N)
+    x = rand_bf16((M, K), seed=M * 3 + 1)
+    got = n_f32(ops.qmm(t_bf16(x, device), t_qw(trip, bits, device)))
+    want = affine.qmm(x, *trip, 64, bits)
+    assert_close(got, want, what=f"qmm {M}x{N}x{K} b{bits}")
+
+
+def test_qmm_residual_and_dispatch(device):
+    M, N, K, bits = 40, 192, 256, 4
+    trip = rand_quantized(N, K, bits, seed=5)
+    x = rand_bf16((M, K), seed=6)
+    r = rand_bf16((M, N), seed=7)
+    got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device), residual=t_bf16(r, device)))
+    want = affine.bf16_round(affine.qmm(x, *trip, 64, bits) + r)
+    assert_close(got, want, what="qmm+residual")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("x_rows", ["one", "topk"])
+def test_gather_qmv(device, bits, x_rows):
+    E, N, K, T, topk = 6, 96, 768, 3, 4
+    trip = rand_quantized(N, K, bits, seed=40, E=E)
+    idx = rng(41).integers(0, E, size=(T, topk)).astype(np.int32)
+    R = 1 if x_rows == "one" else topk
+    x = rand_bf16((T, R, K), seed=42)
+    got = n_f32(ops.gather_qmm(t_bf16(x, device), t_qw(trip, bits, device), torch.from_numpy(idx).to(device)))
+    want = affine.gather_qmm(x, *trip, idx, 64, bits)
+    assert_close(got, want, what="gather_qmv")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gather_qmv_swiglu(device, bits):
+    E, N, K, T, topk = 5, 64, 2048, 2, 3
+    g = rand_quantized(N, K, bits, seed=50, E=E)
+    u = rand_quantized(N, K, bits, seed=51, E=E)
+    idx = rng(52).integers(0, E, size=(T, topk)).astype(np.int32)
+    x = rand_bf16((T, K), seed=53)
+    got = n_f32(ops.gather_qmv_swiglu(t_bf16(x, device), t_qw(g, bits, device), t_qw(u, bits, device), torch.from_numpy(idx).to(device)))
+    want = O.swiglu(affine.gather_qmm(x[:, None], *g, idx, 64, bits), affine.gather_qmm(x[:, None], *u, idx, 64, bits))
+    assert_close(got, want, what="gather_qmv_swiglu")
+
+
+def test_bad_arguments_raise(device):
+    trip = rand_quantized(64, 128, 4, seed=1)
+    qw = t_qw(trip, 4, device)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul(t_bf16(rand_bf16((1, 64), 1), device), qw)
+    lib = native.load()
+    assert lib.exo_qmv(None, None, None, None, None, None, 1, 64, 128, 5, 64, None) == -1
+    assert b"bits" in lib.exo_last_error()
+    assert lib.exo_qmv(None, None, None, None, None, None, 1, 64, 128, 4, 32, None) == -1
+    assert lib.exo_qmv(None, None, None, None, None, None, 17, 64, 128, 4, 64, None) == -1
+
+
+@pytest.mark.parametrize("H", [2048, 4096, 64, 8192])
+@pytest.mark.parametrize("with_res", [False, True])
+def test_add_rmsnorm(device, H, with_res):
+    rows = 5
+    x = rand_bf16((rows, H), seed=H)
+    r = rand_bf16((rows, H), seed=H + 1) if with_res else None
+    w = rand_bf16((H,), seed=H + 2) + 1.0
+    w = affine.bf16_round(w)
+    h, n = ops.add_rms_norm(t_bf16(x, device), t_bf16(r, device) if with_res else None, t_bf16(w, device), 1e-5)
+    hh = affine.bf16_round(x + r) if with_res else x
+    np.testing.assert_array_equal(n_f32(h), hh)
+    assert_close(n_f32(n), O.rms_norm(hh, w, 1e-5), rtol=1e-2, what="rmsnorm")
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 8, 2), (128, 4, 4), (128, 16, 2)])
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_rope_kv_append(device, D, Hq, Hkv, qk_norm):
+    B, T, S_max = 2, 3, 40
+    pos = np.array([5, 17], np.int32)
+    qkv = rand_bf16((B * T, (Hq + 2 * Hkv) * D), seed=D + Hq)
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
+    inv = O.rope_inv_freq(D, 5e5, scaling)
+    qn = affine.bf16_round(rand_bf16((D,), 3) + 1.0) if qk_norm else None
+    kn = affine.bf16_round(rand_bf16((D,), 4) + 1.0) if qk_norm else None
+    kc = torch.zeros(B, Hkv, S_max, D, dtype=torch.bfloat16, device=device)
+    vc = torch.zeros_like(kc)
+    q_out = torch.empty(B * T, Hq * D, dtype=torch.bfloat16, device=device)
+    ops.rope_kv_append(
+        t_bf16(qkv, device), q_out, kc, vc, torch.from_numpy(pos).to(device),
+        torch.from_numpy(inv).to(device), B, T, Hq, Hkv, D,
+        t_bf16(qn, device) if qk_norm else None, t_bf16(kn, device) if qk_norm else None, 1e-6,
+    )
+    x = qkv.reshape(B, T, Hq + 2 * Hkv, D)
+    q, k, v = x[:, :, :Hq], x[:, :, Hq:Hq + Hkv], x[:, :, Hq + Hkv:]
+    if qk_norm:
+        q = O.rms_norm(q, qn, 1e-6)
+        k = O.rms_norm(k, kn, 1e-6)
+    for b in range(B):
+        qr = O.rope(q[b:b + 1].transpose(0, 2, 1, 3), inv, int(pos[b]))  # [1,H,T,D]
+        kr = O.rope(k[b:b + 1].transpose(0, 2, 1, 3), inv, int(pos[b]))
+        got_q = n_f32(q_out).reshape(B, T, Hq, D)[b].transpose(1, 0, 2)
+        assert_close(got_q, qr[0], rtol=1e-2, what="rope q")
+        got_k = n_f32(kc)[b, :, pos[b]:pos[b] + T]
+        assert_close(got_k, kr[0], rtol=1e-2, what="rope k")
+        np.testing.assert_array_equal(n_f32(vc)[b, :, pos[b]:pos[b] + T], v[b].transpose(1, 0, 2))
+    # nothing outside the appended window was written
+    assert float(n_f32(kc)[0, :, :5].sum()) == 0.0 and float(n_f32(kc)[0, :, 8:].sum()) == 0.0
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 32, 4), (128, 64, 4), (128, 4, 4)])
+@pytest.mark.parametrize("lens", [[1, 2], [100, 37], [513, 1024]])
+def test_sdpa_decode(device, D, Hq, Hkv, lens):
+    B, S_max = len(lens), 1024
+    q = rand_bf16((B, Hq * D), seed=D + Hq + lens[0])
+    k = rand_bf16((B, Hkv, S_max, D), seed=11)
+    v = rand_bf16((B, Hkv, S_max, D), seed=12)
+    pos = np.array([n - 1 for n in lens], np.int32)
+    out = torch.empty(B, Hq * D, dtype=torch.bfloat16, device=device)
+    ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+    ops.sdpa_decode(t_bf16(q, device), t_bf16(k, device), t_bf16(v, device), torch.from_numpy(pos).to(device), out, ws, D ** -0.5, B, Hq, Hkv, D)
+    for b in range(B):
+        want = O.sdpa(q[b].reshape(1, Hq, 1, D), k[b:b + 1, :, :lens[b]], v[b:b + 1, :, :lens[b]], D ** -0.5, None)
+        assert_close(n_f32(out)[b].reshape(Hq, D), want[0, :, 0], what=f"sdpa decode len {lens[b]}")
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 8, 2), (128, 8, 2)])
+def test_sdpa_prefill_causal(device, D, Hq, Hkv):
+    B, T, S_max = 2, 19, 64
+    pos = np.array([0, 30], np.int32)
+    q = rand_bf16((B * T, Hq * D), seed=D)
+    k = rand_bf16((B, Hkv, S_max, D), seed=13)
+    v = rand_bf16((B, Hkv, S_max, D), seed=14)
+    out = torch.empty(B * T, Hq * D, dtype=torch.bfloat16, device=device)
+    ops.sdpa_prefill(t_bf16(q, device), t_bf16(k, device), t_bf16(v, device), torch.from_numpy(pos).to(device), out, D ** -0.5, B, T, Hq, Hkv, D)
+    for b in range(B):
+        S = int(pos[b]) + T
+        qq = q.reshape(B, T, Hq, D)[b:b + 1].transpose(0, 2, 1, 3)
+        want = O.sdpa(qq, k[b:b + 1, :, :S], v[b:b + 1, :, :S], D ** -0.5, S - T)
+        got = n_f32(out).reshape(B, T, Hq, D)[b].transpose(1, 0, 2)
+        assert_close(got, want[0], what="sdpa prefill")
+
+
+def test_swiglu(device):
+    g = rand_bf16((3, 1001), seed=1, scale=3.0)
+    u = rand_bf16((3, 1001), seed=2)
+    got = n_f32(ops.swiglu(t_bf16(g, device), t_bf16(u, device)))
+    assert_close(got, O.swiglu(g, u), rtol=1e-2, what="swiglu")
+
+
+@pytest.mark.parametrize("E,k,renorm", [(128, 8, True), (128, 8, False), (60, 4, True), (256, 16, True)])
+def test_router_topk(device, E, k, renorm):
+    rows = 9
+    logits = rand_bf16((rows, E), seed=E + k, scale=2.0)
+    idx, sc = ops.router_topk(t_bf16(logits, device), k, renorm)
+    widx, wsc = O.router_topk(logits, k, renorm)
+    np.testing.assert_array_equal(idx.cpu().numpy(), widx)
+    assert_close(n_f32(sc), wsc, rtol=2.0**-7, what="router scores")
+
+
+def test_moe_combine(device):
+    T, topk, H = 3, 8, 2048
+    y = rand_bf16((T, topk, H), seed=1)
+    s = affine.bf16_round(np.abs(rand_bf16((T, topk), seed=2)) / 8)
+    r = rand_bf16((T, H), seed=3)
+    got = n_f32(ops.moe_combine(t_bf16(y, device), t_bf16(s, device), t_bf16(r, device)))
+    acc = affine.bf16_round(affine.bf16_round(y * s[..., None]).sum(1, dtype=np.float32))
+    assert_close(got, affine.bf16_round(acc + r), rtol=1e-2, what="moe_combine")
+
+
+@pytest.mark.parametrize("V", [128256, 1000, 64])
+def test_argmax_logsumexp(device, V):
+    rows = 3
+    logits = rand_bf16((rows, V), seed=V, scale=2.0)
+    logits[1, 7] = logits[1].max()  # a tie: lowest index must win
+    tok = torch.empty(rows, dtype=torch.int32, device=device)
+    lse = torch.empty(rows, dtype=torch.float32, device=device)
+    lp = torch.empty(rows, dtype=torch.float32, device=device)
+    pos = torch.tensor([4, 5, 6], dtype=torch.int32, device=device)
+    ops.argmax_logsumexp(t_bf16(logits, device), tok, lse, lp, ops.argmax_workspace(rows, device), pos)
+    np.testing.assert_array_equal(tok.cpu().numpy(), np.argmax(logits, -1))
+    want_lse = O.logsumexp(logits)[:, 0]
+    np.testing.assert_allclose(lse.cpu().numpy(), want_lse, rtol=1e-5)
+    np.testing.assert_allclose(lp.cpu().numpy(), logits.max(-1) - want_lse, rtol=1e-4, atol=1e-5)
+    assert pos.cpu().tolist() == [5, 6, 7]
