@@ -1,0 +1,493 @@
+"""The drop-in boundary: ``Builder`` / ``Engine`` for one MI355X.
+
+Mirrors the reference's plugin interface (src/exo/worker/engines/base.py:16-60) and
+its MLX implementations:
+  Mi355xBuilder        <-> MlxBuilder        (src/exo/worker/engines/mlx/builder.py:33-113)
+  BatchGenerator       <-> BatchGenerator    (src/exo/worker/runner/llm_inference/batch_generator.py:320-572)
+  ShardBatchGenerator  <-> ExoBatchGenerator (src/exo/worker/engines/mlx/generator/batch_generate.py:93-536)
+Same method names, argument meaning and error behaviour: ``step`` emits an ErrorChunk
+through ``event_sender`` before re-raising; a cancelled prefill raises
+PrefillCancelled; every method runs on the caller's (the runner's main) thread.
+``event_sender`` needs ``send(obj)``, ``cancel_receiver`` needs ``collect() -> list``;
+exo's MpSender / MpReceiver satisfy both.
+"""
+
+from __future__ import annotations
+
+import os
+import time
+from abc import ABC, abstractmethod
+from collections import deque
+from collections.abc import Callable, Generator, Iterable
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Any
+
+import torch
+
+from .cache import ShardKVCache
+from .config import ModelConfig
+from .generate import (
+    DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, ban_token_ids, extract_top_logprobs,
+    make_sampler, prefill,
+)
+from .loader import load_shard_weights
+from .model import ShardModel
+from .tokenizer import load_tokenizer
+from .types import (
+    BoundInstance, CancelledResponse, ErrorChunk, FinishedResponse, GenerationResponse,
+    GenerationStats, GenerationTask, ModelLoadingResponse, PrefillProgressChunk,
+    TextGenerationTaskParams, TokenChunk, Usage,
+)
+
+EXO_MAX_CONCURRENT_REQUESTS = int(os.environ.get("EXO_MAX_CONCURRENT_REQUESTS", "8"))
+CANCEL_ALL_TASKS = "CANCEL_ALL_TASKS"
+
+
+# ----------------------------------------------------------------------- ABCs
+
+
+class Engine(ABC):
+    _cancelled_tasks: set
+
+    def should_cancel(self, task_id) -> bool:
+        return task_id in self._cancelled_tasks or CANCEL_ALL_TASKS in self._cancelled_tasks
+
+    @abstractmethod
+    def warmup(self) -> None: ...
+
+    @abstractmethod
+    def submit(self, task: GenerationTask) -> None: ...
+
+    @abstractmethod
+    def step(self) -> Iterable[tuple[Any, Any]]: ...
+
+    @abstractmethod
+    def close(self) -> None: ...
+
+    @abstractmethod
+    def serve_prefill(self, request, wfile) -> None: ...
+
+
+class Builder(ABC):
+    @abstractmethod
+    def connect(self, bound_instance: BoundInstance) -> None: ...
+
+    @abstractmethod
+    def load(self, bound_instance: BoundInstance) -> Generator[ModelLoadingResponse, None, None]: ...
+
+    @abstractmethod
+    def build(self) -> Engine: ...
+
+    @abstractmethod
+    def close(self) -> None: ...
+
+
+# ------------------------------------------------------- inner batch generator
+
+
+@dataclass
+class _Seq:
+    uid: int
+    params: TextGenerationTaskParams
+    prompt_tokens: list[int]
+    sampler: Callable
+    processors: list
+    greedy: bool
+    max_tokens: int
+    prefill_tps: float
+    prefill_tokens: int
+    on_generation_token: Callable[[], None] | None
+    stop_sequences: list[str]
+    tokens: list[int] = field(default_factory=list)
+    n_gen: int = 0
+    t_first: float | None = None
+    t_last: float | None = None
+    accumulated: str = ""
+
+
+class ShardBatchGenerator:
+    """Continuous batching over one KV pool of ``max_batch`` rows.  ``submit`` prefills
+    the request into the next free row (batch-1 path) and feeds the last-but-one
+    prompt token as a single-token forward; ``step`` runs ONE graph-replayed
+    single-token forward for all active rows and maps the sampled tokens back to their
+    uids.  Active rows are kept compact at the front of the pool."""
+
+    def __init__(self, model: ShardModel, tokenizer, max_batch: int = EXO_MAX_CONCURRENT_REQUESTS,
+                 max_seq: int = 8192):
+        if not (model.is_first and model.is_last):
+            raise ValueError("the batch generator needs a shard that holds the whole model")
+        self.model, self.tokenizer = model, tokenizer
+        self.max_batch, self.max_seq = max_batch, max_seq
+        self.cache: ShardKVCache = model.make_cache(max_batch, max_seq)
+        self.rows: list[_Seq] = []
+        self._next_uid = 0
+        self._pending_input: list[int] = []  # token to feed per active row
+
+    @property
+    def has_work(self) -> bool:
+        return bool(self.rows)
+
+    def _eos(self) -> list[int]:
+        return list(getattr(self.tokenizer, "eos_token_ids", []) or [])
+
+    def submit(self, task_params: TextGenerationTaskParams, prompt,
+               on_prefill_progress: Callable[[int, int], None] | None = None,
+               distributed_prompt_progress_callback: Callable[[], None] | None = None,
+               on_generation_token: Callable[[], None] | None = None) -> int:
+        if len(self.rows) >= self.max_batch:
+            raise RuntimeError("no free batch row")
+        toks = prompt if not isinstance(prompt, str) else self.tokenizer.encode(prompt)
+        toks = [int(t) for t in toks]
+        if not toks:
+            raise ValueError("empty prompt")
+        max_tokens = task_params.max_output_tokens or MAX_TOKENS
+        if len(toks) + max_tokens + 2 > self.max_seq:
+            max_tokens = self.max_seq - len(toks) - 2
+            if max_tokens <= 0:
+                raise ValueError(f"prompt of {len(toks)} tokens exceeds the cache ({self.max_seq})")
+        row = len(self.rows)
+        self.cache.reset(rows=range(row, row + 1))
+
+        def progress(done: int, total: int) -> None:
+            if distributed_prompt_progress_callback is not None:
+                distributed_prompt_progress_callback()  # may raise PrefillCancelled
+            if on_prefill_progress is not None:
+                on_prefill_progress(done, total)
+
+        try:
+            tps, n = prefill(self.model, toks[:-1], self.cache, progress, row=row)
+        except PrefillCancelled:
+            self.cache.reset(rows=range(row, row + 1))
+            raise
+        if len(toks) >= 2:
+            self.model(torch.tensor([[toks[-2]]], dtype=torch.int32), self.cache, logits="none",
+                       rows=slice(row, row + 1))
+        gen = torch.Generator(device=self.model.device)
+        gen.manual_seed(task_params.seed or 42)
+        processors = [ban_token_ids(self._eos())] if task_params.bench and self._eos() else []
+        temp = task_params.temperature if task_params.temperature is not None else 0.7
+        seq = _Seq(
+            uid=self._next_uid, params=task_params, prompt_tokens=toks,
+            sampler=make_sampler(
+                temp, task_params.top_p if task_params.top_p is not None else 1.0,
+                task_params.min_p if task_params.min_p is not None else 0.05,
+                task_params.top_k if task_params.top_k is not None else 0, gen),
+            processors=processors, greedy=(temp == 0 and not processors), max_tokens=max_tokens,
+            prefill_tps=tps, prefill_tokens=n, on_generation_token=on_generation_token,
+            stop_sequences=[task_params.stop] if isinstance(task_params.stop, str)
+            else list(task_params.stop or []),
+            tokens=list(toks))
+        self._next_uid += 1
+        self.rows.append(seq)
+        self._pending_input.append(toks[-1])
+        return seq.uid
+
+    def step(self) -> list[tuple[int, GenerationResponse]]:
+        B = len(self.rows)
+        if B == 0:
+            return []
+        bufs = self.model._buffers(B, 1)
+        bufs.tokens.copy_(torch.tensor(self._pending_input, dtype=torch.int32))
+        bufs = self.model.decode_step(self.cache, B)
+        greedy_tokens = bufs.next_token.tolist()  # synchronises
+        now = time.perf_counter()
+        out: list[tuple[int, GenerationResponse]] = []
+        finished: list[int] = []
+        for r, seq in enumerate(self.rows):
+            logprobs = None
+            if seq.greedy:
+                tok = int(greedy_tokens[r])
+            else:
+                logits = bufs.logits[r : r + 1].float()
+                for p in seq.processors:
+                    logits = p(torch.tensor(seq.tokens), logits)
+                logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
+                tok = int(seq.sampler(logprobs)[0])
+            seq.n_gen += 1
+            seq.tokens.append(tok)
+            seq.t_first = seq.t_first or now
+            seq.t_last = now
+            self._pending_input[r] = tok
+            text = self.tokenizer.decode([tok]) if self.tokenizer is not None else ""
+            seq.accumulated += text
+            finish = None
+            if tok in self._eos() and not seq.params.bench:
+                finish = "stop"
+            elif seq.n_gen >= seq.max_tokens:
+                finish = "length"
+            for s in seq.stop_sequences:
+                if s and s in seq.accumulated:
+                    cut = seq.accumulated.find(s)
+                    text = seq.accumulated[:cut][len(seq.accumulated) - len(text):]
+                    finish = "stop"
+                    break
+            logprob = top = None
+            if seq.params.logprobs:
+                if logprobs is None:
+                    lg = bufs.logits[r].float()
+                    logprobs = (lg - torch.logsumexp(lg, dim=-1, keepdim=True))[None]
+                logprob, top = extract_top_logprobs(
+                    logprobs[0], self.tokenizer, seq.params.top_logprobs or DEFAULT_TOP_LOGPROBS, tok)
+            stats = usage = None
+            if finish is not None:
+                dt = (seq.t_last - seq.t_first) if seq.n_gen > 1 else 0.0
+                stats = GenerationStats(
+                    prompt_tps=float(seq.prefill_tps),
+                    generation_tps=float((seq.n_gen - 1) / dt) if dt > 0 else 0.0,
+                    prompt_tokens=len(seq.prompt_tokens), generation_tokens=seq.n_gen,
+                    peak_memory_usage=int(torch.cuda.max_memory_allocated(self.model.device)))
+                n_p = len(seq.prompt_tokens)
+                usage = Usage(n_p, seq.n_gen, n_p + seq.n_gen)
+                finished.append(r)
+            if seq.on_generation_token is not None:
+                seq.on_generation_token()
+            out.append((seq.uid, GenerationResponse(text=text, token=tok, logprob=logprob,
+                                                    top_logprobs=top, finish_reason=finish,
+                                                    stats=stats, usage=usage)))
+        self._drop_rows(finished)
+        return out
+
+    def _drop_rows(self, rows: list[int]) -> None:
+        for r in sorted(rows, reverse=True):
+            last = len(self.rows) - 1
+            if r != last:  # keep active rows compact: move the last row into the hole
+                self.cache.copy_row(last, r)
+                self.rows[r] = self.rows[last]
+                self._pending_input[r] = self._pending_input[last]
+            self.rows.pop()
+            self._pending_input.pop()
+
+    def cancel(self, uids: list[int]) -> None:
+        self._drop_rows([r for r, s in enumerate(self.rows) if s.uid in set(uids)])
+
+    def close(self) -> None:
+        self.rows.clear()
+        self._pending_input.clear()
+        self.cache = None  # type: ignore[assignment]
+
+
+# ----------------------------------------------------------------------- Engine
+
+
+def map_responses_to_chunks(r: GenerationResponse, model_id: str) -> TokenChunk:
+    return TokenChunk(model=model_id, text=r.text, token_id=r.token, usage=r.usage,
+                      finish_reason=r.finish_reason, stats=r.stats, logprob=r.logprob,
+                      top_logprobs=r.top_logprobs, is_thinking=r.is_thinking)
+
+
+def _prompt_of(tokenizer, params: TextGenerationTaskParams):
+    """The reference renders ``params.input`` through the tokenizer's chat template
+    (apply_chat_template, utils_mlx.py:413-510).  Here: a list of ints is taken as token
+    ids; strings / message dicts are joined and encoded as plain text."""
+    inp = params.input
+    if inp and all(isinstance(t, int) for t in inp):
+        return list(inp)
+    parts = []
+    for m in inp:
+        parts.append(m if isinstance(m, str) else str(m.get("content", "")) if isinstance(m, dict)
+                     else str(getattr(m, "content", m)))
+    return "\n".join(parts)
+
+
+@dataclass(eq=False)
+class BatchGenerator(Engine):
+    model: ShardModel
+    tokenizer: Any
+    model_id: str
+    device_rank: int = 0
+    cancel_receiver: Any = None
+    event_sender: Any = None
+    check_for_cancel_every: int = 50
+    max_seq: int = 8192
+    _cancelled_tasks: set = field(default_factory=set, init=False)
+    _all_tasks: dict = field(default_factory=dict, init=False)
+    _queue: deque = field(default_factory=deque, init=False)
+    _active_tasks: dict = field(default_factory=dict, init=False)
+
+    def __post_init__(self) -> None:
+        self._gen = ShardBatchGenerator(self.model, self.tokenizer, EXO_MAX_CONCURRENT_REQUESTS,
+                                        self.max_seq)
+
+    def warmup(self) -> None:
+        """generate.py:399-462: a short greedy generation on a fixed prompt; sets how
+        often a running generation checks for cancellation (about once per second)."""
+        params = TextGenerationTaskParams(model=self.model_id, max_output_tokens=50, temperature=0.0,
+                                          bench=True)
+        prompt = [1 % self.model.cfg.vocab_size] * 16
+        uid = self._gen.submit(params, prompt)
+        t0 = time.perf_counter()
+        n = 0
+        while self._gen.has_work:
+            self._gen.step()
+            n += 1
+        dt = time.perf_counter() - t0
+        del uid
+        self.check_for_cancel_every = max(1, min(100, int(n / dt))) if dt > 0 else 50
+
+    def submit(self, task: GenerationTask) -> None:
+        self._cancelled_tasks.discard(CANCEL_ALL_TASKS)
+        self._all_tasks[task.task_id] = task
+        self._queue.append(task)
+
+    def agree_on_cancellations(self) -> None:
+        if self.cancel_receiver is None:
+            return
+        for task_id in self.cancel_receiver.collect():
+            if task_id == CANCEL_ALL_TASKS:
+                self._cancelled_tasks.add(CANCEL_ALL_TASKS)
+            elif task_id in self._all_tasks:
+                self._cancelled_tasks.add(task_id)
+
+    def step(self):
+        while self._queue and len(self._active_tasks) < EXO_MAX_CONCURRENT_REQUESTS:
+            task = self._queue.popleft()
+            try:
+                uid = self._start_task(task)
+            except PrefillCancelled:
+                continue
+            except Exception as e:
+                self._send_error(task, e)
+                raise
+            self._active_tasks[uid] = task
+        if not self._gen.has_work:
+            return list(self._apply_cancellations())
+        try:
+            results = self._gen.step()
+        except Exception as e:
+            for task in self._active_tasks.values():
+                self._send_error(task, e)
+            raise
+        output: list[tuple[Any, Any]] = []
+        for uid, response in results:
+            task = self._active_tasks.get(uid)
+            if task is None:
+                continue
+            if self.device_rank == 0:
+                output.append((task.task_id, map_responses_to_chunks(response, self.model_id)))
+            if response.finish_reason is not None:
+                output.append((task.task_id, FinishedResponse()))
+                del self._active_tasks[uid]
+        output.extend(self._apply_cancellations())
+        return output
+
+    def _apply_cancellations(self):
+        if not self._cancelled_tasks:
+            return []
+        cancel_all = CANCEL_ALL_TASKS in self._cancelled_tasks
+        uids, results = [], []
+        for uid, task in list(self._active_tasks.items()):
+            if task.task_id in self._cancelled_tasks or cancel_all:
+                uids.append(uid)
+                results.append((task.task_id, CancelledResponse()))
+                del self._active_tasks[uid]
+        if uids:
+            self._gen.cancel(uids)
+        done = {tid for tid, _ in results}
+        for tid in self._cancelled_tasks:
+            if tid != CANCEL_ALL_TASKS and tid not in done:
+                results.append((tid, CancelledResponse()))
+        self._cancelled_tasks.clear()
+        return results
+
+    def _send_error(self, task: GenerationTask, e: Exception) -> None:
+        if self.device_rank == 0 and self.event_sender is not None:
+            self.event_sender.send(
+                (task.command_id, ErrorChunk(model=self.model_id, error_message=str(e))))
+
+    def _start_task(self, task: GenerationTask) -> int:
+        prompt = _prompt_of(self.tokenizer, task.task_params)
+
+        def on_prefill_progress(processed: int, total: int) -> None:
+            if self.device_rank == 0 and self.event_sender is not None:
+                self.event_sender.send(
+                    (task.command_id, PrefillProgressChunk(self.model_id, processed, total)))
+
+        def distributed_prompt_progress_callback() -> None:
+            self.agree_on_cancellations()
+            if self.should_cancel(task.task_id):
+                raise PrefillCancelled()
+
+        since = self.check_for_cancel_every
+
+        def on_generation_token() -> None:
+            nonlocal since
+            since += 1
+            if since >= self.check_for_cancel_every:
+                since = 0
+                self.agree_on_cancellations()
+
+        return self._gen.submit(task.task_params, prompt, on_prefill_progress,
+                                distributed_prompt_progress_callback, on_generation_token)
+
+    def close(self) -> None:
+        self._gen.close()
+        self.model = None  # type: ignore[assignment]
+        self.tokenizer = None
+
+    def serve_prefill(self, request, wfile) -> None:
+        raise NotImplementedError("disaggregated prefill serving is not part of this engine yet")
+
+
+# ----------------------------------------------------------------------- Builder
+
+
+def build_model_path(model_id: str) -> Path:
+    """src/exo/download/download_utils.py:152-178: first directory that holds the model
+    among EXO_MODELS_READ_ONLY_DIRS, EXO_MODELS_DIRS, else EXO_DEFAULT_MODELS_DIR."""
+    name = model_id.replace("/", "--")
+    cands = []
+    for var in ("EXO_MODELS_READ_ONLY_DIRS", "EXO_MODELS_DIRS"):
+        cands += [Path(p) / name for p in os.environ.get(var, "").split(":") if p]
+    default = Path(os.environ.get("EXO_DEFAULT_MODELS_DIR", str(Path.home() / ".exo" / "models")))
+    cands.append(default / name)
+    for c in cands:
+        if (c / "config.json").exists():
+            return c
+    return cands[-1]
+
+
+@dataclass
+class Mi355xBuilder(Builder):
+    model_id: str
+    event_sender: Any = None
+    cancel_receiver: Any = None
+    device: str = "cuda:0"
+    max_seq: int = 8192
+    inference_model: ShardModel | None = None
+    tokenizer: Any = None
+
+    def connect(self, bound_instance: BoundInstance) -> None:
+        if bound_instance.bound_shard.world_size != 1:
+            raise NotImplementedError(
+                "this engine serves single-device instances; multi-device groups are not wired")
+
+    def load(self, bound_instance: BoundInstance) -> Generator[ModelLoadingResponse, None, None]:
+        shard = bound_instance.bound_shard
+        if shard.immediate_exception:
+            raise RuntimeError("immediate_exception requested by shard metadata")
+        path = Path(bound_instance.model_path) if bound_instance.model_path else build_model_path(
+            shard.model_id)
+        cfg = ModelConfig.from_path(path)
+        if shard.n_layers != cfg.num_hidden_layers:
+            raise ValueError(f"shard says {shard.n_layers} layers, checkpoint has {cfg.num_hidden_layers}")
+        it = load_shard_weights(path, cfg, shard.start_layer, shard.end_layer, self.device)
+        try:
+            while True:
+                done, total = next(it)
+                yield ModelLoadingResponse(layers_loaded=done, total=total)
+        except StopIteration as stop:
+            weights = stop.value
+        self.inference_model = ShardModel(cfg, weights, shard.start_layer, shard.end_layer, self.device)
+        self.tokenizer = load_tokenizer(path, cfg.vocab_size)
+
+    def build(self) -> Engine:
+        assert self.inference_model is not None
+        return BatchGenerator(model=self.inference_model, tokenizer=self.tokenizer,
+                              model_id=self.model_id, device_rank=0,
+                              cancel_receiver=self.cancel_receiver, event_sender=self.event_sender,
+                              max_seq=self.max_seq)
+
+    def close(self) -> None:
+        self.inference_model = None
+        self.tokenizer = None

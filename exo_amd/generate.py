@@ -1,0 +1,228 @@
+"""Prefill and sequential generation with the reference's protocol.
+
+Mirrors src/exo/worker/engines/mlx/generator/generate.py:
+  ``prefill`` (:282-396)   feeds n tokens so that the cache ends up holding n-1
+  ``mlx_generate`` (:532-827) -> ``generate`` here: prefill on prompt[:-1], then the
+      last TWO prompt tokens are fed as single-token forwards, then one single-token
+      forward per generated token.
+Single-token forwards always take the GEMV path (like the reference's M=1 calls), so
+token N-2 of the prompt is not folded into the prefill GEMM.
+"""
+
+from __future__ import annotations
+
+import time
+from collections.abc import Callable, Generator
+
+import torch
+
+from . import ops
+from .cache import ShardKVCache, cache_length
+from .model import ShardModel
+from .types import GenerationResponse, GenerationStats, TextGenerationTaskParams, TopLogprobItem, Usage
+
+MAX_TOKENS = 32168  # src/exo/worker/engines/mlx/constants.py:7
+DEFAULT_TOP_LOGPROBS = 5
+PREFILL_STEP_SIZE = 4096  # generate.py:334
+
+
+class PrefillCancelled(BaseException):
+    """Raised from a progress callback to abandon a prefill (generate.py:153-154)."""
+
+
+# ---------------------------------------------------------------------- sampling
+
+
+def make_sampler(temp: float = 0.0, top_p: float = 1.0, min_p: float = 0.0, top_k: int = 0,
+                 generator: torch.Generator | None = None) -> Callable[[torch.Tensor], torch.Tensor]:
+    """mlx_lm ``make_sampler`` semantics (.typings/mlx_lm/sample_utils.pyi:10-45) on
+    float32 log-probabilities [B,V] -> token ids int64 [B]: temp 0 is argmax; otherwise
+    top_p, then min_p, then top_k filters are applied to the log-probabilities and a
+    token is drawn from softmax(logprobs / temp)."""
+    if temp == 0:
+        return lambda lp: torch.argmax(lp, dim=-1)
+
+    def sample(lp: torch.Tensor) -> torch.Tensor:
+        lp = lp.float()
+        if 0 < top_p < 1.0:
+            probs = lp.exp()
+            sp, si = torch.sort(probs, dim=-1)  # ascending
+            cum = sp.cumsum(-1)
+            keep = cum > (1 - top_p)
+            masked = torch.where(keep, lp.gather(-1, si), torch.full_like(lp, -float("inf")))
+            lp = torch.empty_like(lp).scatter_(-1, si, masked)
+        if min_p > 0:
+            top = lp.max(-1, keepdim=True).values
+            lp = torch.where(lp < top + torch.log(torch.tensor(min_p, device=lp.device)),
+                             torch.full_like(lp, -float("inf")), lp)
+        if top_k > 0:
+            kth = lp.topk(min(top_k, lp.shape[-1]), dim=-1).values[..., -1:]
+            lp = torch.where(lp < kth, torch.full_like(lp, -float("inf")), lp)
+        p = torch.softmax(lp / temp, dim=-1)
+        return torch.multinomial(p, 1, generator=generator).squeeze(-1)
+
+    return sample
+
+
+def ban_token_ids(token_ids: list[int]) -> Callable[[torch.Tensor, torch.Tensor], torch.Tensor]:
+    """generate.py:465-473: set the banned logits to -1e9."""
+    ids = list(token_ids)
+
+    def proc(_tokens: torch.Tensor, logits: torch.Tensor) -> torch.Tensor:
+        if ids:
+            logits = logits.clone()
+            logits[..., ids] = -1e9
+        return logits
+
+    return proc
+
+
+def extract_top_logprobs(logprobs: torch.Tensor, tokenizer, top_logprobs: int,
+                         selected_token: int) -> tuple[float, list[TopLogprobItem]]:
+    """generate.py:483-529: the selected token's logprob and the k most likely tokens,
+    descending."""
+    k = min(top_logprobs, logprobs.shape[-1])
+    vals, idx = torch.topk(logprobs.float(), k)
+    items = []
+    for v, i in zip(vals.tolist(), idx.tolist()):
+        text = tokenizer.decode([i]) if tokenizer is not None else str(i)
+        items.append(TopLogprobItem(token=text, logprob=float(v), bytes=list(text.encode("utf-8"))))
+    return float(logprobs[selected_token]), items
+
+
+# ---------------------------------------------------------------------- prefill
+
+
+def prefill(model: ShardModel, prompt_tokens, cache: ShardKVCache,
+            on_prefill_progress: Callable[[int, int], None] | None = None,
+            step: int = PREFILL_STEP_SIZE, faithful_extra_steps: bool = True,
+            row: int = 0) -> tuple[float, int]:
+    """Fill cache row ``row`` from ``prompt_tokens`` (n ids).  After it the row holds
+    n-1 entries (invariant asserted by the reference's test_kv_prefix_cache.py:157).
+
+    Protocol (generate.py:354-387): chunks of at most ``step`` tokens cover the first
+    n-1 tokens; token n-1 is then run as a single-token forward whose sample is
+    discarded, the generator it came from had already computed one more single-token
+    forward, and ``trim(2)`` removes both entries.  ``faithful_extra_steps=False``
+    skips those two forwards (same cache contents, less work).
+    Returns (tokens_per_sec, n)."""
+    n = len(prompt_tokens)
+    if n == 0:
+        return 0.0, 0
+    t0 = time.perf_counter()
+    toks = torch.as_tensor(prompt_tokens, dtype=torch.int32).reshape(1, -1)
+    rows = slice(row, row + 1)
+    done = 0
+    while n - done > 1:
+        m = min(step, n - done - 1)
+        model(toks[:, done : done + m], cache, logits="none", rows=rows)
+        done += m
+        if on_prefill_progress is not None:
+            on_prefill_progress(done, n)
+    if faithful_extra_steps:
+        lg = model(toks[:, done : done + 1], cache, logits="last", rows=rows)
+        nxt = torch.argmax(lg[0, -1].float()).reshape(1, 1)
+        model(nxt, cache, logits="last", rows=rows)
+        cache.trim(2, rows=range(row, row + 1))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return (n / dt if dt > 0 else 0.0), n
+
+
+# ---------------------------------------------------------------------- generate
+
+
+def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, prompt_tokens: list[int],
+             on_prefill_progress: Callable[[int, int], None] | None = None,
+             on_generation_token: Callable[[], None] | None = None,
+             max_seq: int | None = None, eos_token_ids: list[int] | None = None,
+             ) -> Generator[GenerationResponse, None, None]:
+    """Sequential (batch 1) generation for a full-model shard: yields one
+    GenerationResponse per token; the last carries finish_reason, stats and usage."""
+    if not (model.is_first and model.is_last):
+        raise ValueError("generate() needs a shard that holds the whole model")
+    seed = task.seed or 42
+    gen = torch.Generator(device=model.device)
+    gen.manual_seed(seed)
+    max_tokens = task.max_output_tokens or MAX_TOKENS
+    n_prompt = len(prompt_tokens)
+    if n_prompt == 0:
+        raise ValueError("empty prompt")
+    cache = model.make_cache(1, max_seq or (n_prompt + max_tokens + 8))
+    torch.cuda.reset_peak_memory_stats(model.device)
+
+    eos = list(eos_token_ids or [])
+    processors = []
+    if task.bench:
+        processors.append(ban_token_ids(eos))  # bench: exactly max_tokens are produced
+    sampler = make_sampler(
+        temp=task.temperature if task.temperature is not None else 0.7,
+        top_p=task.top_p if task.top_p is not None else 1.0,
+        min_p=task.min_p if task.min_p is not None else 0.05,
+        top_k=task.top_k if task.top_k is not None else 0, generator=gen)
+    greedy = (task.temperature == 0) and not processors
+    stop_sequences = [task.stop] if isinstance(task.stop, str) else list(task.stop or [])
+
+    prefill_tps, prefill_tokens = prefill(model, prompt_tokens[:-1], cache, on_prefill_progress)
+    assert cache_length(cache) == max(n_prompt - 2, 0)
+
+    # the last two prompt tokens, one forward each (generate.py:710-733)
+    if n_prompt >= 2:
+        model(torch.tensor([[prompt_tokens[-2]]], dtype=torch.int32), cache, logits="none")
+    tok = int(prompt_tokens[-1])
+    history = list(prompt_tokens)
+    accumulated = ""
+    t_first = t_last = None
+    for n_gen in range(1, max_tokens + 1):
+        bufs = model._buffers(1, 1)
+        bufs.tokens[0] = tok
+        bufs = model.decode_step(cache, 1)
+        if greedy:
+            tok = int(bufs.next_token[0])
+            logprobs = None
+        else:
+            logits = bufs.logits[0:1].float()
+            for p in processors:
+                logits = p(torch.tensor(history), logits)
+            logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
+            tok = int(sampler(logprobs)[0])
+        now = time.perf_counter()
+        t_first = t_first or now
+        t_last = now
+        history.append(tok)
+        text = tokenizer.decode([tok]) if tokenizer is not None else ""
+        accumulated += text
+        finish = None
+        if tok in eos and not task.bench:
+            finish = "stop"
+        elif n_gen >= max_tokens:
+            finish = "length"
+        for s in stop_sequences:
+            if s and s in accumulated:
+                cut = accumulated.find(s)
+                chunk_start = len(accumulated) - len(text)
+                text = accumulated[:cut][chunk_start:]
+                finish = "stop"
+                break
+        logprob = top = None
+        if task.logprobs:
+            if logprobs is None:
+                lg = bufs.logits[0].float()
+                logprobs = (lg - torch.logsumexp(lg, dim=-1, keepdim=True))[None]
+            logprob, top = extract_top_logprobs(logprobs[0], tokenizer,
+                                                task.top_logprobs or DEFAULT_TOP_LOGPROBS, tok)
+        stats = usage = None
+        if finish is not None:
+            # generation_tps = (n-1)/(t_last - t_first)  (batch_generate.py:418-426)
+            dt = (t_last - t_first) if n_gen > 1 else 0.0
+            stats = GenerationStats(
+                prompt_tps=float(prefill_tps), generation_tps=float((n_gen - 1) / dt) if dt > 0 else 0.0,
+                prompt_tokens=int(prefill_tokens + min(n_prompt, 2)), generation_tokens=n_gen,
+                peak_memory_usage=int(torch.cuda.max_memory_allocated(model.device)))
+            usage = Usage(n_prompt, n_gen, n_prompt + n_gen)
+        if on_generation_token is not None:
+            on_generation_token()
+        yield GenerationResponse(text=text, token=tok, logprob=logprob, top_logprobs=top,
+                                 finish_reason=finish, stats=stats, usage=usage)
+        if finish is not None:
+            break

@@ -1,0 +1,311 @@
+"""The per-shard transformer forward over a contiguous layer range.
+
+What the reference obtains from mlx_lm's ``llama.Model`` / ``qwen3_moe.Model`` after
+``pipeline_auto_parallel`` has kept ``layers[start:end]``
+(src/exo/worker/engines/mlx/auto_parallel.py:276-395), behind the ``Model`` protocol
+of src/exo/worker/engines/mlx/types.py:29-37: ``model(tokens, cache,
+input_embeddings=None)``.  The first shard embeds the tokens, every other shard
+receives the hidden state [B,T,H] (what PipelineFirstLayer would ``recv_like``,
+auto_parallel.py:132-139); the last shard applies the final norm and lm_head, every
+other one returns the hidden state leaving its last local layer.
+
+Every operator is a HIP kernel reached through the C ABI (exo_amd.ops).  Single-token
+steps (B*T <= 16 rows) use the fused dequant-GEMV family and can be replayed from a
+HIP graph (``decode_step``); longer inputs use the matrix-core GEMM and the causal
+prefill attention.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import ops
+from .cache import ShardKVCache
+from .config import ModelConfig
+from .ops import QuantizedWeight
+
+GEMV_MAX_ROWS = ops.QMV_MAX_M
+
+
+def rope_inv_freq(cfg: ModelConfig) -> torch.Tensor:
+    """Per-pair inverse frequencies (float32, CPU): theta^(-2i/d), with the llama3
+    piecewise rescale of mlx_lm's Llama3RoPE (.typings/mlx_lm/models/rope_utils.pyi:20-51)."""
+    d = cfg.head_dim
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+    sc = cfg.rope_scaling
+    if sc and sc.get("rope_type", sc.get("type")) == "llama3":
+        factor = float(sc["factor"])
+        lo = float(sc.get("low_freq_factor", 1.0))
+        hi = float(sc.get("high_freq_factor", 4.0))
+        old = float(sc.get("original_max_position_embeddings", 8192))
+        wl = 2 * math.pi / inv
+        scaled = torch.where(wl > old / lo, inv / factor, inv)
+        smooth = (old / wl - lo) / (hi - lo)
+        mid = (1 - smooth) * inv / factor + smooth * inv
+        is_mid = (wl <= old / lo) & (wl >= old / hi)
+        inv = torch.where(is_mid, mid, scaled)
+    elif sc and sc.get("rope_type", sc.get("type")) not in (None, "default", "linear"):
+        raise ValueError(f"rope_scaling {sc} not supported")
+    if sc and sc.get("rope_type", sc.get("type")) == "linear":
+        inv = inv / float(sc["factor"])
+    return inv.to(torch.float32)
+
+
+class _Layer:
+    """Weights of one transformer block (device resident)."""
+
+    def __init__(self, cfg: ModelConfig, w: dict, i: int):
+        p = f"model.layers.{i}."
+        bits = cfg.bits
+
+        def q(name: str) -> QuantizedWeight:
+            return QuantizedWeight(w[p + name + ".weight"], w[p + name + ".scales"],
+                                   w[p + name + ".biases"], bits, cfg.group_size)
+
+        self.index = i
+        self.in_norm = w[p + "input_layernorm.weight"]
+        self.post_norm = w[p + "post_attention_layernorm.weight"]
+        qp, kp, vp = q("self_attn.q_proj"), q("self_attn.k_proj"), q("self_attn.v_proj")
+        # q|k|v concatenated along the output rows: one launch instead of three
+        self.qkv = QuantizedWeight(
+            torch.cat([qp.weight, kp.weight, vp.weight]).contiguous(),
+            torch.cat([qp.scales, kp.scales, vp.scales]).contiguous(),
+            torch.cat([qp.biases, kp.biases, vp.biases]).contiguous(), bits, cfg.group_size)
+        self.o = q("self_attn.o_proj")
+        self.q_norm = w.get(p + "self_attn.q_norm.weight")
+        self.k_norm = w.get(p + "self_attn.k_norm.weight")
+        if cfg.is_moe:
+            self.router = q("mlp.gate")
+            self.gate = q("mlp.switch_mlp.gate_proj")
+            self.up = q("mlp.switch_mlp.up_proj")
+            self.down = q("mlp.switch_mlp.down_proj")
+        else:
+            self.gate, self.up, self.down = q("mlp.gate_proj"), q("mlp.up_proj"), q("mlp.down_proj")
+
+    def nbytes(self) -> int:
+        n = self.qkv.nbytes + self.o.nbytes + self.gate.nbytes + self.up.nbytes + self.down.nbytes
+        return n + (self.router.nbytes if hasattr(self, "router") else 0)
+
+
+class _Buffers:
+    """Activation workspace for R = B*T rows."""
+
+    def __init__(self, m: "ShardModel", R: int, B: int, device):
+        c = m.cfg
+        bf = dict(dtype=torch.bfloat16, device=device)
+        Hq, Hkv, D = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+        self.R = R
+        self.tokens = torch.zeros(R, dtype=torch.int32, device=device)
+        self.h = torch.empty(R, c.hidden_size, **bf)
+        self.n = torch.empty(R, c.hidden_size, **bf)
+        self.qkv = torch.empty(R, (Hq + 2 * Hkv) * D, **bf)
+        self.q = torch.empty(R, Hq * D, **bf)
+        self.attn = torch.empty(R, Hq * D, **bf)
+        if c.is_moe:
+            k, Ie = c.num_experts_per_tok, c.moe_intermediate_size
+            self.router_logits = torch.empty(R, c.num_experts, **bf)
+            self.act = torch.empty(R, k, Ie, **bf)
+            self.expert_out = torch.empty(R, k, c.hidden_size, **bf)
+        else:
+            self.act = torch.empty(R, c.intermediate_size, **bf)
+            self.gate = self.up = None
+        self.sdpa_ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+        # sampling outputs (last shard)
+        self.logits = None
+        self.next_token = torch.zeros(B, dtype=torch.int32, device=device)
+        self.lse = torch.zeros(B, dtype=torch.float32, device=device)
+        self.logprob = torch.zeros(B, dtype=torch.float32, device=device)
+        self.argmax_ws = ops.argmax_workspace(B, device)
+
+
+class ShardModel:
+    def __init__(self, cfg: ModelConfig, weights: dict[str, torch.Tensor], start_layer: int = 0,
+                 end_layer: int | None = None, device="cuda:0"):
+        self.cfg = cfg
+        self.device = torch.device(device)
+        self.start_layer = start_layer
+        self.end_layer = cfg.num_hidden_layers if end_layer is None else end_layer
+        if not (0 <= self.start_layer < self.end_layer <= cfg.num_hidden_layers):
+            raise ValueError(f"bad layer range [{start_layer},{end_layer}) of {cfg.num_hidden_layers}")
+        self.layers = [_Layer(cfg, weights, i) for i in range(self.start_layer, self.end_layer)]
+        self.embed_tokens = None
+        if self.is_first or (self.is_last and cfg.tie_word_embeddings):
+            self.embed_tokens = QuantizedWeight(
+                weights["model.embed_tokens.weight"], weights["model.embed_tokens.scales"],
+                weights["model.embed_tokens.biases"], cfg.bits, cfg.group_size)
+        self.norm = self.lm_head = None
+        if self.is_last:
+            self.norm = weights["model.norm.weight"]
+            self.lm_head = self.embed_tokens if cfg.tie_word_embeddings else QuantizedWeight(
+                weights["lm_head.weight"], weights["lm_head.scales"], weights["lm_head.biases"],
+                cfg.bits, cfg.group_size)
+        self.inv_freq = rope_inv_freq(cfg).to(self.device)
+        self.scale = cfg.head_dim ** -0.5
+        self._bufs: dict[tuple[int, int], _Buffers] = {}
+        self._graphs: dict[int, tuple] = {}
+
+    # ------------------------------------------------------------------ properties
+    @property
+    def is_first(self) -> bool:
+        return self.start_layer == 0
+
+    @property
+    def is_last(self) -> bool:
+        return self.end_layer == self.cfg.num_hidden_layers
+
+    def weight_bytes(self) -> int:
+        n = sum(l.nbytes() for l in self.layers)
+        if self.lm_head is not None:
+            n += self.lm_head.nbytes
+        return n
+
+    def make_cache(self, batch: int = 1, max_seq: int = 4096) -> ShardKVCache:
+        c = self.cfg
+        return ShardKVCache(len(self.layers), batch, c.num_key_value_heads, c.head_dim, max_seq,
+                            self.device)
+
+    def _buffers(self, B: int, T: int) -> _Buffers:
+        key = (B, T)
+        if key not in self._bufs:
+            if T > 1 and len(self._bufs) > 8:  # prefill shapes vary; do not hoard them
+                for k in [k for k in self._bufs if k[1] > 1]:
+                    del self._bufs[k]
+            self._bufs[key] = _Buffers(self, B * T, B, self.device)
+        return self._bufs[key]
+
+    # ------------------------------------------------------------------ the forward
+    def _mlp(self, L: _Layer, bf: _Buffers, R: int) -> None:
+        """h <- h + mlp(post_norm(h)) in place; bf.n holds the normed input."""
+        c = self.cfg
+        gemv = R <= GEMV_MAX_ROWS
+        if not c.is_moe:
+            if gemv:
+                ops.qmv_swiglu(bf.n, L.gate, L.up, out=bf.act)
+            else:
+                if bf.gate is None:
+                    bf.gate = torch.empty_like(bf.act)
+                    bf.up = torch.empty_like(bf.act)
+                ops.quantized_matmul(bf.n, L.gate, out=bf.gate)
+                ops.quantized_matmul(bf.n, L.up, out=bf.up)
+                ops.swiglu(bf.gate, bf.up, out=bf.act)
+            ops.quantized_matmul(bf.act, L.down, residual=bf.h, out=bf.h)
+            return
+        ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
+        idx, sc = ops.router_topk(bf.router_logits, c.num_experts_per_tok, c.norm_topk_prob)
+        step = max(1, 65535 // c.num_experts_per_tok)
+        for r0 in range(0, R, step):  # the grouped GEMV takes decode-sized row counts
+            r1 = min(R, r0 + step)
+            ops.gather_qmv_swiglu(bf.n[r0:r1], L.gate, L.up, idx[r0:r1], out=bf.act[r0:r1])
+            ops.gather_qmm(bf.act[r0:r1], L.down, idx[r0:r1], out=bf.expert_out[r0:r1])
+            ops.moe_combine(bf.expert_out[r0:r1], sc[r0:r1], residual=bf.h[r0:r1], out=bf.h[r0:r1])
+
+    def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
+             rows: slice | None = None):
+        """Launch the shard forward for B sequences x T tokens on the current stream.
+        Input: bf.tokens (first shard) or bf.h (other shards).  KV rows ``rows`` of the
+        cache are used (default: the first B)."""
+        c = self.cfg
+        R = B * T
+        Hq, Hkv, D = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+        rsl = rows if rows is not None else slice(0, B)
+        pos = cache.pos[rsl]
+        if self.is_first:
+            ops.embed(bf.tokens, self.embed_tokens, out=bf.h)
+        for li, L in enumerate(self.layers):
+            kc, vc = cache.k[li][rsl], cache.v[li][rsl]
+            ops.rms_norm(bf.h, L.in_norm, c.rms_norm_eps, out=bf.n)
+            ops.quantized_matmul(bf.n, L.qkv, out=bf.qkv)
+            ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
+                               L.q_norm, L.k_norm, c.rms_norm_eps)
+            if T == 1:
+                ops.sdpa_decode(bf.q, kc, vc, pos, bf.attn, bf.sdpa_ws, self.scale, B, Hq, Hkv, D)
+            else:
+                ops.sdpa_prefill(bf.q, kc, vc, pos, bf.attn, self.scale, B, T, Hq, Hkv, D)
+            ops.quantized_matmul(bf.attn, L.o, residual=bf.h, out=bf.h)
+            ops.rms_norm(bf.h, L.post_norm, c.rms_norm_eps, out=bf.n)
+            self._mlp(L, bf, R)
+        if not self.is_last or logits_mode == "none":
+            return bf.h
+        if logits_mode == "last" and T > 1:
+            hl = bf.h.view(B, T, -1)[:, -1].contiguous()
+            n = ops.rms_norm(hl, self.norm, c.rms_norm_eps)
+        else:
+            n = ops.rms_norm(bf.h, self.norm, c.rms_norm_eps, out=bf.n)
+        if bf.logits is None or bf.logits.shape[0] != n.shape[0]:
+            bf.logits = torch.empty(n.shape[0], c.vocab_size, dtype=torch.bfloat16, device=self.device)
+        ops.quantized_matmul(n, self.lm_head, out=bf.logits)
+        return bf.logits
+
+    def __call__(self, tokens: torch.Tensor | None, cache: ShardKVCache,
+                 input_embeddings: torch.Tensor | None = None, logits: str = "all",
+                 rows: slice | None = None) -> torch.Tensor:
+        """tokens int [B,T] (first shard) or input_embeddings bf16 [B,T,H] (other shards).
+        Appends T entries to the cache rows.  Returns bf16 logits [B,T,V] ("all"),
+        [B,1,V] ("last") on the last shard, else the hidden state [B,T,H]."""
+        if self.is_first:
+            assert tokens is not None
+            B, T = tokens.shape
+        else:
+            assert input_embeddings is not None
+            B, T = input_embeddings.shape[:2]
+        nrows = (rows.stop - rows.start) if rows is not None else B
+        if nrows != B or B > cache.batch:
+            raise ValueError(f"batch {B} does not match cache rows {nrows} (cache batch {cache.batch})")
+        r0 = rows.start if rows is not None else 0
+        if max(cache.offsets[r0 : r0 + B]) + T > cache.max_seq:
+            raise ValueError(f"KV cache overflow: {max(cache.offsets[r0:r0 + B])}+{T} > {cache.max_seq}")
+        bf = self._buffers(B, T)
+        if self.is_first:
+            bf.tokens.copy_(tokens.reshape(-1).to(torch.int32))
+        else:
+            bf.h.copy_(input_embeddings.reshape(B * T, -1))
+        out = self._run(B, T, cache, bf, logits if self.is_last else "none", rows)
+        cache.pos[r0 : r0 + B] += T
+        cache.advance_host(T, range(r0, r0 + B))
+        if self.is_last and logits != "none":
+            return out.view(B, -1, self.cfg.vocab_size).clone()
+        return out.view(B, T, -1).clone()
+
+    # ------------------------------------------------------------------ graph decode
+    def decode_step(self, cache: ShardKVCache, B: int, use_graph: bool = True) -> _Buffers:
+        """One single-token step for cache rows [0,B): reads ``bufs.tokens`` (first shard)
+        or ``bufs.h``, leaves logits / next_token / lse / logprob (last shard) or the
+        hidden state in the returned buffers, advances the device positions.  The kernel
+        sequence is captured once per B into a HIP graph and replayed."""
+        bf = self._buffers(B, 1)
+        if max(cache.offsets[:B]) + 1 > cache.max_seq:
+            raise ValueError("KV cache overflow")
+
+        def body():
+            out = self._run(B, 1, cache, bf, "all")
+            if self.is_last:
+                ops.argmax_logsumexp(out, bf.next_token, bf.lse, bf.logprob, bf.argmax_ws,
+                                     cache.pos[:B])
+            else:
+                cache.pos[:B] += 1
+
+        if not use_graph:
+            body()
+        else:
+            key = B
+            if key not in self._graphs or self._graphs[key][1] is not cache:
+                # warm up outside capture (lazy module loads, attribute settings), then
+                # restore the positions the warm-up advanced
+                saved = cache.pos.clone()
+                s = torch.cuda.Stream()
+                s.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(s):
+                    body()
+                torch.cuda.current_stream().wait_stream(s)
+                torch.cuda.synchronize()
+                cache.pos.copy_(saved)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    body()
+                cache.pos.copy_(saved)
+                self._graphs[key] = (g, cache)
+            self._graphs[key][0].replay()
+        cache.advance_host(1, range(B))
+        return bf

@@ -1,0 +1,238 @@
+"""End-to-end parity of the shard forward and the generation protocol on the GPU
+against the CPU oracle, on tiny random-weight checkpoints shared through safetensors."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import models as OM
+from tests.util import assert_close, load_checkpoint_numpy, n_f32, rng, tiny_config
+
+pytestmark = pytest.mark.gpu
+
+from exo_amd.config import ModelConfig  # noqa: E402
+from exo_amd.engine import Mi355xBuilder, ShardBatchGenerator  # noqa: E402
+from exo_amd.generate import generate, prefill  # noqa: E402
+from exo_amd.loader import load_shard_weights  # noqa: E402
+from exo_amd.model import ShardModel  # noqa: E402
+from exo_amd.synth import write_checkpoint  # noqa: E402
+from exo_amd.types import BoundInstance, GenerationTask, ShardMetadata, TextGenerationTaskParams  # noqa: E402
+
+KINDS = [("llama", 4), ("llama_tied_d128", 8), ("qwen3_moe", 4), ("qwen3_moe", 8)]
+
+
+def _load(path, cfg, start, end, device):
+    it = load_shard_weights(path, cfg, start, end, device)
+    progress = []
+    try:
+        while True:
+            progress.append(next(it))
+    except StopIteration as s:
+        return s.value, progress
+
+
+@pytest.fixture(scope="module", params=KINDS, ids=lambda k: f"{k[0]}-b{k[1]}")
+def ckpt(request, tmp_path_factory, device):
+    kind, bits = request.param
+    cfg = tiny_config(kind, bits)
+    path = write_checkpoint(tmp_path_factory.mktemp(f"{kind}{bits}"), cfg, seed=3, device="cpu")
+    ocfg, ow = load_checkpoint_numpy(path)
+    w, progress = _load(path, cfg, 0, cfg.num_hidden_layers, device)
+    assert progress == [(i + 1, cfg.num_hidden_layers) for i in range(cfg.num_hidden_layers)]
+    return dict(cfg=cfg, path=path, oracle=OM.ShardModel(ocfg, ow), model=ShardModel(cfg, w, device=device),
+                ocfg=ocfg, ow=ow)
+
+
+def test_prefill_and_decode_logits_match_oracle(ckpt, device):
+    cfg, om, gm = ckpt["cfg"], ckpt["oracle"], ckpt["model"]
+    prompt = rng(11).integers(0, cfg.vocab_size, size=40)
+    oc = OM.make_kv_cache(om.n_local_layers)
+    gc = gm.make_cache(1, 128)
+    want = om(prompt[None], oc)  # [1,40,V]
+    got = gm(torch.from_numpy(prompt[None].astype(np.int32)), gc)  # T=40 -> MFMA + prefill sdpa
+    assert gc[0].offset == 40 and oc[0].offset == 40
+    assert_close(n_f32(got), want, what="prefill logits")
+    # teacher-forced single-token steps (GEMV + decode sdpa)
+    for step in range(6):
+        t = int(rng(step).integers(0, cfg.vocab_size))
+        want = om(np.array([[t]]), oc)
+        got = gm(torch.tensor([[t]], dtype=torch.int32), gc)
+        assert_close(n_f32(got), want, what=f"decode logits step {step}")
+
+
+def test_short_multi_token_forward_uses_gemv_path(ckpt, device):
+    cfg, om, gm = ckpt["cfg"], ckpt["oracle"], ckpt["model"]
+    toks = rng(5).integers(0, cfg.vocab_size, size=(1, 7))
+    oc, gc = OM.make_kv_cache(om.n_local_layers), gm.make_cache(1, 64)
+    assert_close(n_f32(gm(torch.from_numpy(toks.astype(np.int32)), gc)), om(toks, oc), what="T=7")
+
+
+def test_greedy_tokens_identical_32_steps(ckpt, device):
+    cfg, om, gm = ckpt["cfg"], ckpt["oracle"], ckpt["model"]
+    prompt = [int(t) for t in rng(21).integers(0, cfg.vocab_size, size=24)]
+    want, wl = OM.greedy_generate(om, prompt, 32)
+    task = TextGenerationTaskParams(model="tiny", max_output_tokens=32, temperature=0.0)
+    got = [r.token for r in generate(gm, None, task, prompt)]
+    assert len(got) == 32
+    for i, (a, b) in enumerate(zip(got, want)):
+        if a != b:
+            top2 = np.sort(wl[i])[-2:]
+            margin = float(top2[1] - top2[0])
+            atol = 2e-2 * float(np.sqrt(np.mean(wl[i] ** 2)))
+            assert margin <= 2 * atol, f"step {i}: got {a} want {b}, margin {margin} > {2 * atol}"
+            pytest.xfail(f"near-tie at step {i} (margin {margin:.3e}); sequences diverge after it")
+    assert got == want
+
+
+def test_prefill_protocol_cache_lengths(ckpt, device):
+    gm = ckpt["model"]
+    cache = gm.make_cache(1, 64)
+    tps, n = prefill(gm, list(range(10)), cache)
+    assert n == 10 and cache[0].offset == 9  # len-1 after prefill
+    cache2 = gm.make_cache(1, 64)
+    prefill(gm, list(range(10)), cache2, faithful_extra_steps=False)
+    assert cache2[0].offset == 9
+    k1 = n_f32(cache.k[0][0, :, :9])
+    k2 = n_f32(cache2.k[0][0, :, :9])
+    np.testing.assert_array_equal(k1, k2)
+    c3 = gm.make_cache(1, 64)
+    assert prefill(gm, [], c3) == (0.0, 0) and c3[0].offset == 0
+    prefill(gm, [5], c3)
+    assert c3[0].offset == 0
+
+
+def test_pipeline_shards_compose(ckpt, device):
+    """shard [0,k) -> hidden -> shard [k,L) equals the full model (what config 5
+    compares: the hidden state leaving the last local layer)."""
+    cfg, om, gm, path = ckpt["cfg"], ckpt["oracle"], ckpt["model"], ckpt["path"]
+    L = cfg.num_hidden_layers
+    k = 1
+    w0, _ = _load(path, cfg, 0, k, device)
+    w1, _ = _load(path, cfg, k, L, device)
+    assert not any(n.startswith("lm_head") or n.startswith("model.norm") for n in w0)
+    s0, s1 = ShardModel(cfg, w0, 0, k, device), ShardModel(cfg, w1, k, L, device)
+    toks = rng(8).integers(0, cfg.vocab_size, size=(1, 20))
+    tt = torch.from_numpy(toks.astype(np.int32))
+    c0, c1, cf = s0.make_cache(1, 64), s1.make_cache(1, 64), gm.make_cache(1, 64)
+    assert len(c0) == k and len(c1) == L - k
+    hidden = s0(tt, c0)
+    assert hidden.shape == (1, 20, cfg.hidden_size)
+    o0 = OM.ShardModel(ckpt["ocfg"], ckpt["ow"], 0, k)
+    assert_close(n_f32(hidden), o0(toks, OM.make_kv_cache(k)), what="shard-0 hidden")
+    logits = s1(None, c1, input_embeddings=hidden)
+    full = gm(tt, cf)
+    np.testing.assert_array_equal(n_f32(logits), n_f32(full))
+
+
+def test_batch_generator_b2_equals_b1(ckpt, device):
+    """Port of the reference's B=2 vs B=1 criterion
+    (src/exo/worker/engines/mlx/tests/test_batch_generate.py:164-268): same greedy
+    tokens whether a request runs alone or next to another one."""
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    p1 = [int(t) for t in rng(31).integers(0, cfg.vocab_size, size=12)]
+    p2 = [int(t) for t in rng(32).integers(0, cfg.vocab_size, size=19)]
+    params = TextGenerationTaskParams(model="tiny", max_output_tokens=12, temperature=0.0)
+
+    def run(prompts):
+        g = ShardBatchGenerator(gm, None, max_batch=4, max_seq=128)
+        uids = [g.submit(params, p) for p in prompts]
+        toks = {u: [] for u in uids}
+        while g.has_work:
+            for u, r in g.step():
+                toks[u].append(r.token)
+        return [toks[u] for u in uids]
+
+    a1, = run([p1])
+    a2, = run([p2])
+    b1, b2 = run([p1, p2])
+    assert len(a1) == 12 and a1 == b1 and a2 == b2
+
+
+def test_batch_generator_slot_compaction_and_cancel(ckpt, device):
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    short = TextGenerationTaskParams(model="tiny", max_output_tokens=3, temperature=0.0)
+    long = TextGenerationTaskParams(model="tiny", max_output_tokens=9, temperature=0.0)
+    pa = [int(t) for t in rng(41).integers(0, cfg.vocab_size, size=9)]
+    pb = [int(t) for t in rng(42).integers(0, cfg.vocab_size, size=14)]
+    solo = ShardBatchGenerator(gm, None, 4, 128)
+    solo.submit(long, pb)
+    want = []
+    while solo.has_work:
+        want += [r.token for _, r in solo.step()]
+    g = ShardBatchGenerator(gm, None, 4, 128)
+    ua, ub = g.submit(short, pa), g.submit(long, pb)  # a finishes first; b moves to row 0
+    got, fin = [], {}
+    while g.has_work:
+        for u, r in g.step():
+            if u == ub:
+                got.append(r.token)
+            if r.finish_reason:
+                fin[u] = r.finish_reason
+                assert r.stats is not None and r.usage.completion_tokens in (3, 9)
+    assert got == want and fin == {ua: "length", ub: "length"}
+    uc = g.submit(long, pb)
+    g.step()
+    g.cancel([uc])
+    assert not g.has_work
+
+
+def test_builder_engine_contract(ckpt, device):
+    """Runner-side sequence of src/exo/worker/runner/runner.py:250-386: load (progress
+    events) -> build -> warmup -> submit -> step until Finished."""
+    cfg, path = ckpt["cfg"], ckpt["path"]
+
+    class Sender:
+        def __init__(self):
+            self.sent = []
+
+        def send(self, e):
+            self.sent.append(e)
+
+    class Receiver:
+        def __init__(self):
+            self.pending = []
+
+        def collect(self):
+            p, self.pending = self.pending, []
+            return p
+
+    sender, recv = Sender(), Receiver()
+    b = Mi355xBuilder("tiny/model", sender, recv, device=str(device), max_seq=256)
+    shard = ShardMetadata("tiny/model", 0, cfg.num_hidden_layers, cfg.num_hidden_layers)
+    inst = BoundInstance(shard, str(path))
+    prog = list(b.load(inst))
+    assert [(p.layers_loaded, p.total) for p in prog] == [
+        (i + 1, cfg.num_hidden_layers) for i in range(cfg.num_hidden_layers)]
+    eng = b.build()
+    eng.warmup()
+    assert eng.check_for_cancel_every >= 1
+    prompt = [int(t) for t in rng(51).integers(0, cfg.vocab_size, size=20)]
+    params = TextGenerationTaskParams(model="tiny/model", input=prompt, max_output_tokens=5,
+                                      temperature=0.0, bench=True)
+    eng.submit(GenerationTask("task-1", "cmd-1", params))
+    events = []
+    for _ in range(20):
+        events += list(eng.step())
+        if events and type(events[-1][1]).__name__ == "FinishedResponse":
+            break
+    kinds = [type(e).__name__ for _, e in events]
+    assert kinds == ["TokenChunk"] * 5 + ["FinishedResponse"]
+    assert events[4][1].finish_reason == "length" and events[4][1].stats.generation_tokens == 5
+    assert all(tid == "task-1" for tid, _ in events)
+    # cancellation of a running task
+    eng.submit(GenerationTask("task-2", "cmd-2", TextGenerationTaskParams(
+        model="tiny/model", input=prompt, max_output_tokens=500, temperature=0.0)))
+    list(eng.step())
+    recv.pending.append("task-2")
+    eng.check_for_cancel_every = 1
+    out = []
+    for _ in range(5):
+        out += list(eng.step())
+    assert ("task-2", "CancelledResponse") in [(t, type(e).__name__) for t, e in out]
+    # an error inside step is reported as an ErrorChunk before it propagates
+    eng.submit(GenerationTask("task-3", "cmd-3", TextGenerationTaskParams(model="tiny/model", input=[])))
+    with pytest.raises(ValueError):
+        list(eng.step())
+    assert type(sender.sent[-1][1]).__name__ == "ErrorChunk" and sender.sent[-1][0] == "cmd-3"
+    eng.close()
+    b.close()

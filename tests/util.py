@@ -80,3 +80,47 @@ def t_qw(triple, bits, device):
 
     w, s, b = triple
     return QuantizedWeight(t_u32(w, device), t_bf16(s, device), t_bf16(b, device), bits)
+
+
+# ---- checkpoints shared by the oracle and the GPU engine
+
+
+def load_checkpoint_numpy(path):
+    """MLX-layout safetensors -> {name: numpy} (uint32 words, uint16 bf16 bits) plus the
+    oracle Config."""
+    import json
+    from pathlib import Path
+
+    import torch
+    from safetensors.torch import load_file
+
+    from oracle.models import Config
+
+    path = Path(path)
+    out = {}
+    for f in sorted(path.glob("*.safetensors")):
+        for k, v in load_file(str(f)).items():
+            if v.dtype == torch.uint32:
+                out[k] = v.view(torch.int32).numpy().view(np.uint32)
+            elif v.dtype == torch.bfloat16:
+                out[k] = v.view(torch.int16).numpy().view(np.uint16)
+            else:
+                raise TypeError(f"{k}: {v.dtype}")
+    with open(path / "config.json") as fh:
+        cfg = Config.from_json(json.load(fh))
+    return cfg, out
+
+
+def tiny_config(kind: str, bits: int = 4):
+    from exo_amd.config import LLAMA3_SCALING, ModelConfig
+
+    if kind == "llama":
+        return ModelConfig("llama", 256, 3, 8, 2, 64, 512, 1000, 1e-5, 5e5,
+                           dict(LLAMA3_SCALING, factor=32.0), False, 64, bits)
+    if kind == "llama_tied_d128":
+        return ModelConfig("llama", 512, 2, 4, 2, 128, 1024, 777, 1e-5, 5e5,
+                           dict(LLAMA3_SCALING, factor=8.0), True, 64, bits)
+    if kind == "qwen3_moe":
+        return ModelConfig("qwen3_moe", 256, 2, 8, 2, 128, 0, 600, 1e-6, 1e6, None, False, 64, bits,
+                           8, 2, 128, True)
+    raise KeyError(kind)
