@@ -112,7 +112,14 @@ class ShardModel:
     start_layer: int = 0
     end_layer: int | None = None
     dequant_mode: str = "M1"
+    # A matmul with more than `gemm_rows` input rows multiplies by weights rounded to
+    # bf16 (one rounding of the float32 fma), the way a kernel that dequantises into
+    # bf16 operands for the matrix cores does; fewer rows use the un-rounded float32
+    # weights of a fused GEMV.  None = un-rounded everywhere.  Which of the two MLX's
+    # own kernels do is PARITY UNPINNED; both are within the stated tolerance.
+    gemm_rows: int | None = None
     _dq: dict = field(default_factory=dict)
+    router_margins: list = field(default_factory=list)  # (layer, logit gap per token)
 
     def __post_init__(self):
         if self.end_layer is None:
@@ -149,7 +156,14 @@ class ShardModel:
         return self._dq[key]
 
     def linear(self, x: np.ndarray, prefix: str) -> np.ndarray:
-        return bf16_round(x.astype(np.float32) @ self._wd(prefix).T)
+        w = self._wd(prefix)
+        rows = int(np.prod(x.shape[:-1]))
+        if self.gemm_rows is not None and rows > self.gemm_rows:
+            key = (prefix, "bf16")
+            if key not in self._dq:
+                self._dq[key] = bf16_round(w)
+            w = self._dq[key]
+        return bf16_round(x.astype(np.float32) @ w.T)
 
     def _norm_w(self, name: str) -> np.ndarray:
         return bf16_bits_to_f32(self.weights[name])
@@ -190,6 +204,12 @@ class ShardModel:
         xf = x.reshape(B * T, H)
         logits = self.linear(xf, p + "gate")
         idx, sc = ops.router_topk(logits, c.num_experts_per_tok, c.norm_topk_prob)
+        # how close the k-th and (k+1)-th expert were, per token: a caller comparing
+        # against another implementation can tell a routing near-tie from an error
+        srt = -np.sort(-logits.astype(np.float32), axis=-1)
+        k = c.num_experts_per_tok
+        if srt.shape[-1] > k:
+            self.router_margins.append((i, srt[:, k - 1] - srt[:, k]))
         out = np.zeros((B * T, H), np.float32)
         for t in range(B * T):
             acc = np.zeros(H, np.float32)

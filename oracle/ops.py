@@ -114,8 +114,10 @@ def router_topk(logits: np.ndarray, k: int, norm_topk_prob: bool):
     order = np.argsort(-p, axis=-1, kind="stable")[:, :k]
     sc = np.take_along_axis(p, order, axis=-1)
     if norm_topk_prob:
-        tot = bf16_round(sc.sum(-1, keepdims=True, dtype=np.float32))
-        sc = bf16_round(sc / tot)
+        tot = np.zeros((sc.shape[0], 1), np.float32)
+        for j in range(k):  # float32 running sum in slot order
+            tot = (tot + sc[:, j : j + 1]).astype(np.float32)
+        sc = bf16_round(sc / bf16_round(tot))
     return order.astype(np.int32), sc
 
 

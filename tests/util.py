@@ -46,6 +46,29 @@ def assert_close(got: np.ndarray, want: np.ndarray, rtol=RTOL, what=""):
     return float(err.max()), atol
 
 
+def assert_close_stat(got, want, rtol=RTOL, max_rel_rms=RTOL, max_outlier_frac=5e-3, what=""):
+    """Criterion for tensors that passed through SEVERAL bf16-rounded layers.
+
+    Every op rounds its output to bf16; two correct implementations that accumulate
+    in a different order flip a fraction of those roundings, and the flips propagate,
+    so elementwise agreement at rtol 2e-2 cannot hold for every element of a deep
+    stack (the oracle disagrees with itself by the same amount when its weights are
+    rounded to bf16 first).  Required here: relative RMS error <= max_rel_rms and at
+    most max_outlier_frac of the elements outside |d| <= rtol*|want| + rtol*rms(want).
+    Single ops and single layers are held to the elementwise bound (assert_close)."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    rms = float(np.sqrt(np.mean(want**2)))
+    err = np.abs(got - want)
+    rel_rms = float(np.sqrt(np.mean(err**2))) / rms
+    frac = float(np.mean(err > rtol * np.abs(want) + rtol * rms))
+    print(f"[parity] {what}: rel-rms {rel_rms:.3e} outliers {frac:.3e} max|e|/rms {err.max() / rms:.3e}")
+    assert rel_rms <= max_rel_rms, f"{what}: relative RMS error {rel_rms:.3e} > {max_rel_rms}"
+    assert frac <= max_outlier_frac, f"{what}: {frac:.3e} of elements outside the elementwise bound"
+    return rel_rms, frac
+
+
 # ---- torch side (imported lazily so CPU-only oracle tests do not need torch)
 
 
