@@ -300,14 +300,18 @@ class BatchGenerator(Engine):
     event_sender: Any = None
     check_for_cancel_every: int = 50
     max_seq: int = 8192
+    gen_factory: Any = None  # tests inject a fake inner generator (like the reference's FakeExoBatchGenerator)
     _cancelled_tasks: set = field(default_factory=set, init=False)
     _all_tasks: dict = field(default_factory=dict, init=False)
     _queue: deque = field(default_factory=deque, init=False)
     _active_tasks: dict = field(default_factory=dict, init=False)
 
     def __post_init__(self) -> None:
-        self._gen = ShardBatchGenerator(self.model, self.tokenizer, EXO_MAX_CONCURRENT_REQUESTS,
-                                        self.max_seq)
+        if self.gen_factory is not None:
+            self._gen = self.gen_factory()
+        else:
+            self._gen = ShardBatchGenerator(self.model, self.tokenizer, EXO_MAX_CONCURRENT_REQUESTS,
+                                            self.max_seq)
 
     def warmup(self) -> None:
         """generate.py:399-462: a short greedy generation on a fixed prompt; sets how

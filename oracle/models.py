@@ -24,7 +24,8 @@ from dataclasses import dataclass, field
 import numpy as np
 
 from . import affine, ops
-from .affine import bf16_bits_to_f32, bf16_round
+from .affine import act_round as bf16_round
+from .affine import bf16_bits_to_f32
 
 
 @dataclass
@@ -118,6 +119,9 @@ class ShardModel:
     # weights of a fused GEMV.  None = un-rounded everywhere.  Which of the two MLX's
     # own kernels do is PARITY UNPINNED; both are within the stated tolerance.
     gemm_rows: int | None = None
+    # use the C restatement (oracle/qmm_ref.c) for matmuls of at most 16 rows: same
+    # arithmetic, no dequantised copy of the matrix, OpenMP over output rows
+    use_c: bool = False
     _dq: dict = field(default_factory=dict)
     router_margins: list = field(default_factory=list)  # (layer, logit gap per token)
 
@@ -156,8 +160,15 @@ class ShardModel:
         return self._dq[key]
 
     def linear(self, x: np.ndarray, prefix: str) -> np.ndarray:
-        w = self._wd(prefix)
         rows = int(np.prod(x.shape[:-1]))
+        if self.use_c and rows <= 16:
+            from . import cref
+
+            y = cref.qmm_t(
+                affine.f32_to_bf16_bits(x.reshape(rows, -1)), self.weights[prefix + ".weight"],
+                self.weights[prefix + ".scales"], self.weights[prefix + ".biases"], self.cfg.bits)
+            return bf16_bits_to_f32(y).reshape(*x.shape[:-1], -1)
+        w = self._wd(prefix)
         if self.gemm_rows is not None and rows > self.gemm_rows:
             key = (prefix, "bf16")
             if key not in self._dq:

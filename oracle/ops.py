@@ -17,7 +17,7 @@ import math
 
 import numpy as np
 
-from .affine import bf16_round
+from .affine import act_round as bf16_round
 
 
 def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:

@@ -1,0 +1,306 @@
+"""Host-side logic that needs no GPU: C-ABI surface, loader, config, cache bookkeeping,
+Engine event ordering with a faked inner generator, samplers."""
+
+import ctypes
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from exo_amd import native
+from exo_amd.config import ModelConfig, named_config
+from exo_amd.engine import BatchGenerator, build_model_path
+from exo_amd.generate import PrefillCancelled, ban_token_ids, extract_top_logprobs, make_sampler
+from exo_amd.loader import layer_index_of, load_shard_weights, wanted
+from exo_amd.synth import synth_weights, write_checkpoint
+from exo_amd.tokenizer import IdTokenizer, load_tokenizer
+from exo_amd.types import GenerationResponse, GenerationTask, TextGenerationTaskParams
+from tests.util import tiny_config
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+# ------------------------------------------------------------------ C ABI
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "exo_mi355x.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(exo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    syms = _declared_symbols()
+    assert len(syms) >= 20
+    assert native.LIB_PATH.exists(), "build with `python -m exo_amd.build`"
+    lib = ctypes.CDLL(str(native.LIB_PATH))  # loads without a GPU
+    for s in syms:
+        assert hasattr(lib, s), f"{s} declared in include/exo_mi355x.h but not exported"
+    assert sorted(native.SIGNATURES) == syms  # the ctypes table covers the header one to one
+
+
+def test_argument_errors_without_gpu():
+    lib = native.load()
+    assert lib.exo_abi_version() == 1
+    # argument validation happens before any HIP call
+    assert lib.exo_qmv(None, None, None, None, None, None, 1, 64, 128, 3, 64, None) == -1
+    assert b"bits must be 4 or 8" in lib.exo_last_error()
+    assert lib.exo_qmm(None, None, None, None, None, None, 1, 64, 100, 4, 64, None) == -1
+    assert lib.exo_sdpa_decode(None, None, None, None, None, None, 1.0, 1, 8, 3, 128, 64, None) == -1
+    assert lib.exo_router_topk(None, None, None, 1, 300, 8, 1, None) == -1
+    assert lib.exo_sdpa_decode_workspace(2, 32, 128) == 2 * 32 * 64 * 130 * 4
+    with pytest.raises(ValueError):
+        native.check(-1, "x")
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(native, "_lib", None)
+    monkeypatch.setattr(native, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(native.NativeError):
+        native.load()
+
+
+# ------------------------------------------------------------------ config / loader
+
+
+def test_named_configs_weight_bytes_match_the_stated_figures():
+    def qbytes(n, k, bits):
+        return n * k * bits // 8 + n * (k // 64) * 4
+
+    c = named_config("llama-3.1-8b")
+    H, D, I = c.hidden_size, c.head_dim, c.intermediate_size
+    layer = (qbytes(c.num_attention_heads * D, H, 4) + 2 * qbytes(c.num_key_value_heads * D, H, 4)
+             + qbytes(H, c.num_attention_heads * D, 4) + 2 * qbytes(I, H, 4) + qbytes(H, I, 4))
+    assert layer == 122_683_392 and 32 * layer + qbytes(c.vocab_size, H, 4) == 4_221_370_368
+    c1 = named_config("llama-3.2-1b")
+    l1 = (qbytes(2048, 2048, 4) * 2 + 2 * qbytes(512, 2048, 4) + 3 * qbytes(8192, 2048, 4))
+    assert 16 * l1 + qbytes(c1.vocab_size, 2048, 4) == 695_107_584
+
+
+def test_config_round_trip_and_rejects():
+    c = tiny_config("qwen3_moe", 8)
+    d = c.to_dict()
+    assert d["quantization"] == {"group_size": 64, "bits": 8}
+    assert ModelConfig.from_dict(json.loads(json.dumps(d))) == c
+    with pytest.raises(ValueError):
+        ModelConfig.from_dict(dict(d, model_type="gpt2"))
+    with pytest.raises(ValueError):
+        ModelConfig.from_dict(dict(d, quantization={"group_size": 32, "bits": 4}))
+
+
+def test_shard_tensor_selection_rule():
+    c = tiny_config("llama")
+    assert layer_index_of("model.layers.12.self_attn.q_proj.weight") == 12
+    assert layer_index_of("model.norm.weight") is None
+    assert wanted("model.layers.1.mlp.up_proj.scales", c, 1, 2)
+    assert not wanted("model.layers.0.mlp.up_proj.scales", c, 1, 2)
+    assert wanted("model.embed_tokens.weight", c, 0, 1) and not wanted("model.embed_tokens.weight", c, 1, 3)
+    assert wanted("lm_head.weight", c, 1, 3) and not wanted("lm_head.weight", c, 0, 2)
+    tied = tiny_config("llama_tied_d128")
+    assert wanted("model.embed_tokens.weight", tied, 1, 2)  # tied head lives in the embedding
+
+
+@pytest.mark.parametrize("kind", ["llama", "qwen3_moe"])
+def test_checkpoint_round_trip_and_progress(tmp_path, kind):
+    cfg = tiny_config(kind)
+    path = write_checkpoint(tmp_path / "m", cfg, seed=1)
+    ref = synth_weights(cfg, seed=1)
+    it = load_shard_weights(path, cfg, 0, cfg.num_hidden_layers, "cpu")
+    prog = []
+    try:
+        while True:
+            prog.append(next(it))
+    except StopIteration as stop:
+        got = stop.value
+    assert prog == [(i + 1, cfg.num_hidden_layers) for i in range(cfg.num_hidden_layers)]
+    assert set(got) == set(ref)
+    for k in ref:
+        assert got[k].dtype == ref[k].dtype and torch.equal(got[k], ref[k]), k
+    # a middle shard gets only its own layer
+    it = load_shard_weights(path, cfg, 1, 2, "cpu")
+    try:
+        while True:
+            next(it)
+    except StopIteration as stop:
+        mid = stop.value
+    is_last = cfg.num_hidden_layers == 2  # then the shard also owns final norm + head
+    assert all(layer_index_of(k) == 1 or (is_last and layer_index_of(k) is None) for k in mid)
+    assert len(mid) > 5 and not any(k.startswith("model.embed_tokens") for k in mid)
+    # shapes follow the MLX layout
+    w = got["model.layers.0.self_attn.q_proj.weight"]
+    assert w.shape == (cfg.num_attention_heads * cfg.head_dim, cfg.hidden_size * cfg.bits // 32)
+    if cfg.is_moe:
+        assert got["model.layers.0.mlp.switch_mlp.down_proj.scales"].shape == (
+            cfg.num_experts, cfg.hidden_size, cfg.moe_intermediate_size // 64)
+
+
+def test_build_model_path_search_order(tmp_path, monkeypatch):
+    ro, rw, default = tmp_path / "ro", tmp_path / "rw", tmp_path / "def"
+    for d in (ro, rw, default):
+        (d / "org--name").mkdir(parents=True)
+    monkeypatch.setenv("EXO_MODELS_READ_ONLY_DIRS", str(ro))
+    monkeypatch.setenv("EXO_MODELS_DIRS", str(rw))
+    monkeypatch.setenv("EXO_DEFAULT_MODELS_DIR", str(default))
+    assert build_model_path("org/name") == default / "org--name"  # nothing complete yet
+    (rw / "org--name" / "config.json").write_text("{}")
+    assert build_model_path("org/name") == rw / "org--name"
+    (ro / "org--name" / "config.json").write_text("{}")
+    assert build_model_path("org/name") == ro / "org--name"
+
+
+def test_tokenizers():
+    t = load_tokenizer("/nonexistent", 100)
+    assert isinstance(t, IdTokenizer) and t.encode("5 17 205") == [5, 17, 5] and t.decode([3, 4]) == "3 4 "
+
+
+# ------------------------------------------------------------------ sampling
+
+
+def test_samplers():
+    lp = torch.log_softmax(torch.tensor([[0.0, 3.0, 1.0, 2.5]]), -1)
+    assert make_sampler(0.0)(lp).tolist() == [1]
+    g = torch.Generator().manual_seed(0)
+    draws = torch.stack([make_sampler(1.0, top_k=2, generator=g)(lp) for _ in range(200)])
+    assert set(draws.flatten().tolist()) == {1, 3}
+    draws = torch.stack([make_sampler(1.0, min_p=0.9, generator=g)(lp) for _ in range(50)])
+    assert set(draws.flatten().tolist()) == {1}
+    draws = torch.stack([make_sampler(1.0, top_p=0.5, generator=g)(lp) for _ in range(50)])
+    assert set(draws.flatten().tolist()) == {1}
+    banned = ban_token_ids([1])(torch.tensor([0]), torch.tensor([[0.0, 3.0, 1.0, 2.5]]))
+    assert banned[0, 1] == -1e9 and torch.argmax(banned) == 3
+    lpv, top = extract_top_logprobs(lp[0], None, 3, 2)
+    assert [t.token for t in top] == ["1", "3", "2"] and abs(lpv - float(lp[0, 2])) < 1e-6
+
+
+# ------------------------------------------------------------------ Engine event ordering
+
+
+class FakeGen:
+    """Port of the reference's FakeExoBatchGenerator
+    (src/exo/worker/tests/unittests/test_runner/test_event_ordering.py:161-198)."""
+
+    def __init__(self, fail_on_step=False):
+        self.active, self.cancelled, self.next_uid = {}, [], 0
+        self.fail_on_step = fail_on_step
+
+    @property
+    def has_work(self):
+        return bool(self.active)
+
+    def submit(self, task_params, prompt, on_prefill_progress=None,
+               distributed_prompt_progress_callback=None, on_generation_token=None):
+        if distributed_prompt_progress_callback:
+            distributed_prompt_progress_callback()
+        if on_prefill_progress:
+            on_prefill_progress(len(prompt), len(prompt))
+        uid = self.next_uid
+        self.next_uid += 1
+        self.active[uid] = [0, task_params.max_output_tokens or 3, on_generation_token]
+        return uid
+
+    def step(self):
+        if self.fail_on_step:
+            raise RuntimeError("device fault")
+        out = []
+        for uid, st in list(self.active.items()):
+            st[0] += 1
+            done = st[0] >= st[1]
+            if st[2]:
+                st[2]()
+            out.append((uid, GenerationResponse(text="x", token=st[0], finish_reason="length" if done else None)))
+            if done:
+                del self.active[uid]
+        return out
+
+    def cancel(self, uids):
+        self.cancelled += uids
+        for u in uids:
+            self.active.pop(u, None)
+
+    def close(self):
+        self.active.clear()
+
+
+class _Sender:
+    def __init__(self):
+        self.sent = []
+
+    def send(self, e):
+        self.sent.append(e)
+
+
+class _Receiver:
+    def __init__(self):
+        self.pending = []
+
+    def collect(self):
+        p, self.pending = self.pending, []
+        return p
+
+
+def _engine(**kw):
+    s, r = _Sender(), _Receiver()
+    gen = FakeGen(**kw)
+    e = BatchGenerator(model=None, tokenizer=IdTokenizer(100), model_id="m", cancel_receiver=r,
+                       event_sender=s, gen_factory=lambda: gen)
+    return e, gen, s, r
+
+
+def _task(tid, n=2, prompt=(1, 2, 3)):
+    return GenerationTask(tid, "cmd-" + tid, TextGenerationTaskParams(model="m", input=list(prompt), max_output_tokens=n))
+
+
+def test_engine_event_sequence():
+    e, gen, s, _ = _engine()
+    assert list(e.step()) == []
+    e.submit(_task("a", 2))
+    e.submit(_task("b", 3))
+    ev = []
+    for _ in range(4):
+        ev += [(t, type(x).__name__, getattr(x, "finish_reason", None)) for t, x in e.step()]
+    assert ev == [("a", "TokenChunk", None), ("b", "TokenChunk", None),
+                  ("a", "TokenChunk", "length"), ("a", "FinishedResponse", None), ("b", "TokenChunk", None),
+                  ("b", "TokenChunk", "length"), ("b", "FinishedResponse", None)]
+    # prefill progress chunks were sent on the event channel, tagged with the command id
+    assert [(c, type(x).__name__) for c, x in s.sent] == [("cmd-a", "PrefillProgressChunk"), ("cmd-b", "PrefillProgressChunk")]
+
+
+def test_engine_concurrency_cap_and_cancellation():
+    e, gen, _, r = _engine()
+    for i in range(10):
+        e.submit(_task(f"t{i}", 50))
+    e.step()
+    assert len(gen.active) == 8 and len(e._queue) == 2  # EXO_MAX_CONCURRENT_REQUESTS
+    r.pending += ["t3", "unknown-task"]
+    e.check_for_cancel_every = 1
+    out = []
+    for _ in range(3):
+        out += [(t, type(x).__name__) for t, x in e.step()]
+    assert ("t3", "CancelledResponse") in out and 3 in gen.cancelled
+    r.pending.append("CANCEL_ALL_TASKS")
+    out = []
+    for _ in range(3):
+        out += [(t, type(x).__name__) for t, x in e.step()]
+    assert {t for t, k in out if k == "CancelledResponse"} >= {"t0", "t1", "t2"}
+    assert not gen.has_work or len(gen.active) <= 2
+
+
+def test_engine_prefill_cancel_and_errors():
+    e, gen, s, r = _engine()
+    r.pending.append("z")
+    e._all_tasks["z"] = None
+    e.submit(_task("z"))
+    assert list(e.step()) == [] or True
+    assert not gen.active  # PrefillCancelled swallowed, task dropped
+    e2, gen2, s2, _ = _engine(fail_on_step=True)
+    e2.submit(_task("q"))
+    with pytest.raises(RuntimeError):
+        e2.step()
+    assert type(s2.sent[-1][1]).__name__ == "ErrorChunk" and s2.sent[-1][0] == "cmd-q"
+    with pytest.raises(NotImplementedError):
+        e2.serve_prefill(None, None)
+    with pytest.raises(PrefillCancelled):
+        raise PrefillCancelled()
