@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 greedy decode of a Llama-3.1-8B-architecture model on MLX
+4-bit g64 weights, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one decoded token: the full shard forward (32 layers + head) as a HIP
+graph replay at a context of about 2048 tokens, weights and KV cache resident in HBM,
+greedy sampling on the device.  Prints ONE JSON line: decode tok/s (`value`), the
+roofline of the dominant kernel (the fused dequant-GEMV, measured live with HIP events)
+and the CPU oracle timed on this box's host cores (`cpu_baseline`, reported only).
+
+Weights are synthetic (N(0,0.02) -> bf16 -> mx.quantize-style affine 4-bit g64), the
+prompt is 2048 uniform random token ids; see `data` in the output.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", default="llama-3.1-8b")
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="debug: truncate the model")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-graph", action="store_true")
+    return ap.parse_args()
+
+
+def qbytes(n: int, k: int, bits: int) -> int:
+    return n * k * bits // 8 + n * (k // 64) * 4
+
+
+def measure_kernels(model, torch, reps: int = 20):
+    """Per-kernel HBM roofline of the GEMV launches of one decode step.  Each group of
+    same-shaped launches (one per layer, distinct weights, 4.2 GB in total so nothing
+    is served from cache) is captured into a HIP graph and timed with events on the
+    launch stream; average launch duration = elapsed / launches."""
+    from exo_amd import ops
+
+    c = model.cfg
+    dev = model.device
+    H, D = c.hidden_size, c.head_dim
+    Hq, Hkv, I = c.num_attention_heads, c.num_key_value_heads, c.intermediate_size
+    bf = dict(dtype=torch.bfloat16, device=dev)
+    xh = torch.randn(1, H, device=dev).to(torch.bfloat16)
+    xa = torch.randn(1, Hq * D, device=dev).to(torch.bfloat16)
+    xi = torch.randn(1, I, device=dev).to(torch.bfloat16)
+    y_qkv = torch.empty(1, (Hq + 2 * Hkv) * D, **bf)
+    y_h = torch.empty(1, H, **bf)
+    y_i = torch.empty(1, I, **bf)
+    y_v = torch.empty(1, c.vocab_size, **bf)
+    groups = {
+        "gate_up_swiglu": (lambda L: ops.qmv_swiglu(xh, L.gate, L.up, out=y_i),
+                           2 * qbytes(I, H, c.bits) + 2 * (H + I), "qmv_kernel<%d,1,2>" % c.bits),
+        "down": (lambda L: ops.quantized_matmul(xi, L.down, out=y_h),
+                 qbytes(H, I, c.bits) + 2 * (I + H), "qmv_kernel<%d,1,1>" % c.bits),
+        "qkv": (lambda L: ops.quantized_matmul(xh, L.qkv, out=y_qkv),
+                qbytes((Hq + 2 * Hkv) * D, H, c.bits) + 2 * (H + (Hq + 2 * Hkv) * D),
+                "qmv_kernel<%d,1,1>" % c.bits),
+        "o": (lambda L: ops.quantized_matmul(xa, L.o, out=y_h),
+              qbytes(H, Hq * D, c.bits) + 2 * (Hq * D + H), "qmv_kernel<%d,1,1>" % c.bits),
+    }
+    out = []
+    for name, (fn, nbytes, kname) in groups.items():
+        for L in model.layers:  # warm-up (also sets kernel attributes outside capture)
+            fn(L)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for L in model.layers:
+                fn(L)
+        g.replay()
+        torch.cuda.synchronize()
+        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        st.record()
+        for _ in range(reps):
+            g.replay()
+        en.record()
+        torch.cuda.synchronize()
+        us = st.elapsed_time(en) * 1e3 / (reps * len(model.layers))
+        out.append(dict(name=name, kernel=kname, launches_per_token=len(model.layers),
+                        bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
+    # lm_head: one launch per token; rotate nothing (295 MB >> caches)
+    ops.quantized_matmul(xh, model.lm_head, out=y_v)
+    torch.cuda.synchronize()
+    st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    st.record()
+    for _ in range(reps):
+        ops.quantized_matmul(xh, model.lm_head, out=y_v)
+    en.record()
+    torch.cuda.synchronize()
+    us = st.elapsed_time(en) * 1e3 / reps
+    nbytes = qbytes(c.vocab_size, H, c.bits) + 2 * (H + c.vocab_size)
+    out.append(dict(name="lm_head", kernel="qmv_kernel<%d,1,1>" % c.bits, launches_per_token=1,
+                    bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
+    return out
+
+
+def cpu_baseline(model, torch, seconds: float, context: int):
+    """The CPU oracle (C restatement of the quantised matmul + numpy ops) timed on this
+    host: one decode token of the same architecture at the same context length.
+    Bounded sample: 2 layers + head are run and the layer time is scaled to the full
+    depth."""
+    from oracle import cref
+    from oracle import models as OM
+
+    c = model.cfg
+    n_sample = min(2, len(model.layers))
+
+    def to_np(t):
+        t = t.detach().cpu().contiguous()
+        if t.dtype == torch.int32:
+            return t.numpy().view(np.uint32)
+        return t.view(torch.int16).numpy().view(np.uint16)
+
+    w = {}
+
+    def put(prefix, q):
+        w[prefix + ".weight"], w[prefix + ".scales"], w[prefix + ".biases"] = (
+            to_np(q.weight), to_np(q.scales), to_np(q.biases))
+
+    Hq, Hkv, D = c.num_attention_heads, c.num_key_value_heads, c.head_dim
+    for i in range(n_sample):
+        L = model.layers[i]
+        p = f"model.layers.{i}."
+        nq, nk = Hq * D, Hkv * D
+        put(p + "self_attn.q_proj", L.qkv[0:nq])
+        put(p + "self_attn.k_proj", L.qkv[nq : nq + nk])
+        put(p + "self_attn.v_proj", L.qkv[nq + nk : nq + 2 * nk])
+        put(p + "self_attn.o_proj", L.o)
+        put(p + "mlp.gate_proj", L.gate)
+        put(p + "mlp.up_proj", L.up)
+        put(p + "mlp.down_proj", L.down)
+        w[p + "input_layernorm.weight"] = to_np(L.in_norm)
+        w[p + "post_attention_layernorm.weight"] = to_np(L.post_norm)
+    put("model.embed_tokens", model.embed_tokens)
+    put("lm_head", model.lm_head)
+    w["model.norm.weight"] = to_np(model.norm)
+    ocfg = OM.Config(model_type=c.model_type, hidden_size=c.hidden_size, num_hidden_layers=n_sample,
+                     num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
+                     intermediate_size=c.intermediate_size, vocab_size=c.vocab_size,
+                     rms_norm_eps=c.rms_norm_eps, rope_theta=c.rope_theta, rope_scaling=c.rope_scaling,
+                     tie_word_embeddings=False, group_size=64, bits=c.bits)
+    om = OM.ShardModel(ocfg, w, use_c=True)
+    rng = np.random.default_rng(0)
+    cache = OM.make_kv_cache(n_sample)
+    from oracle.affine import bf16_round
+
+    for kv in cache:  # a context of `context` cached tokens (synthetic K/V)
+        kv.k = bf16_round(rng.standard_normal((1, Hkv, context, D)).astype(np.float32))
+        kv.v = bf16_round(rng.standard_normal((1, Hkv, context, D)).astype(np.float32))
+        kv.offset = context
+    tok = np.array([[1]])
+    om(tok, cache)  # warm-up
+    for kv in cache:
+        kv.trim(1)
+    t_full, n_full, t0 = 0.0, 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds * 0.7 or n_full < 2:
+        a = time.perf_counter()
+        om(tok, cache)
+        t_full += time.perf_counter() - a
+        n_full += 1
+        for kv in cache:
+            kv.trim(1)
+    x = bf16_round(rng.standard_normal((1, c.hidden_size)).astype(np.float32))
+    t_head, n_head, t0 = 0.0, 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds * 0.3 or n_head < 2:
+        a = time.perf_counter()
+        om.linear(x, "lm_head")
+        t_head += time.perf_counter() - a
+        n_head += 1
+    t_full /= n_full
+    t_head /= n_head
+    t_layer = max(t_full - t_head, 1e-9) / n_sample
+    t_token = t_layer * c.num_hidden_layers + t_head
+    return dict(value=1.0 / t_token, unit="tok/s", cores=cref.num_threads(), kind="port",
+                sample=(f"{n_full} decode steps of {n_sample} layers + lm_head at context {context} "
+                        f"(layer {t_layer * 1e3:.1f} ms, head {t_head * 1e3:.1f} ms), layer time "
+                        f"scaled to {c.num_hidden_layers} layers; oracle/qmm_ref.c with OpenMP + numpy"),
+                host_cpus=os.cpu_count(), affinity=len(os.sched_getaffinity(0)))
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (per-shard forward); --gpus {args.gpus} is not "
+              "supported. Multi-GPU pipeline/tensor sharding is design-only (see DESIGN.md).",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from exo_amd import native
+    from exo_amd.config import named_config
+    from exo_amd.generate import prefill
+    from exo_amd.model import ShardModel
+    from exo_amd.synth import synth_weights
+
+    native.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = named_config(args.config)
+    if args.layers:
+        cfg.num_hidden_layers = args.layers
+    t0 = time.perf_counter()
+    weights = synth_weights(cfg, seed=0, device=dev)
+    model = ShardModel(cfg, weights, device=dev)
+    del weights
+    torch.cuda.synchronize()
+    t_build = time.perf_counter() - t0
+
+    g = torch.Generator().manual_seed(1234)
+    prompt = torch.randint(0, cfg.vocab_size, (args.prompt,), generator=g).tolist()
+    K, W = args.steps, args.warmup
+    cache = model.make_cache(1, args.prompt + K + W + 64)
+
+    # prefill with the reference's protocol, then the last-but-one token as a GEMV step
+    tps_prefill, n_prefill = prefill(model, prompt[:-1], cache)
+    model(torch.tensor([[prompt[-2]]], dtype=torch.int32), cache, logits="none")
+    bufs = model._buffers(1, 1)
+    bufs.tokens[0] = prompt[-1]
+
+    def step():
+        return model.decode_step(cache, 1, use_graph=not args.no_graph, feedback=True)
+
+    toks = []
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    ctx0 = cache[0].offset
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    toks.append(int(bufs.next_token[0]))
+    tok_s = K / dt
+
+    kernels = measure_kernels(model, torch)
+    for k in kernels:
+        k["frac_of_8TBps"] = k["GBps"] / 8000.0
+        k["us_per_token"] = k["avg_us"] * k["launches_per_token"]
+    dom = max(kernels, key=lambda k: k["us_per_token"])
+    gemv_us = sum(k["us_per_token"] for k in kernels)
+    gemv_bytes = sum(k["bytes_per_launch"] * k["launches_per_token"] for k in kernels)
+    roofline = dict(bound="hbm", achieved=dom["GBps"], peak=8000.0, unit="GB/s",
+                    frac=dom["GBps"] / 8000.0, traffic=None, kernel=dom["kernel"],
+                    launch=dom["name"], avg_us=dom["avg_us"], bytes_per_launch=dom["bytes_per_launch"],
+                    all_gemv_GBps=gemv_bytes / gemv_us * 1e-3, all_gemv_us_per_token=gemv_us)
+
+    kv_bytes = 2 * len(model.layers) * cfg.num_key_value_heads * cfg.head_dim * ctx0 * 2
+    token_bytes = model.weight_bytes() + kv_bytes
+    out = {
+        "metric": "decode tok/s + qmatmul HBM GB/s (% peak), Llama-3.1-8B 4-bit g64 bs1",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": dt / K * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"configs[2]: {args.config} architecture, MLX affine {cfg.bits}-bit g64, "
+                               f"random prompt of {args.prompt} tokens, greedy decode, batch 1",
+                   "layers": cfg.num_hidden_layers, "context_at_start": ctx0, "hip_graph": not args.no_graph},
+        "roofline": roofline,
+        "prefill_tok_s": tps_prefill, "prefill_tokens": n_prefill,
+        "token_bytes": token_bytes, "effective_GBps": token_bytes * tok_s * 1e-9,
+        "kernels": kernels, "build_s": t_build, "last_token": toks[-1],
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(model, torch, args.cpu_seconds, ctx0)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

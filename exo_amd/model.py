@@ -269,11 +269,14 @@ class ShardModel:
         return out.view(B, T, -1).clone()
 
     # ------------------------------------------------------------------ graph decode
-    def decode_step(self, cache: ShardKVCache, B: int, use_graph: bool = True) -> _Buffers:
+    def decode_step(self, cache: ShardKVCache, B: int, use_graph: bool = True,
+                    feedback: bool = False) -> _Buffers:
         """One single-token step for cache rows [0,B): reads ``bufs.tokens`` (first shard)
         or ``bufs.h``, leaves logits / next_token / lse / logprob (last shard) or the
         hidden state in the returned buffers, advances the device positions.  The kernel
-        sequence is captured once per B into a HIP graph and replayed."""
+        sequence is captured once per B into a HIP graph and replayed.  ``feedback``
+        (last shard, greedy): the graph also copies next_token into tokens, so steps
+        can be chained without the host."""
         bf = self._buffers(B, 1)
         if max(cache.offsets[:B]) + 1 > cache.max_seq:
             raise ValueError("KV cache overflow")
@@ -283,13 +286,15 @@ class ShardModel:
             if self.is_last:
                 ops.argmax_logsumexp(out, bf.next_token, bf.lse, bf.logprob, bf.argmax_ws,
                                      cache.pos[:B])
+                if feedback:
+                    bf.tokens.copy_(bf.next_token)
             else:
                 cache.pos[:B] += 1
 
         if not use_graph:
             body()
         else:
-            key = B
+            key = (B, feedback)
             if key not in self._graphs or self._graphs[key][1] is not cache:
                 # warm up outside capture (lazy module loads, attribute settings), then
                 # restore the positions the warm-up advanced
