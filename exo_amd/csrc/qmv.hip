@@ -90,6 +90,79 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
   }
 }
 
+// Two-phase staging for the row-streaming kernel (wpr == 256*ITERS, so every thread
+// owns exactly ITERS words per activation row): the global loads are issued first and
+// consumed after the first weight batches are in flight.
+template <int BITS, int MT, int ITERS>
+struct XStage {
+  uint4 r[MT][ITERS];  // 8-bit uses .x/.y only
+};
+
+template <int BITS, int MT, int ITERS>
+__device__ __forceinline__ void stage_x_load(const QmvParams& p, const bf16_t* x,
+                                             XStage<BITS, MT, ITERS>& st) {
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int wi = threadIdx.x + it * kThreads;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      st.r[m][it] = make_uint4(0, 0, 0, 0);
+      if (m < p.M) {
+        if (BITS == 4) {
+          st.r[m][it] = *reinterpret_cast<const uint4*>(x + (size_t)m * p.K + (size_t)wi * 8);
+        } else {
+          const uint2 v = *reinterpret_cast<const uint2*>(x + (size_t)m * p.K + (size_t)wi * 4);
+          st.r[m][it].x = v.x;
+          st.r[m][it].y = v.y;
+        }
+      }
+    }
+  }
+}
+
+template <int BITS, int MT, int ITERS>
+__device__ __forceinline__ void stage_x_store(const XStage<BITS, MT, ITERS>& st, uint4* xs,
+                                              float2* sx) {
+  constexpr int WPR = 256 * ITERS, CPR = 64 * ITERS;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int wi = threadIdx.x + it * kThreads;
+    const int c = wi >> 2, t = wi & 3;
+    const int j = c >> 6, sl = c & 63;
+    const int dst = (((j << 2) + t) << 6) + sl;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const uint4 xv = st.r[m][it];
+      uint4 o;
+      float stored, truesum;
+      if (BITS == 4) {
+        o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
+        o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
+        o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
+        o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
+        truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
+                  (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
+        stored = truesum;
+      } else {
+        const uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);   // (x0,x2)
+        const uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u);  // (x1,x3)
+        o.x = a;
+        o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
+        o.z = c2;
+        o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
+        truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
+        stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
+      }
+      xs[m * WPR + dst] = o;
+      stored += __shfl_xor(stored, 1, 64);
+      truesum += __shfl_xor(truesum, 1, 64);
+      stored += __shfl_xor(stored, 2, 64);
+      truesum += __shfl_xor(truesum, 2, 64);
+      if (t == 0) sx[m * CPR + c] = make_float2(128.f * stored, truesum);
+    }
+  }
+}
+
 template <int BITS>
 __device__ __forceinline__ void unpack_word(uint32_t w, uint32_t (&pr)[4]) {
   // nibble t and nibble t+4 of the word as (128+n_t, 128+n_{t+4}) in bf16
@@ -97,6 +170,15 @@ __device__ __forceinline__ void unpack_word(uint32_t w, uint32_t (&pr)[4]) {
   pr[1] = ((w >> 4) & 0x000F000Fu) | 0x43004300u;
   pr[2] = ((w >> 8) & 0x000F000Fu) | 0x43004300u;
   pr[3] = ((w >> 12) & 0x000F000Fu) | 0x43004300u;
+}
+// Same, with the mask and the exponent pattern held in registers (gfx9 VOP3 takes no
+// literals), so each pair is one v_and_or_b32.
+__device__ __forceinline__ void unpack_word_r(uint32_t w, uint32_t mask, uint32_t magic,
+                                              uint32_t (&pr)[4]) {
+  pr[0] = (w & mask) | magic;
+  pr[1] = ((w >> 4) & mask) | magic;
+  pr[2] = ((w >> 8) & mask) | magic;
+  pr[3] = ((w >> 12) & mask) | magic;
 }
 
 // NMAT == 2: the pair (gate, up) with the SwiGLU epilogue.
@@ -288,6 +370,205 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Fast path: rows long enough that 64 lanes x 16 B tile them exactly
+// (K*bits/128 = 64*ITERS chunks).  One row per wave instruction, so the flat unit
+// index u = row*ITERS + j addresses weights (u * 1 KiB), scales and biases
+// (u * 64>>GSHIFT elements) linearly: no per-unit address arithmetic beyond a scalar
+// add.  ITERS is a template parameter: the per-row loop, the LDS offsets of x and the
+// point where a row ends are all static.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+// sum over the wave; the total lands in lane 63
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_get<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+  v += dpp_get<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+  v += dpp_get<0x141, 0xf>(v);  // row_half_mirror
+  v += dpp_get<0x140, 0xf>(v);  // row_mirror: every lane holds its row-of-16 total
+  v += dpp_get<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_get<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+template <int BITS, int MT, int NMAT, int ITERS>
+__global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
+  extern __shared__ uint4 smem[];
+  uint4* xs = smem;
+  float2* sx = reinterpret_cast<float2*>(smem + (size_t)MT * p.wpr);
+  constexpr int GSHIFT = (BITS == 4) ? 1 : 2;
+  constexpr int UG = 64 >> GSHIFT;  // scale elements per unit
+  constexpr int R0 = 8 / (ITERS * NMAT);
+  constexpr int R = R0 < 1 ? 1 : R0;  // rows per batch
+  constexpr int UB = R * ITERS;       // units per batch and matrix
+  constexpr int CPR = 64 * ITERS;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int G = p.K >> 6;
+
+  // balanced contiguous row range of this wave
+  const int nwaves = gridDim.x * kWaves;
+  const int gw = blockIdx.x * kWaves + wave;
+  const int base = p.N / nwaves, rem = p.N - base * nwaves;
+  const int r0 = gw * base + min(gw, rem);
+  const int r1 = r0 + base + (gw < rem ? 1 : 0);
+  const int nrows = r1 - r0;
+
+  const bf16_t* xin = p.x;
+  bf16_t* yout = p.y;
+  size_t ew = 0, eg = 0;
+  if (p.idx) {
+    const int pair = blockIdx.y;
+    int e = p.idx[pair];
+    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+    ew = (size_t)e * p.N * p.wpr;
+    eg = (size_t)e * p.N * G;
+    xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
+    yout += (size_t)pair * p.N;
+  }
+  const char* wb[NMAT];
+  const char* sb[NMAT];
+  const char* bb[NMAT];
+#pragma unroll
+  for (int a = 0; a < NMAT; ++a) {
+    wb[a] = reinterpret_cast<const char*>(p.w[a] + ew);
+    sb[a] = reinterpret_cast<const char*>(p.s[a] + eg);
+    bb[a] = reinterpret_cast<const char*>(p.b[a] + eg);
+  }
+  const uint32_t lw = lane * 16;               // byte offset of the lane inside a unit
+  const uint32_t ls = (lane >> GSHIFT) * 2;    // byte offset of the lane's scale
+
+  struct Batch {
+    uint4 w[NMAT][UB];
+    bf16_t s[NMAT][UB], b[NMAT][UB];
+  };
+
+  auto issue = [&](Batch& bt, int row_first) {
+#pragma unroll
+    for (int i = 0; i < UB; ++i) {
+      // rows past the end of the range re-read its last row (results are dropped)
+      const int row = min(row_first + i / ITERS, r1 - 1);
+      const uint32_t u = (uint32_t)row * ITERS + (i % ITERS);
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a) {
+        bt.w[a][i] = *reinterpret_cast<const uint4*>(wb[a] + (size_t)u * 1024 + lw);
+        bt.s[a][i] = *reinterpret_cast<const bf16_t*>(sb[a] + (size_t)u * (UG * 2) + ls);
+        bt.b[a][i] = *reinterpret_cast<const bf16_t*>(bb[a] + (size_t)u * (UG * 2) + ls);
+      }
+    }
+  };
+
+  // Short rows: the compiler keeps the (loop-invariant) activations in registers.
+  // Long rows: that would cost hundreds of VGPRs and the occupancy that hides HBM
+  // latency, so the LDS offset is made opaque per batch and x is re-read from LDS.
+  constexpr bool X_IN_REGS = ITERS * MT <= 2;
+  int xlane = lane;
+  uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
+  asm volatile("" : "+s"(kmask));
+  asm volatile("" : "+v"(kmagic));
+
+  auto compute = [&](const Batch& bt, int rb) {
+    if (!X_IN_REGS) asm volatile("" : "+v"(xlane));
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = rb + r;
+      if (row < r1) {
+        float acc[NMAT][MT];
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+          for (int m = 0; m < MT; ++m) acc[a][m] = 0.f;
+#pragma unroll
+        for (int j = 0; j < ITERS; ++j) {
+          const int i = r * ITERS + j;
+          // d starts at -128*Sx so the offset of the (128+q) trick needs no extra op
+          float2 sm[MT];
+          float d[NMAT][MT];
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            sm[m] = sx[m * CPR + j * 64 + xlane];
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) d[a][m] = -sm[m].x;
+          }
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            uint32_t pr[NMAT][4];
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a)
+              unpack_word_r(reinterpret_cast<const uint32_t*>(&bt.w[a][i])[t], kmask, kmagic, pr[a]);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+              const uint4 xv = xs[m * (4 * CPR) + (j * 4 + t) * 64 + xlane];
+#pragma unroll
+              for (int a = 0; a < NMAT; ++a) {
+                d[a][m] = dot2_bf16(pr[a][0], xv.x, d[a][m]);
+                d[a][m] = dot2_bf16(pr[a][1], xv.y, d[a][m]);
+                d[a][m] = dot2_bf16(pr[a][2], xv.z, d[a][m]);
+                d[a][m] = dot2_bf16(pr[a][3], xv.w, d[a][m]);
+              }
+            }
+          }
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) {
+              acc[a][m] = fmaf(bf2f(bt.s[a][i]), d[a][m], acc[a][m]);
+              acc[a][m] = fmaf(bf2f(bt.b[a][i]), sm[m].y, acc[a][m]);
+            }
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          float rsum[NMAT];
+#pragma unroll
+          for (int a = 0; a < NMAT; ++a) rsum[a] = wave_sum_to_lane63(acc[a][m]);
+          if (lane == 63 && m < p.M) {
+            const size_t o = (size_t)m * p.N + row;
+            float out;
+            if (NMAT == 2) {
+              const float g = bf2f(f2bf(rsum[0])), up = bf2f(f2bf(rsum[NMAT - 1]));
+              out = g / (1.f + __expf(-g)) * up;
+            } else {
+              out = rsum[0];
+              if (p.residual) out = bf2f(f2bf(out)) + bf2f(p.residual[o]);
+            }
+            yout[o] = f2bf(out);
+          }
+        }
+      }
+    }
+  };
+
+  // Order of the prologue: activations first (they sit in L2 and are waited for with
+  // the weight loads still outstanding), then two weight batches, then the LDS staging.
+  XStage<BITS, MT, ITERS> xst;
+  stage_x_load<BITS, MT, ITERS>(p, xin, xst);
+  Batch ba, bb2;
+  if (nrows > 0) issue(ba, r0);
+  if (nrows > R) issue(bb2, r0 + R);
+  stage_x_store<BITS, MT, ITERS>(xst, xs, sx);
+  __syncthreads();
+  if (nrows <= 0) return;
+
+  // two register buffers in ping-pong: two batches are in flight while one is consumed,
+  // without copying registers
+  int rb = r0;
+  for (;;) {
+    compute(ba, rb);
+    rb += R;
+    if (rb >= r1) break;
+    if (rb + R < r1) issue(ba, rb + R);
+    compute(bb2, rb);
+    rb += R;
+    if (rb >= r1) break;
+    if (rb + R < r1) issue(bb2, rb + R);
+  }
+}
+
 struct Plan {
   int lpr_log2, iters, slots, spw, grid, ragged;
   size_t lds;
@@ -319,8 +600,45 @@ bool make_plan(int N, int K, int bits, int mt, Plan* pl) {
   return true;
 }
 
+template <int BITS, int MT, int NMAT, int ITERS>
+int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
+  auto kern = qmv_rows_kernel<BITS, MT, NMAT, ITERS>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+      return EXO_ERR_HIP;
+    }
+    attr_done = true;
+  }
+  // waves get contiguous, balanced row ranges; aim at 4 workgroups per CU (LDS
+  // permitting) and at least 2 rows-batches of work per wave
+  int per_cu = pl.lds <= 36 * 1024 ? 4 : (pl.lds <= 72 * 1024 ? 2 : 1);
+  int grid = 256 * per_cu;
+  const int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
+  int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
+  if (grid > max_grid) grid = max_grid;
+  if (grid < 1) grid = 1;
+  kern<<<dim3(grid, pairs), dim3(kThreads), pl.lds, st>>>(p);
+  return EXO_OK;
+}
+
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
+  if (MT <= 2 && pl.lpr_log2 == 6 && !pl.ragged) {
+    constexpr int MTR = MT <= 2 ? MT : 1;  // (no instantiation for larger tiles)
+    switch (pl.iters) {
+      case 1: return launch_rows<BITS, MTR, NMAT, 1>(p, pl, pairs, st);
+      case 2: return launch_rows<BITS, MTR, NMAT, 2>(p, pl, pairs, st);
+      case 4: return launch_rows<BITS, MTR, NMAT, 4>(p, pl, pairs, st);
+      case 7: return launch_rows<BITS, MTR, NMAT, 7>(p, pl, pairs, st);
+      case 8: return launch_rows<BITS, MTR, NMAT, 8>(p, pl, pairs, st);
+      case 14: return launch_rows<BITS, MTR, NMAT, 14>(p, pl, pairs, st);
+      default: break;
+    }
+  }
   auto kern = qmv_kernel<BITS, MT, NMAT>;
   static bool attr_done = false;
   if (!attr_done) {
