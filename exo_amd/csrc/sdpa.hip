@@ -2,13 +2,15 @@
 //
 // One workgroup serves ONE kv head and all G = Hq/Hkv query heads that share it, so
 // every K/V byte read from HBM is used G times.  A key row (D bf16) is spread over
-// D/8 lanes, 16 bytes each; a wave covers 512/D keys per load instruction and keeps
-// four such loads of K and of V in flight.  Scores, softmax and the output
-// accumulation are float32 (online softmax, one rescale per block of 4 keys).
+// D/8 lanes, 16 bytes each; one load instruction of a wave reads 512/D consecutive
+// keys (1 KiB contiguous); two tiles of four such K and V loads are in flight per lane.
+// Scores, softmax and the output accumulation are float32 (online softmax, one
+// rescale per block of 4 keys).
 //
 // decode : grid (splits, Hkv, B); each split owns a contiguous key range, writes
-//          (max, sum, acc[D]) per query head to the workspace; a second kernel merges
-//          the splits.  The grid is fixed (positions are read on the device), so the
+//          (max, sum, acc[D]) per query head to the workspace; the last workgroup of a
+//          (sequence, kv head) to arrive - an atomic counter, no spinning - merges the
+//          splits.  The grid is fixed (positions are read on the device), so the
 //          launch can be replayed from a HIP graph while the sequence grows.
 // prefill: grid (T, Hkv, B); one workgroup per new token, causal limit pos+t+1,
 //          writes the output directly.
@@ -19,7 +21,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kMaxSplits = 64;
+constexpr int kMaxSplits = 16;
 constexpr int kBlk = 4;  // keys per lane group per step
 
 struct SdpaParams {
@@ -29,15 +31,25 @@ struct SdpaParams {
   const int32_t* pos;  // [B]
   bf16_t* out;         // [B*T, Hq*D]
   float* ws;           // decode partials
+  int* counters;       // decode: arrival counter per (sequence, kv head); zero between launches
   float scale;
   int B, T, Hq, Hkv, S_max, splits;
 };
 
+__device__ __forceinline__ void st_dev(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_dev(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int D, int G, bool DECODE>
 __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
-  constexpr int LPK = D / 8;     // lanes per key
-  constexpr int KPI = 64 / LPK;  // keys per wave instruction
+  constexpr int LPK = D / 8;        // lanes per key
+  constexpr int KPI = 64 / LPK;     // keys per wave instruction
+  constexpr int STEP = KPI * kBlk;  // keys per wave per step
   __shared__ float red[kWaves][G][D + 2];
+  __shared__ int s_last;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane / LPK, sl = lane % LPK;
@@ -47,10 +59,14 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   int k_begin = 0, k_end = len;
   if (DECODE) {
     int chunk = (len + p.splits - 1) / p.splits;
-    chunk = (chunk + 15) & ~15;
-    k_begin = min(blockIdx.x * chunk, len);
+    chunk = (chunk + STEP * kWaves - 1) / (STEP * kWaves) * (STEP * kWaves);
+    k_begin = min((int)blockIdx.x * chunk, len);
     k_end = min(k_begin + chunk, len);
   }
+  // each wave owns a contiguous quarter of the workgroup's range (multiple of STEP keys)
+  const int per_wave = ((k_end - k_begin + kWaves - 1) / kWaves + STEP - 1) / STEP * STEP;
+  const int w_begin = min(k_begin + wave * per_wave, k_end);
+  const int w_end = min(w_begin + per_wave, k_end);
 
   // q slices for the G heads: 8 elements = 4 bf16 pairs per head per lane
   uint4 qv[G];
@@ -72,39 +88,45 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   const bf16_t* kb = p.kc + head_base + sl * 8;
   const bf16_t* vb = p.vc + head_base + sl * 8;
 
-  // lane group (wave, sub) takes keys k_begin + (step*kWaves*KPI + wave*KPI + sub)*kBlk + i
-  for (int k0 = k_begin + (wave * KPI + sub) * kBlk; k0 < k_end; k0 += kWaves * KPI * kBlk) {
-    uint4 kk[kBlk], vv[kBlk];
+  struct Tile {
+    uint4 k[kBlk], v[kBlk];
+  };
+  // instruction i of a step reads KPI consecutive keys (KPI*D*2 contiguous bytes)
+  auto load = [&](Tile& tl, int k0) {
 #pragma unroll
     for (int i = 0; i < kBlk; ++i) {
-      const int key = min(k0 + i, k_end - 1);
-      kk[i] = *reinterpret_cast<const uint4*>(kb + (size_t)key * D);
-      vv[i] = *reinterpret_cast<const uint4*>(vb + (size_t)key * D);
+      const int key = min(k0 + i * KPI + sub, w_end - 1);
+      tl.k[i] = *reinterpret_cast<const uint4*>(kb + (size_t)key * D);
+      tl.v[i] = *reinterpret_cast<const uint4*>(vb + (size_t)key * D);
     }
+  };
+  auto consume = [&](const Tile& tl, int k0) {
     float s[G][kBlk];
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int i = 0; i < kBlk; ++i) {
-        float d = dot2_bf16(qv[g].x, kk[i].x, 0.f);
-        d = dot2_bf16(qv[g].y, kk[i].y, d);
-        d = dot2_bf16(qv[g].z, kk[i].z, d);
-        d = dot2_bf16(qv[g].w, kk[i].w, d);
+        float d = dot2_bf16(qv[g].x, tl.k[i].x, 0.f);
+        d = dot2_bf16(qv[g].y, tl.k[i].y, d);
+        d = dot2_bf16(qv[g].z, tl.k[i].z, d);
+        d = dot2_bf16(qv[g].w, tl.k[i].w, d);
 #pragma unroll
         for (int off = LPK >> 1; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
-        s[g][i] = (k0 + i < k_end) ? d * p.scale : -INFINITY;
+        s[g][i] = (k0 + i * KPI + sub < w_end) ? d * p.scale : -INFINITY;
       }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float bm = s[g][0];
 #pragma unroll
       for (int i = 1; i < kBlk; ++i) bm = fmaxf(bm, s[g][i]);
-      const float mn = fmaxf(m[g], bm);  // finite: key k0 is always valid
-      const float sc = __expf(m[g] - mn);
+      const float mn = fmaxf(m[g], bm);
+      // a lane group that has seen no valid key yet keeps (m=-inf, l=0, o=0)
+      const float base = (mn == -INFINITY) ? 0.f : mn;
+      const float sc = __expf(m[g] - base);
       float pr[kBlk], ps = 0.f;
 #pragma unroll
       for (int i = 0; i < kBlk; ++i) {
-        pr[i] = __expf(s[g][i] - mn);
+        pr[i] = __expf(s[g][i] - base);
         ps += pr[i];
       }
       l[g] = l[g] * sc + ps;
@@ -113,13 +135,29 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
       for (int e = 0; e < 8; ++e) o[g][e] *= sc;
 #pragma unroll
       for (int i = 0; i < kBlk; ++i) {
-        const uint32_t* v4 = reinterpret_cast<const uint32_t*>(&vv[i]);
+        const uint32_t* v4 = reinterpret_cast<const uint32_t*>(&tl.v[i]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           o[g][2 * e] = fmaf(pr[i], bf_lo(v4[e]), o[g][2 * e]);
           o[g][2 * e + 1] = fmaf(pr[i], bf_hi(v4[e]), o[g][2 * e + 1]);
         }
       }
+    }
+  };
+
+  if (w_begin < w_end) {
+    Tile ta, tb;
+    load(ta, w_begin);
+    int k0 = w_begin;
+    for (;;) {
+      if (k0 + STEP < w_end) load(tb, k0 + STEP);
+      consume(ta, k0);
+      k0 += STEP;
+      if (k0 >= w_end) break;
+      if (k0 + STEP < w_end) load(ta, k0 + STEP);
+      consume(tb, k0);
+      k0 += STEP;
+      if (k0 >= w_end) break;
     }
   }
 
@@ -167,33 +205,61 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     }
     const int h = kvh * G + g;
     if (DECODE) {
+      // device-scope (write-through) stores: the merging workgroup may run on another
+      // XCD, whose L2 is not coherent with this one
       float* dst = p.ws + ((size_t)(b * p.Hq + h) * p.splits + blockIdx.x) * (D + 2);
-      dst[e] = acc;
+      st_dev(dst + e, acc);
       if (e == 0) {
-        dst[D] = mw;
-        dst[D + 1] = lsum;
+        st_dev(dst + D, mw);
+        st_dev(dst + D + 1, lsum);
       }
     } else {
       p.out[qrow + (size_t)h * D + e] = f2bf(acc / lsum);
     }
   }
-}
+  if (!DECODE) return;
 
-template <int D>
-__global__ __launch_bounds__(D) void sdpa_merge_kernel(const float* __restrict__ ws,
-                                                       bf16_t* __restrict__ out, int splits) {
-  const int bh = blockIdx.x, e = threadIdx.x;
-  const float* src = ws + (size_t)bh * splits * (D + 2);
-  float mw = -INFINITY;
-  for (int s = 0; s < splits; ++s) mw = fmaxf(mw, src[(size_t)s * (D + 2) + D]);
-  float acc = 0.f, lsum = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float mm = src[(size_t)s * (D + 2) + D];
-    const float sc = (mm == -INFINITY) ? 0.f : __expf(mm - mw);
-    acc += src[(size_t)s * (D + 2) + e] * sc;
-    lsum += src[(size_t)s * (D + 2) + D + 1] * sc;
+  // The last workgroup of this (sequence, kv head) to finish merges the splits.  The
+  // counter returns to zero, so the launch can be replayed without re-initialising it.
+  // No device-wide fence (an L2 write-back on this chip): the partials were stored and
+  // are loaded at device scope, and the workgroup-scope release below only waits for
+  // this workgroup's stores to complete before the counter is bumped.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* cnt = &p.counters[b * p.Hkv + kvh];
+    const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == p.splits - 1);
+    if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  out[(size_t)bh * D + e] = f2bf(acc / lsum);
+  __syncthreads();
+  if (!s_last) return;
+  for (int idx = threadIdx.x; idx < G * D; idx += kThreads) {
+    const int g = idx / D, e = idx % D;
+    const int h = kvh * G + g;
+    const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
+    // all loads of all splits are issued before any is used (they miss every cache)
+    float pm[kMaxSplits], pl[kMaxSplits], po[kMaxSplits];
+#pragma unroll
+    for (int sp = 0; sp < kMaxSplits; ++sp) {
+      const int spc = min(sp, p.splits - 1);
+      pm[sp] = ld_dev(src + (size_t)spc * (D + 2) + D);
+      pl[sp] = ld_dev(src + (size_t)spc * (D + 2) + D + 1);
+      po[sp] = ld_dev(src + (size_t)spc * (D + 2) + e);
+    }
+    float mw = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < kMaxSplits; ++sp)
+      if (sp < p.splits) mw = fmaxf(mw, pm[sp]);
+    float acc = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < kMaxSplits; ++sp) {
+      const float sc = (sp >= p.splits || pm[sp] == -INFINITY) ? 0.f : __expf(pm[sp] - mw);
+      acc += po[sp] * sc;
+      lsum += pl[sp] * sc;
+    }
+    p.out[qrow + (size_t)h * D + e] = f2bf(acc / lsum);
+  }
 }
 
 int pick_splits(int B, int Hkv, int S_max) {
@@ -219,8 +285,6 @@ int launch_sdpa(const SdpaParams& p, hipStream_t st) {
       exo_set_error("sdpa: unsupported Hq/Hkv=%d (1,2,4,8,16)", G);
       return EXO_ERR_ARG;
   }
-  if (DECODE)
-    sdpa_merge_kernel<D><<<dim3(p.B * p.Hq), D, 0, st>>>(p.ws, p.out, p.splits);
   return EXO_OK;
 }
 
@@ -232,10 +296,15 @@ int check(const char* name, int B, int T, int Hq, int Hkv, int D, int S_max) {
   return EXO_OK;
 }
 
+// partials for kMaxSplits splits, then one int counter per (sequence, kv head)
+int64_t ws_partial_floats(int B, int Hq, int D) {
+  return (int64_t)B * Hq * kMaxSplits * (D + 2);
+}
+
 }  // namespace
 
 extern "C" int64_t exo_sdpa_decode_workspace(int B, int Hq, int D) {
-  return (int64_t)B * Hq * kMaxSplits * (D + 2) * (int64_t)sizeof(float);
+  return (ws_partial_floats(B, Hq, D) + (int64_t)B * Hq) * (int64_t)sizeof(float);
 }
 
 extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
@@ -246,8 +315,9 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out && workspace,
               "exo_sdpa_decode: null pointer");
-  SdpaParams p{q, k_cache, v_cache, pos, out, workspace, scale, B, 1, Hq, Hkv, S_max,
-               pick_splits(B, Hkv, S_max)};
+  SdpaParams p{q, k_cache, v_cache, pos, out, workspace,
+               reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
+               Hkv, S_max, pick_splits(B, Hkv, S_max)};
   rc = (D == 64) ? launch_sdpa<64, true>(p, (hipStream_t)stream)
                  : launch_sdpa<128, true>(p, (hipStream_t)stream);
   if (rc) return rc;
@@ -262,7 +332,7 @@ extern "C" int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache,
   int rc = check("exo_sdpa_prefill", B, T, Hq, Hkv, D, S_max);
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out, "exo_sdpa_prefill: null pointer");
-  SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, scale, B, T, Hq, Hkv, S_max, 1};
+  SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, nullptr, scale, B, T, Hq, Hkv, S_max, 1};
   rc = (D == 64) ? launch_sdpa<64, false>(p, (hipStream_t)stream)
                  : launch_sdpa<128, false>(p, (hipStream_t)stream);
   if (rc) return rc;

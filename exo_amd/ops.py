@@ -273,7 +273,7 @@ def rope_kv_append(qkv, q_out, k_cache, v_cache, pos, inv_freq, B, T, Hq, Hkv, D
 
 def sdpa_decode_workspace(B: int, Hq: int, D: int, device) -> torch.Tensor:
     n = native.load().exo_sdpa_decode_workspace(B, Hq, D)
-    return torch.empty(n // 4, dtype=torch.float32, device=device)
+    return torch.zeros(n // 4, dtype=torch.float32, device=device)  # counters start at 0
 
 
 def sdpa_decode(q, k_cache, v_cache, pos, out, workspace, scale, B, Hq, Hkv, D):

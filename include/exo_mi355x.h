@@ -114,7 +114,9 @@ int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
 
 /* K7 decode: scaled_dot_product_attention for one new token per sequence over the
  * cache, grouped-query: q bf16 [B, Hq*D]; lens int32 [B] = pos[b]+1 valid keys;
- * out bf16 [B, Hq*D].  `workspace` float, exo_sdpa_decode_workspace(B,Hq,D) bytes.
+ * out bf16 [B, Hq*D].  `workspace`: exo_sdpa_decode_workspace(B,Hq,D) bytes, zeroed ONCE
+ * by the caller before its first use (it ends with arrival counters that every launch
+ * leaves at zero); launches that share a workspace must not overlap.
  * (.typings/mlx_lm/models/base.pyi:39-47) */
 int64_t exo_sdpa_decode_workspace(int B, int Hq, int D);
 int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
