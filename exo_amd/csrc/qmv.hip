@@ -40,16 +40,76 @@ struct QmvParams {
   // gather (MoE) mode: blockIdx.y = (token, slot) pair; expert = idx[pair]
   const int32_t* idx;  // [T*topk] or null
   int E, topk, x_rows;
+  // fused RMSNorm of the input rows: x <- bf16(x * rsqrt(mean(x^2) + eps) * norm_w)
+  const bf16_t* norm_w;  // [K] or null
+  float eps;
 };
+
+// sum over the 256 threads of the workgroup, for MT values at once
+template <int MT>
+__device__ __forceinline__ void block_sum(float (&v)[MT], float* red /* [4*MT] */) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const float t = wave_sum(v[m]);
+    if (lane == 0) red[wave * MT + m] = t;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+    v[m] = red[m] + red[MT + m] + red[2 * MT + m] + red[3 * MT + m];
+  __syncthreads();
+}
+
+// 8 (4-bit layout) or 4 (8-bit layout) bf16 values of one word: v <- bf16(v * inv * w)
+template <int BITS>
+__device__ __forceinline__ void norm_word(uint4& xv, const uint4& wv, float inv) {
+  xv.x = pack_bf2(bf_lo(xv.x) * inv * bf_lo(wv.x), bf_hi(xv.x) * inv * bf_hi(wv.x));
+  xv.y = pack_bf2(bf_lo(xv.y) * inv * bf_lo(wv.y), bf_hi(xv.y) * inv * bf_hi(wv.y));
+  if (BITS == 4) {
+    xv.z = pack_bf2(bf_lo(xv.z) * inv * bf_lo(wv.z), bf_hi(xv.z) * inv * bf_hi(wv.z));
+    xv.w = pack_bf2(bf_lo(xv.w) * inv * bf_lo(wv.w), bf_hi(xv.w) * inv * bf_hi(wv.w));
+  }
+}
+template <int BITS>
+__device__ __forceinline__ float sumsq_word(const uint4& xv) {
+  float s = bf_lo(xv.x) * bf_lo(xv.x) + bf_hi(xv.x) * bf_hi(xv.x) +
+            bf_lo(xv.y) * bf_lo(xv.y) + bf_hi(xv.y) * bf_hi(xv.y);
+  if (BITS == 4)
+    s += bf_lo(xv.z) * bf_lo(xv.z) + bf_hi(xv.z) * bf_hi(xv.z) +
+         bf_lo(xv.w) * bf_lo(xv.w) + bf_hi(xv.w) * bf_hi(xv.w);
+  return s;
+}
+template <int BITS>
+__device__ __forceinline__ uint4 load_word_x(const bf16_t* base, int wi) {
+  if (BITS == 4) return *reinterpret_cast<const uint4*>(base + (size_t)wi * 8);
+  const uint2 v = *reinterpret_cast<const uint2*>(base + (size_t)wi * 4);
+  return make_uint4(v.x, v.y, 0, 0);
+}
 
 // Stage x (rows m0..m0+MT) into LDS in dot2 register order; compute chunk sums.
 // xs layout per m: uint4[(j*4 + t) * LPR + sl]  for chunk c = sl + j*LPR, word t.
 // sx layout per m: float2[c] = (128 * sum(stored), sum(x)).
 template <int BITS, int MT>
 __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uint4* xs,
-                                        float2* sx) {
+                                        float2* sx, float* red) {
   const int cpr = p.wpr >> 2;
   const int lpr_mask = (1 << p.lpr_log2) - 1;
+  float inv[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) inv[m] = 1.f;
+  if (p.norm_w) {
+    float ss[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) ss[m] = 0.f;
+    for (int wi = threadIdx.x; wi < p.wpr; wi += kThreads)
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        if (m < p.M) ss[m] += sumsq_word<BITS>(load_word_x<BITS>(x + (size_t)m * p.K, wi));
+    block_sum<MT>(ss, red);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) inv[m] = rsqrtf(ss[m] / (float)p.K + p.eps);
+  }
   for (int wi = threadIdx.x; wi < p.wpr; wi += kThreads) {
     const int c = wi >> 2, t = wi & 3;
     const int j = c >> p.lpr_log2, sl = c & lpr_mask;
@@ -59,8 +119,9 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
       uint4 o = make_uint4(0, 0, 0, 0);
       float stored = 0.f, truesum = 0.f;
       if (m < p.M) {
+        uint4 xv = load_word_x<BITS>(x + (size_t)m * p.K, wi);
+        if (p.norm_w) norm_word<BITS>(xv, load_word_x<BITS>(p.norm_w, wi), inv[m]);
         if (BITS == 4) {
-          uint4 xv = *reinterpret_cast<const uint4*>(x + (size_t)m * p.K + (size_t)wi * 8);
           o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
           o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
           o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
@@ -69,7 +130,6 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
                     (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
           stored = truesum;
         } else {
-          uint2 xv = *reinterpret_cast<const uint2*>(x + (size_t)m * p.K + (size_t)wi * 4);
           uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);  // (x0,x2)
           uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u); // (x1,x3)
           o.x = a;
@@ -96,6 +156,7 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
 template <int BITS, int MT, int ITERS>
 struct XStage {
   uint4 r[MT][ITERS];  // 8-bit uses .x/.y only
+  uint4 nw[ITERS];     // norm weights of the same words (when fused)
 };
 
 template <int BITS, int MT, int ITERS>
@@ -107,23 +168,32 @@ __device__ __forceinline__ void stage_x_load(const QmvParams& p, const bf16_t* x
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       st.r[m][it] = make_uint4(0, 0, 0, 0);
-      if (m < p.M) {
-        if (BITS == 4) {
-          st.r[m][it] = *reinterpret_cast<const uint4*>(x + (size_t)m * p.K + (size_t)wi * 8);
-        } else {
-          const uint2 v = *reinterpret_cast<const uint2*>(x + (size_t)m * p.K + (size_t)wi * 4);
-          st.r[m][it].x = v.x;
-          st.r[m][it].y = v.y;
-        }
-      }
+      if (m < p.M) st.r[m][it] = load_word_x<BITS>(x + (size_t)m * p.K, wi);
     }
+    if (p.norm_w) st.nw[it] = load_word_x<BITS>(p.norm_w, wi);
   }
 }
 
 template <int BITS, int MT, int ITERS>
-__device__ __forceinline__ void stage_x_store(const XStage<BITS, MT, ITERS>& st, uint4* xs,
-                                              float2* sx) {
+__device__ __forceinline__ void stage_x_store(const QmvParams& p, XStage<BITS, MT, ITERS>& st,
+                                              uint4* xs, float2* sx, float* red) {
   constexpr int WPR = 256 * ITERS, CPR = 64 * ITERS;
+  if (p.norm_w) {
+    float ss[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      ss[m] = 0.f;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) ss[m] += sumsq_word<BITS>(st.r[m][it]);
+    }
+    block_sum<MT>(ss, red);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const float inv = rsqrtf(ss[m] / (float)p.K + p.eps);
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) norm_word<BITS>(st.r[m][it], st.nw[it], inv);
+    }
+  }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int wi = threadIdx.x + it * kThreads;
@@ -269,7 +339,8 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   };
 
   if (total > 0) issue(0);
-  stage_x<BITS, MT>(p, xin, xs, sx);
+  __shared__ float s_red[4 * MT];
+  stage_x<BITS, MT>(p, xin, xs, sx, s_red);
   __syncthreads();
   if (total <= 0) return;
 
@@ -550,7 +621,8 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   Batch ba, bb2;
   if (nrows > 0) issue(ba, r0);
   if (nrows > R) issue(bb2, r0 + R);
-  stage_x_store<BITS, MT, ITERS>(xst, xs, sx);
+  __shared__ float s_red[4 * MT];
+  stage_x_store<BITS, MT, ITERS>(p, xst, xs, sx, s_red);
   __syncthreads();
   if (nrows <= 0) return;
 
@@ -606,7 +678,7 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
     if (e != hipSuccess) {
       exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
       return EXO_ERR_HIP;
@@ -643,7 +715,7 @@ int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
     if (e != hipSuccess) {
       exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
       return EXO_ERR_HIP;
@@ -663,7 +735,7 @@ template <int NMAT>
 int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const* s,
                  const bf16_t* const* b, const bf16_t* residual, bf16_t* y, int M, int N,
                  int K, int bits, hipStream_t st, const char* name,
-                 const Gather& ga = Gather()) {
+                 const Gather& ga = Gather(), const bf16_t* norm_w = nullptr, float eps = 0.f) {
   // M is processed in tiles of at most 4 rows (bounded by LDS: the whole K of every
   // row of the tile is resident); each tile re-streams W.
   int m0 = 0;
@@ -705,6 +777,8 @@ int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const*
     p.E = ga.E;
     p.topk = ga.topk;
     p.x_rows = ga.x_rows;
+    p.norm_w = norm_w;
+    p.eps = eps;
     const int pairs = ga.idx ? ga.pairs : 1;
     int rc;
     if (bits == 4) {
@@ -745,6 +819,14 @@ int check_common(const char* name, int M, int N, int K, int bits, int group_size
 extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M,
                        int N, int K, int bits, int group_size, exo_stream_t stream) {
+  return exo_norm_qmv(x, nullptr, 0.f, w, scales, biases, residual, y, M, N, K, bits, group_size,
+                      stream);
+}
+
+extern "C" int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                            const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* residual, uint16_t* y, int M, int N, int K,
+                            int bits, int group_size, exo_stream_t stream) {
   int rc = check_common("exo_qmv", M, N, K, bits, group_size);
   if (rc) return rc;
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmv: null pointer");
@@ -753,7 +835,7 @@ extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* sca
   const bf16_t* ss[1] = {scales};
   const bf16_t* bs[1] = {biases};
   rc = qmv_dispatch<1>(x, ws, ss, bs, residual, y, M, N, K, bits, (hipStream_t)stream,
-                       "exo_qmv");
+                       "exo_qmv", Gather(), norm_weight, eps);
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_qmv");
   return EXO_OK;
@@ -763,6 +845,15 @@ extern "C" int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint1
                               const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
                               const uint16_t* bu, uint16_t* y, int M, int N, int K, int bits,
                               int group_size, exo_stream_t stream) {
+  return exo_norm_qmv_swiglu(x, nullptr, 0.f, wg, sg, bg, wu, su, bu, y, M, N, K, bits,
+                             group_size, stream);
+}
+
+extern "C" int exo_norm_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                                   const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                                   const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
+                                   uint16_t* y, int M, int N, int K, int bits, int group_size,
+                                   exo_stream_t stream) {
   int rc = check_common("exo_qmv_swiglu", M, N, K, bits, group_size);
   if (rc) return rc;
   EXO_REQUIRE(x && wg && sg && bg && wu && su && bu && y, "exo_qmv_swiglu: null pointer");
@@ -771,7 +862,7 @@ extern "C" int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint1
   const bf16_t* ss[2] = {sg, su};
   const bf16_t* bs[2] = {bg, bu};
   rc = qmv_dispatch<2>(x, ws, ss, bs, nullptr, y, M, N, K, bits, (hipStream_t)stream,
-                       "exo_qmv_swiglu");
+                       "exo_qmv_swiglu", Gather(), norm_weight, eps);
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_qmv_swiglu");
   return EXO_OK;

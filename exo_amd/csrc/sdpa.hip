@@ -34,6 +34,12 @@ struct SdpaParams {
   int* counters;       // decode: arrival counter per (sequence, kv head); zero between launches
   float scale;
   int B, T, Hq, Hkv, S_max, splits;
+  // fused decode (q/k RoPE, optional head RMSNorm and the cache append done here)
+  const bf16_t* qkv;        // [B, (Hq+2*Hkv)*D]
+  const float* inv_freq;    // [D/2]
+  const bf16_t* qn;         // [D] or null
+  const bf16_t* kn;
+  float eps;
 };
 
 __device__ __forceinline__ void st_dev(float* p, float v) {
@@ -43,8 +49,53 @@ __device__ __forceinline__ float ld_dev(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int D, int G, bool DECODE>
+// One head slice (8 elements of this lane, the head spread over LPK lanes) taken from a
+// fused qkv row: optional per-head RMSNorm (rounded to bf16 like a separate rms_norm),
+// then rotate-half RoPE with the lane's 8 (cos, sin) pairs, rounded to bf16.
+template <int D, bool ROPE>
+__device__ __forceinline__ uint4 head_slice(const bf16_t* src, int sl, const bf16_t* nw,
+                                            float eps, const float (&cs)[8], const float (&sn)[8]) {
+  constexpr int LPK = D / 8;
+  const uint4 raw = *reinterpret_cast<const uint4*>(src + sl * 8);
+  if (!ROPE) return raw;
+  const uint32_t* r4 = reinterpret_cast<const uint32_t*>(&raw);
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = bf_lo(r4[e]);
+    x[2 * e + 1] = bf_hi(r4[e]);
+  }
+  if (nw) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+#pragma unroll
+    for (int off = LPK >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float inv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = bf2f(f2bf(x[e] * inv * bf2f(nw[sl * 8 + e])));
+  }
+  const bool first = sl < LPK / 2;  // this lane holds elements of the first half
+  uint4 out;
+  uint32_t* o4 = reinterpret_cast<uint32_t*>(&out);
+  float y[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float other = __shfl_xor(x[e], LPK / 2, 64);
+    // first half: x1*c - x2*s ; second half: x2*c + x1*s
+    y[e] = first ? (x[e] * cs[e] - other * sn[e]) : (x[e] * cs[e] + other * sn[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o4[e] = pack_bf2(y[2 * e], y[2 * e + 1]);
+  return out;
+}
+
+// MODE 0: prefill (one workgroup per new token); 1: decode over a cache that already
+// holds the new token; 2: decode fused with RoPE / head norm / cache append.
+template <int D, int G, int MODE>
 __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
+  constexpr bool DECODE = MODE != 0;
+  constexpr bool FUSED = MODE == 2;
   constexpr int LPK = D / 8;        // lanes per key
   constexpr int KPI = 64 / LPK;     // keys per wave instruction
   constexpr int STEP = KPI * kBlk;  // keys per wave per step
@@ -57,11 +108,17 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   const int t = DECODE ? 0 : blockIdx.x;
   const int len = min(p.pos[b] + t + 1, p.S_max);  // keys visible to this query
   int k_begin = 0, k_end = len;
+  bool own_new = false;  // fused: this workgroup handles the new token's key/value
   if (DECODE) {
     int chunk = (len + p.splits - 1) / p.splits;
     chunk = (chunk + STEP * kWaves - 1) / (STEP * kWaves) * (STEP * kWaves);
     k_begin = min((int)blockIdx.x * chunk, len);
     k_end = min(k_begin + chunk, len);
+    if (FUSED) {  // the cache holds keys [0, len-1); key len-1 comes from the qkv row
+      own_new = (len - 1) / chunk == (int)blockIdx.x;
+      k_begin = min(k_begin, len - 1);
+      k_end = min(k_end, len - 1);
+    }
   }
   // each wave owns a contiguous quarter of the workgroup's range (multiple of STEP keys)
   const int per_wave = ((k_end - k_begin + kWaves - 1) / kWaves + STEP - 1) / STEP * STEP;
@@ -70,10 +127,26 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
 
   // q slices for the G heads: 8 elements = 4 bf16 pairs per head per lane
   uint4 qv[G];
+  uint4 knew = make_uint4(0, 0, 0, 0), vnew = make_uint4(0, 0, 0, 0);
   const size_t qrow = (size_t)(b * p.T + t) * p.Hq * D;
+  if (FUSED) {
+    float cs[8], sn[8];
+    const float fpos = (float)(len - 1);
 #pragma unroll
-  for (int g = 0; g < G; ++g)
-    qv[g] = *reinterpret_cast<const uint4*>(p.q + qrow + (size_t)(kvh * G + g) * D + sl * 8);
+    for (int e = 0; e < 8; ++e) sincosf(fpos * p.inv_freq[(sl * 8 + e) % (D / 2)], &sn[e], &cs[e]);
+    const bf16_t* row = p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+      qv[g] = head_slice<D, true>(row + (size_t)(kvh * G + g) * D, sl, p.qn, p.eps, cs, sn);
+    if (own_new && wave == 0) {
+      knew = head_slice<D, true>(row + (size_t)(p.Hq + kvh) * D, sl, p.kn, p.eps, cs, sn);
+      vnew = head_slice<D, false>(row + (size_t)(p.Hq + p.Hkv + kvh) * D, sl, nullptr, 0.f, cs, sn);
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+      qv[g] = *reinterpret_cast<const uint4*>(p.q + qrow + (size_t)(kvh * G + g) * D + sl * 8);
+  }
 
   float m[G], l[G], o[G][8];
 #pragma unroll
@@ -100,7 +173,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
       tl.v[i] = *reinterpret_cast<const uint4*>(vb + (size_t)key * D);
     }
   };
-  auto consume = [&](const Tile& tl, int k0) {
+  auto consume = [&](const Tile& tl, int k0, int limit) {
     float s[G][kBlk];
 #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -112,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
         d = dot2_bf16(qv[g].w, tl.k[i].w, d);
 #pragma unroll
         for (int off = LPK >> 1; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
-        s[g][i] = (k0 + i * KPI + sub < w_end) ? d * p.scale : -INFINITY;
+        s[g][i] = (k0 + i * KPI + sub < limit) ? d * p.scale : -INFINITY;
       }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -151,13 +224,29 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     int k0 = w_begin;
     for (;;) {
       if (k0 + STEP < w_end) load(tb, k0 + STEP);
-      consume(ta, k0);
+      consume(ta, k0, w_end);
       k0 += STEP;
       if (k0 >= w_end) break;
       if (k0 + STEP < w_end) load(ta, k0 + STEP);
-      consume(tb, k0);
+      consume(tb, k0, w_end);
       k0 += STEP;
       if (k0 >= w_end) break;
+    }
+  }
+  if (FUSED && own_new && wave == 0) {
+    // the new token: key/value straight from registers (only lane group 0, slot 0 is
+    // valid), and appended to the cache for the following steps
+    Tile tn;
+#pragma unroll
+    for (int i = 0; i < kBlk; ++i) {
+      tn.k[i] = i == 0 ? knew : make_uint4(0, 0, 0, 0);
+      tn.v[i] = i == 0 ? vnew : make_uint4(0, 0, 0, 0);
+    }
+    consume(tn, len - 1, len);
+    if (sub == 0) {
+      const size_t o = head_base + (size_t)(len - 1) * D + sl * 8;
+      *reinterpret_cast<uint4*>(const_cast<bf16_t*>(p.kc) + o) = knew;
+      *reinterpret_cast<uint4*>(const_cast<bf16_t*>(p.vc) + o) = vnew;
     }
   }
 
@@ -271,16 +360,16 @@ int pick_splits(int B, int Hkv, int S_max) {
   return s;
 }
 
-template <int D, bool DECODE>
+template <int D, int MODE>
 int launch_sdpa(const SdpaParams& p, hipStream_t st) {
   const int G = p.Hq / p.Hkv;
-  dim3 grid(DECODE ? p.splits : p.T, p.Hkv, p.B);
+  dim3 grid(MODE != 0 ? p.splits : p.T, p.Hkv, p.B);
   switch (G) {
-    case 1: sdpa_kernel<D, 1, DECODE><<<grid, kThreads, 0, st>>>(p); break;
-    case 2: sdpa_kernel<D, 2, DECODE><<<grid, kThreads, 0, st>>>(p); break;
-    case 4: sdpa_kernel<D, 4, DECODE><<<grid, kThreads, 0, st>>>(p); break;
-    case 8: sdpa_kernel<D, 8, DECODE><<<grid, kThreads, 0, st>>>(p); break;
-    case 16: sdpa_kernel<D, 16, DECODE><<<grid, kThreads, 0, st>>>(p); break;
+    case 1: sdpa_kernel<D, 1, MODE><<<grid, kThreads, 0, st>>>(p); break;
+    case 2: sdpa_kernel<D, 2, MODE><<<grid, kThreads, 0, st>>>(p); break;
+    case 4: sdpa_kernel<D, 4, MODE><<<grid, kThreads, 0, st>>>(p); break;
+    case 8: sdpa_kernel<D, 8, MODE><<<grid, kThreads, 0, st>>>(p); break;
+    case 16: sdpa_kernel<D, 16, MODE><<<grid, kThreads, 0, st>>>(p); break;
     default:
       exo_set_error("sdpa: unsupported Hq/Hkv=%d (1,2,4,8,16)", G);
       return EXO_ERR_ARG;
@@ -317,11 +406,30 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
               "exo_sdpa_decode: null pointer");
   SdpaParams p{q, k_cache, v_cache, pos, out, workspace,
                reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
-               Hkv, S_max, pick_splits(B, Hkv, S_max)};
-  rc = (D == 64) ? launch_sdpa<64, true>(p, (hipStream_t)stream)
-                 : launch_sdpa<128, true>(p, (hipStream_t)stream);
+               Hkv, S_max, pick_splits(B, Hkv, S_max), nullptr, nullptr, nullptr, nullptr, 0.f};
+  rc = (D == 64) ? launch_sdpa<64, 1>(p, (hipStream_t)stream)
+                 : launch_sdpa<128, 1>(p, (hipStream_t)stream);
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_sdpa_decode");
+  return EXO_OK;
+}
+
+extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
+                               const int32_t* pos, const float* inv_freq,
+                               const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
+                               uint16_t* out, float* workspace, float scale, int B, int Hq,
+                               int Hkv, int D, int S_max, exo_stream_t stream) {
+  int rc = check("exo_attn_decode", B, 1, Hq, Hkv, D, S_max);
+  if (rc) return rc;
+  EXO_REQUIRE(qkv && k_cache && v_cache && pos && inv_freq && out && workspace,
+              "exo_attn_decode: null pointer");
+  SdpaParams p{nullptr, k_cache, v_cache, pos, out, workspace,
+               reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
+               Hkv, S_max, pick_splits(B, Hkv, S_max), qkv, inv_freq, q_norm_w, k_norm_w, eps};
+  rc = (D == 64) ? launch_sdpa<64, 2>(p, (hipStream_t)stream)
+                 : launch_sdpa<128, 2>(p, (hipStream_t)stream);
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_attn_decode");
   return EXO_OK;
 }
 
@@ -332,9 +440,10 @@ extern "C" int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache,
   int rc = check("exo_sdpa_prefill", B, T, Hq, Hkv, D, S_max);
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out, "exo_sdpa_prefill: null pointer");
-  SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, nullptr, scale, B, T, Hq, Hkv, S_max, 1};
-  rc = (D == 64) ? launch_sdpa<64, false>(p, (hipStream_t)stream)
-                 : launch_sdpa<128, false>(p, (hipStream_t)stream);
+  SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, nullptr, scale, B, T, Hq, Hkv, S_max, 1,
+               nullptr, nullptr, nullptr, nullptr, 0.f};
+  rc = (D == 64) ? launch_sdpa<64, 0>(p, (hipStream_t)stream)
+                 : launch_sdpa<128, 0>(p, (hipStream_t)stream);
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_sdpa_prefill");
   return EXO_OK;

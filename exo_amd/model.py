@@ -181,8 +181,9 @@ class ShardModel:
         c = self.cfg
         gemv = R <= GEMV_MAX_ROWS
         if not c.is_moe:
-            if gemv:
-                ops.qmv_swiglu(bf.n, L.gate, L.up, out=bf.act)
+            if gemv:  # post-attention norm fused into the gate/up GEMV
+                ops.qmv_swiglu(bf.h, L.gate, L.up, out=bf.act, norm_weight=L.post_norm,
+                               eps=c.rms_norm_eps)
             else:
                 if bf.gate is None:
                     bf.gate = torch.empty_like(bf.act)
@@ -213,29 +214,38 @@ class ShardModel:
         pos = cache.pos[rsl]
         if self.is_first:
             ops.embed(bf.tokens, self.embed_tokens, out=bf.h)
+        gemv = R <= GEMV_MAX_ROWS
         for li, L in enumerate(self.layers):
             kc, vc = cache.k[li][rsl], cache.v[li][rsl]
-            ops.rms_norm(bf.h, L.in_norm, c.rms_norm_eps, out=bf.n)
-            ops.quantized_matmul(bf.n, L.qkv, out=bf.qkv)
-            ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
-                               L.q_norm, L.k_norm, c.rms_norm_eps)
-            if T == 1:
-                ops.sdpa_decode(bf.q, kc, vc, pos, bf.attn, bf.sdpa_ws, self.scale, B, Hq, Hkv, D)
+            if gemv:  # input norm fused into the q|k|v GEMV
+                ops.quantized_matmul(bf.h, L.qkv, out=bf.qkv, norm_weight=L.in_norm,
+                                     eps=c.rms_norm_eps)
             else:
+                ops.rms_norm(bf.h, L.in_norm, c.rms_norm_eps, out=bf.n)
+                ops.quantized_matmul(bf.n, L.qkv, out=bf.qkv)
+            if T == 1:  # rope + append + attention in one launch
+                ops.attn_decode(bf.qkv, kc, vc, pos, self.inv_freq, bf.attn, bf.sdpa_ws, self.scale,
+                                B, Hq, Hkv, D, L.q_norm, L.k_norm, c.rms_norm_eps)
+            else:
+                ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
+                                   L.q_norm, L.k_norm, c.rms_norm_eps)
                 ops.sdpa_prefill(bf.q, kc, vc, pos, bf.attn, self.scale, B, T, Hq, Hkv, D)
             ops.quantized_matmul(bf.attn, L.o, residual=bf.h, out=bf.h)
-            ops.rms_norm(bf.h, L.post_norm, c.rms_norm_eps, out=bf.n)
+            if c.is_moe or not gemv:
+                ops.rms_norm(bf.h, L.post_norm, c.rms_norm_eps, out=bf.n)
             self._mlp(L, bf, R)
         if not self.is_last or logits_mode == "none":
             return bf.h
-        if logits_mode == "last" and T > 1:
-            hl = bf.h.view(B, T, -1)[:, -1].contiguous()
-            n = ops.rms_norm(hl, self.norm, c.rms_norm_eps)
+        hl = bf.h.view(B, T, -1)[:, -1].contiguous() if (logits_mode == "last" and T > 1) else bf.h
+        rows = hl.shape[0]
+        if bf.logits is None or bf.logits.shape[0] != rows:
+            bf.logits = torch.empty(rows, c.vocab_size, dtype=torch.bfloat16, device=self.device)
+        if rows <= GEMV_MAX_ROWS:  # final norm fused into the lm_head GEMV
+            ops.quantized_matmul(hl, self.lm_head, out=bf.logits, norm_weight=self.norm,
+                                 eps=c.rms_norm_eps)
         else:
-            n = ops.rms_norm(bf.h, self.norm, c.rms_norm_eps, out=bf.n)
-        if bf.logits is None or bf.logits.shape[0] != n.shape[0]:
-            bf.logits = torch.empty(n.shape[0], c.vocab_size, dtype=torch.bfloat16, device=self.device)
-        ops.quantized_matmul(n, self.lm_head, out=bf.logits)
+            n = ops.rms_norm(hl, self.norm, c.rms_norm_eps)
+            ops.quantized_matmul(n, self.lm_head, out=bf.logits)
         return bf.logits
 
     def __call__(self, tokens: torch.Tensor | None, cache: ShardKVCache,

@@ -26,6 +26,8 @@ SIGNATURES: dict[str, tuple] = {
     "exo_embed_dequant": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "exo_qmv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "exo_qmv_swiglu": (_i, [_vp] * 8 + [_i, _i, _i, _i, _i, _vp]),
+    "exo_norm_qmv": (_i, [_vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "exo_norm_qmv_swiglu": (_i, [_vp, _vp, _f] + [_vp] * 7 + [_i, _i, _i, _i, _i, _vp]),
     "exo_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "exo_gather_qmv": (_i, [_vp] * 6 + [_i] * 8 + [_vp]),
     "exo_gather_qmv_swiglu": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
@@ -33,6 +35,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_rope_kv_append": (_i, [_vp] * 8 + [_f] + [_i] * 6 + [_vp]),
     "exo_sdpa_decode_workspace": (_i64, [_i, _i, _i]),
     "exo_sdpa_decode": (_i, [_vp] * 6 + [_f] + [_i] * 5 + [_vp]),
+    "exo_attn_decode": (_i, [_vp] * 7 + [_f, _vp, _vp, _f] + [_i] * 5 + [_vp]),
     "exo_sdpa_prefill": (_i, [_vp] * 5 + [_f] + [_i] * 6 + [_vp]),
     "exo_swiglu": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "exo_router_topk": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),

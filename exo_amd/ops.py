@@ -135,10 +135,13 @@ def quantized_matmul(
     qw: QuantizedWeight,
     residual: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
+    norm_weight: torch.Tensor | None = None,
+    eps: float = 0.0,
 ) -> torch.Tensor:
     """mx.quantized_matmul(x, w, scales, biases, transpose=True): x bf16 [M,K] ->
     bf16 [M,N].  M <= 16 runs the fused dequant-GEMV, larger M the MFMA GEMM.
-    ``residual`` (bf16 [M,N]) fuses the block's ``h + r``."""
+    ``residual`` (bf16 [M,N]) fuses the block's ``h + r``; ``norm_weight`` (M <= 16
+    only) fuses a preceding rms_norm(x, norm_weight, eps)."""
     lib = native.load()
     assert x.dtype == torch.bfloat16 and x.dim() == 2
     M, K = x.shape
@@ -146,6 +149,18 @@ def quantized_matmul(
         raise ValueError(f"quantized_matmul: x has K={K}, weight has K={qw.K}")
     if out is None:
         out = torch.empty(M, qw.N, dtype=torch.bfloat16, device=x.device)
+    if norm_weight is not None:
+        if M > QMV_MAX_M:
+            raise ValueError("fused rms_norm is only available on the GEMV path (M <= 16)")
+        check(
+            lib.exo_norm_qmv(
+                _ptr(x), _ptr(norm_weight), eps, _ptr(qw.weight), _ptr(qw.scales),
+                _ptr(qw.biases), _ptr(residual), _ptr(out), M, qw.N, K, qw.bits, qw.group_size,
+                _stream(),
+            ),
+            "quantized_matmul(norm)",
+        )
+        return out
     fn = lib.exo_qmv if M <= QMV_MAX_M else lib.exo_qmm
     check(
         fn(
@@ -173,16 +188,17 @@ def qmm(x, qw: QuantizedWeight, residual=None, out=None) -> torch.Tensor:
     return out
 
 
-def qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None) -> torch.Tensor:
-    """silu(x @ gate^T) * (x @ up^T) for M <= 16."""
+def qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None, norm_weight=None,
+               eps: float = 0.0) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) for M <= 16, optionally on rms_norm(x)."""
     lib = native.load()
     M, K = x.shape
     assert gate.N == up.N and gate.K == up.K == K and gate.bits == up.bits
     if out is None:
         out = torch.empty(M, gate.N, dtype=torch.bfloat16, device=x.device)
     check(
-        lib.exo_qmv_swiglu(
-            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+        lib.exo_norm_qmv_swiglu(
+            _ptr(x), _ptr(norm_weight), eps, _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
             _ptr(up.scales), _ptr(up.biases), _ptr(out), M, gate.N, K, gate.bits,
             gate.group_size, _stream(),
         ),
@@ -284,6 +300,20 @@ def sdpa_decode(q, k_cache, v_cache, pos, out, workspace, scale, B, Hq, Hkv, D):
             B, Hq, Hkv, D, k_cache.shape[2], _stream(),
         ),
         "sdpa_decode",
+    )
+
+
+def attn_decode(qkv, k_cache, v_cache, pos, inv_freq, out, workspace, scale, B, Hq, Hkv, D,
+                q_norm_w=None, k_norm_w=None, eps: float = 0.0):
+    """rope (+ head norm) + cache append + attention for one new token per sequence."""
+    lib = native.load()
+    check(
+        lib.exo_attn_decode(
+            _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), _ptr(q_norm_w),
+            _ptr(k_norm_w), eps, _ptr(out), _ptr(workspace), scale, B, Hq, Hkv, D,
+            k_cache.shape[2], _stream(),
+        ),
+        "attn_decode",
     )
 
 

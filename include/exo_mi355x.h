@@ -64,6 +64,19 @@ int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
                    const uint16_t* bu, uint16_t* y, int M, int N, int K, int bits,
                    int group_size, exo_stream_t stream);
 
+/* K5+K1 fused: the same two operators with mx.fast.rms_norm applied to the input rows
+ * on the fly (no separate pass over HBM): x <- bf16(x * rsqrt(mean(x^2)+eps) * norm_weight),
+ * norm_weight bf16 [K]; null norm_weight = no normalisation.  This is how a transformer
+ * block's `proj(norm(h))` runs in decode.  (rms_norm + nn.QuantizedLinear.__call__) */
+int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps, const uint32_t* w,
+                 const uint16_t* scales, const uint16_t* biases, const uint16_t* residual,
+                 uint16_t* y, int M, int N, int K, int bits, int group_size,
+                 exo_stream_t stream);
+int exo_norm_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                        const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                        const uint32_t* wu, const uint16_t* su, const uint16_t* bu, uint16_t* y,
+                        int M, int N, int K, int bits, int group_size, exo_stream_t stream);
+
 /* K2: the same operator for any M (prefill): weights are dequantised to bf16 in
  * LDS and multiplied on the matrix cores, float32 accumulation, bf16 out. */
 int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
@@ -122,6 +135,17 @@ int64_t exo_sdpa_decode_workspace(int B, int Hq, int D);
 int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
                     const int32_t* pos, uint16_t* out, float* workspace, float scale, int B,
                     int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
+
+/* K6+K10+K7 fused for decode: one launch per layer does what exo_rope_kv_append followed
+ * by exo_sdpa_decode do for T == 1: q and k heads of the fused qkv row [B,(Hq+2Hkv)*D] are
+ * (head-normalised and) rotated at position pos[b], the new k,v are appended to the
+ * cache at pos[b], and attention runs over pos[b]+1 keys.  Same workspace contract as
+ * exo_sdpa_decode.  No separate reference operator: it is rope + update_and_fetch +
+ * scaled_dot_product_attention of one attention block. */
+int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
+                    const int32_t* pos, const float* inv_freq, const uint16_t* q_norm_w,
+                    const uint16_t* k_norm_w, float eps, uint16_t* out, float* workspace,
+                    float scale, int B, int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
 
 /* K7 prefill: causal attention of T new tokens per sequence (already appended to the
  * cache) over pos[b]+T keys.  q bf16 [B*T, Hq*D] -> out same shape. */

@@ -302,3 +302,57 @@ def test_argmax_logsumexp(device, V):
     np.testing.assert_allclose(lse.cpu().numpy(), want_lse, rtol=1e-5)
     np.testing.assert_allclose(lp.cpu().numpy(), logits.max(-1) - want_lse, rtol=1e-4, atol=1e-5)
     assert pos.cpu().tolist() == [5, 6, 7]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("N,K,M", [(256, 4096, 1), (128, 14336, 2), (96, 768, 1), (64, 2048, 4), (72, 192, 3)])
+def test_norm_qmv_fused(device, bits, N, K, M):
+    trip = rand_quantized(N, K, bits, seed=N + K)
+    x = rand_bf16((M, K), seed=K + M, scale=3.0)
+    w = affine.bf16_round(rand_bf16((K,), seed=5) * 0.1 + 1.0)
+    got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device), norm_weight=t_bf16(w, device), eps=1e-5))
+    want = affine.qmm(O.rms_norm(x, w, 1e-5), *trip, 64, bits)
+    assert_close(got, want, what="norm+qmv")
+    g = rand_quantized(N, K, bits, seed=N + K + 1)
+    got = n_f32(ops.qmv_swiglu(t_bf16(x, device), t_qw(trip, bits, device), t_qw(g, bits, device), norm_weight=t_bf16(w, device), eps=1e-5))
+    xn = O.rms_norm(x, w, 1e-5)
+    assert_close(got, O.swiglu(affine.qmm(xn, *trip, 64, bits), affine.qmm(xn, *g, 64, bits)), what="norm+qmv_swiglu")
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 64, 4), (128, 4, 4)])
+@pytest.mark.parametrize("qk_norm", [False, True])
+@pytest.mark.parametrize("lens", [[1, 2], [100, 37], [513, 1000]])
+def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens):
+    """rope + head norm + cache append + attention in one launch == the three oracle ops."""
+    B, S_max = len(lens), 1024
+    pos = np.array([n - 1 for n in lens], np.int32)
+    qkv = rand_bf16((B, (Hq + 2 * Hkv) * D), seed=D + Hq + lens[0])
+    k = rand_bf16((B, Hkv, S_max, D), seed=11)
+    v = rand_bf16((B, Hkv, S_max, D), seed=12)
+    inv = O.rope_inv_freq(D, 5e5, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                   "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
+    qn = affine.bf16_round(rand_bf16((D,), 3) * 0.1 + 1.0) if qk_norm else None
+    kn = affine.bf16_round(rand_bf16((D,), 4) * 0.1 + 1.0) if qk_norm else None
+    kc, vc = t_bf16(k, device), t_bf16(v, device)
+    out = torch.empty(B, Hq * D, dtype=torch.bfloat16, device=device)
+    ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+    for _ in range(2):  # twice: the arrival counters must be back at zero
+        ops.attn_decode(t_bf16(qkv, device), kc, vc, torch.from_numpy(pos).to(device),
+                        torch.from_numpy(inv).to(device), out, ws, D ** -0.5, B, Hq, Hkv, D,
+                        t_bf16(qn, device) if qk_norm else None, t_bf16(kn, device) if qk_norm else None, 1e-6)
+    x = qkv.reshape(B, 1, Hq + 2 * Hkv, D)
+    q, kk, vv = x[:, :, :Hq], x[:, :, Hq:Hq + Hkv], x[:, :, Hq + Hkv:]
+    if qk_norm:
+        q, kk = O.rms_norm(q, qn, 1e-6), O.rms_norm(kk, kn, 1e-6)
+    for b in range(B):
+        p = int(pos[b])
+        qr = O.rope(q[b:b + 1].transpose(0, 2, 1, 3), inv, p)
+        kr = O.rope(kk[b:b + 1].transpose(0, 2, 1, 3), inv, p)
+        kfull = np.concatenate([k[b:b + 1, :, :p], kr], axis=2)
+        vfull = np.concatenate([v[b:b + 1, :, :p], vv[b:b + 1].transpose(0, 2, 1, 3)], axis=2)
+        want = O.sdpa(qr, kfull, vfull, D ** -0.5, None)
+        assert_close(n_f32(out)[b].reshape(Hq, D), want[0, :, 0], what=f"attn_decode len {lens[b]}")
+        assert_close(n_f32(kc)[b, :, p], kr[0, :, 0], rtol=1e-2, what="appended k")
+        np.testing.assert_array_equal(n_f32(vc)[b, :, p], vv[b, 0])
+        np.testing.assert_array_equal(n_f32(kc)[b, :, p + 1:], k[b, :, p + 1:])  # nothing else touched
+        np.testing.assert_array_equal(n_f32(kc)[b, :, :p], k[b, :, :p])
