@@ -685,8 +685,8 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
     }
     attr_done = true;
   }
-  // waves get contiguous, balanced row ranges; aim at 4 workgroups per CU (LDS
-  // permitting) and at least 2 rows-batches of work per wave
+  // waves get contiguous, balanced row ranges; 4 workgroups per CU (LDS permitting) and
+  // at least one full batch of rows per wave
   int per_cu = pl.lds <= 36 * 1024 ? 4 : (pl.lds <= 72 * 1024 ? 2 : 1);
   int grid = 256 * per_cu;
   const int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
