@@ -62,16 +62,20 @@ def measure_kernels(model, torch, reps: int = 20):
     y_h = torch.empty(1, H, **bf)
     y_i = torch.empty(1, I, **bf)
     y_v = torch.empty(1, c.vocab_size, **bf)
+    def kernel_name(nmat, K):  # template arguments <bits, rows of x, matrices, 1 KiB units per row>
+        return "qmv_rows_kernel<%d,1,%d,%d>" % (c.bits, nmat, K * c.bits // 8 // 1024)
+
+    nw, eps = torch.ones(H, **bf), c.rms_norm_eps
     groups = {
-        "gate_up_swiglu": (lambda L: ops.qmv_swiglu(xh, L.gate, L.up, out=y_i),
-                           2 * qbytes(I, H, c.bits) + 2 * (H + I), "qmv_kernel<%d,1,2>" % c.bits),
-        "down": (lambda L: ops.quantized_matmul(xi, L.down, out=y_h),
-                 qbytes(H, I, c.bits) + 2 * (I + H), "qmv_kernel<%d,1,1>" % c.bits),
-        "qkv": (lambda L: ops.quantized_matmul(xh, L.qkv, out=y_qkv),
-                qbytes((Hq + 2 * Hkv) * D, H, c.bits) + 2 * (H + (Hq + 2 * Hkv) * D),
-                "qmv_kernel<%d,1,1>" % c.bits),
-        "o": (lambda L: ops.quantized_matmul(xa, L.o, out=y_h),
-              qbytes(H, Hq * D, c.bits) + 2 * (Hq * D + H), "qmv_kernel<%d,1,1>" % c.bits),
+        "norm_gate_up_swiglu": (lambda L: ops.qmv_swiglu(xh, L.gate, L.up, out=y_i, norm_weight=nw, eps=eps),
+                                2 * qbytes(I, H, c.bits) + 2 * (2 * H + I), kernel_name(2, H)),
+        "down_residual": (lambda L: ops.quantized_matmul(xi, L.down, residual=y_h, out=y_h),
+                          qbytes(H, I, c.bits) + 2 * (I + 2 * H), kernel_name(1, I)),
+        "norm_qkv": (lambda L: ops.quantized_matmul(xh, L.qkv, out=y_qkv, norm_weight=nw, eps=eps),
+                     qbytes((Hq + 2 * Hkv) * D, H, c.bits) + 2 * (2 * H + (Hq + 2 * Hkv) * D),
+                     kernel_name(1, H)),
+        "o_residual": (lambda L: ops.quantized_matmul(xa, L.o, residual=y_h, out=y_h),
+                       qbytes(H, Hq * D, c.bits) + 2 * (Hq * D + 2 * H), kernel_name(1, Hq * D)),
     }
     out = []
     for name, (fn, nbytes, kname) in groups.items():
@@ -104,7 +108,7 @@ def measure_kernels(model, torch, reps: int = 20):
     torch.cuda.synchronize()
     us = st.elapsed_time(en) * 1e3 / reps
     nbytes = qbytes(c.vocab_size, H, c.bits) + 2 * (H + c.vocab_size)
-    out.append(dict(name="lm_head", kernel="qmv_kernel<%d,1,1>" % c.bits, launches_per_token=1,
+    out.append(dict(name="lm_head", kernel=kernel_name(1, H), launches_per_token=1,
                     bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
     return out
 

@@ -37,10 +37,38 @@ struct SdpaParams {
   // fused decode (q/k RoPE, optional head RMSNorm and the cache append done here)
   const bf16_t* qkv;        // [B, (Hq+2*Hkv)*D]
   const float* inv_freq;    // [D/2]
+  const float2* rope_tab;   // [S_max, D/2] (cos, sin) per position, or null
   const bf16_t* qn;         // [D] or null
   const bf16_t* kn;
   float eps;
 };
+
+// Sum over the LPK lanes of a key's lane group.  16 lanes are one DPP row: four
+// full-rate VALU ops instead of four LDS-crossbar permutes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LPK>
+__device__ __forceinline__ float group_sum_lpk(float d) {
+  if (LPK == 16) {
+    d += dpp_f<0xB1>(d);   // quad_perm [1,0,3,2]
+    d += dpp_f<0x4E>(d);   // quad_perm [2,3,0,1]
+    d += dpp_f<0x141>(d);  // row_half_mirror
+    d += dpp_f<0x140>(d);  // row_mirror
+    return d;
+  }
+#pragma unroll
+  for (int off = LPK >> 1; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+  return d;
+}
+// value of the lane LPK/2 away inside the lane group (the RoPE partner)
+template <int LPK>
+__device__ __forceinline__ float partner_lpk(float v) {
+  if (LPK == 16) return dpp_f<0x128>(v);  // row_ror:8
+  return __shfl_xor(v, LPK / 2, 64);
+}
 
 __device__ __forceinline__ void st_dev(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -69,8 +97,7 @@ __device__ __forceinline__ uint4 head_slice(const bf16_t* src, int sl, const bf1
     float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
-#pragma unroll
-    for (int off = LPK >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    ss = group_sum_lpk<LPK>(ss);
     const float inv = rsqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = bf2f(f2bf(x[e] * inv * bf2f(nw[sl * 8 + e])));
@@ -81,7 +108,7 @@ __device__ __forceinline__ uint4 head_slice(const bf16_t* src, int sl, const bf1
   float y[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float other = __shfl_xor(x[e], LPK / 2, 64);
+    const float other = partner_lpk<LPK>(x[e]);
     // first half: x1*c - x2*s ; second half: x2*c + x1*s
     y[e] = first ? (x[e] * cs[e] - other * sn[e]) : (x[e] * cs[e] + other * sn[e]);
   }
@@ -125,15 +152,49 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   const int w_begin = min(k_begin + wave * per_wave, k_end);
   const int w_end = min(w_begin + per_wave, k_end);
 
+  const size_t head_base = ((size_t)b * p.Hkv + kvh) * p.S_max * D;
+  const bf16_t* kb = p.kc + head_base + sl * 8;
+  const bf16_t* vb = p.vc + head_base + sl * 8;
+
+  struct Tile {
+    uint4 k[kBlk], v[kBlk];
+  };
+  // instruction i of a step reads KPI consecutive keys (KPI*D*2 contiguous bytes)
+  auto load = [&](Tile& tl, int k0) {
+#pragma unroll
+    for (int i = 0; i < kBlk; ++i) {
+      const int key = min(k0 + i * KPI + sub, w_end - 1);
+      tl.k[i] = *reinterpret_cast<const uint4*>(kb + (size_t)key * D);
+      tl.v[i] = *reinterpret_cast<const uint4*>(vb + (size_t)key * D);
+    }
+  };
+  // the first K/V tile is requested before the q work so its latency overlaps it
+  Tile ta, tb;
+  if (w_begin < w_end) load(ta, w_begin);
+
   // q slices for the G heads: 8 elements = 4 bf16 pairs per head per lane
   uint4 qv[G];
   uint4 knew = make_uint4(0, 0, 0, 0), vnew = make_uint4(0, 0, 0, 0);
   const size_t qrow = (size_t)(b * p.T + t) * p.Hq * D;
   if (FUSED) {
     float cs[8], sn[8];
-    const float fpos = (float)(len - 1);
+    if (p.rope_tab) {  // 8 consecutive (cos, sin) pairs of this position: 64 bytes
+      const float4* tp = reinterpret_cast<const float4*>(
+          p.rope_tab + (size_t)(len - 1) * (D / 2) + (sl * 8) % (D / 2));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sincosf(fpos * p.inv_freq[(sl * 8 + e) % (D / 2)], &sn[e], &cs[e]);
+      for (int e = 0; e < 4; ++e) {
+        const float4 v = tp[e];
+        cs[2 * e] = v.x;
+        sn[2 * e] = v.y;
+        cs[2 * e + 1] = v.z;
+        sn[2 * e + 1] = v.w;
+      }
+    } else {
+      const float fpos = (float)(len - 1);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        sincosf(fpos * p.inv_freq[(sl * 8 + e) % (D / 2)], &sn[e], &cs[e]);
+    }
     const bf16_t* row = p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
 #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -157,22 +218,6 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
   }
 
-  const size_t head_base = ((size_t)b * p.Hkv + kvh) * p.S_max * D;
-  const bf16_t* kb = p.kc + head_base + sl * 8;
-  const bf16_t* vb = p.vc + head_base + sl * 8;
-
-  struct Tile {
-    uint4 k[kBlk], v[kBlk];
-  };
-  // instruction i of a step reads KPI consecutive keys (KPI*D*2 contiguous bytes)
-  auto load = [&](Tile& tl, int k0) {
-#pragma unroll
-    for (int i = 0; i < kBlk; ++i) {
-      const int key = min(k0 + i * KPI + sub, w_end - 1);
-      tl.k[i] = *reinterpret_cast<const uint4*>(kb + (size_t)key * D);
-      tl.v[i] = *reinterpret_cast<const uint4*>(vb + (size_t)key * D);
-    }
-  };
   auto consume = [&](const Tile& tl, int k0, int limit) {
     float s[G][kBlk];
 #pragma unroll
@@ -183,8 +228,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
         d = dot2_bf16(qv[g].y, tl.k[i].y, d);
         d = dot2_bf16(qv[g].z, tl.k[i].z, d);
         d = dot2_bf16(qv[g].w, tl.k[i].w, d);
-#pragma unroll
-        for (int off = LPK >> 1; off > 0; off >>= 1) d += __shfl_xor(d, off, 64);
+        d = group_sum_lpk<LPK>(d);
         s[g][i] = (k0 + i * KPI + sub < limit) ? d * p.scale : -INFINITY;
       }
 #pragma unroll
@@ -219,8 +263,6 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   };
 
   if (w_begin < w_end) {
-    Tile ta, tb;
-    load(ta, w_begin);
     int k0 = w_begin;
     for (;;) {
       if (k0 + STEP < w_end) load(tb, k0 + STEP);
@@ -406,7 +448,8 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
               "exo_sdpa_decode: null pointer");
   SdpaParams p{q, k_cache, v_cache, pos, out, workspace,
                reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
-               Hkv, S_max, pick_splits(B, Hkv, S_max), nullptr, nullptr, nullptr, nullptr, 0.f};
+               Hkv, S_max, pick_splits(B, Hkv, S_max), nullptr, nullptr, nullptr, nullptr, nullptr,
+               0.f};
   rc = (D == 64) ? launch_sdpa<64, 1>(p, (hipStream_t)stream)
                  : launch_sdpa<128, 1>(p, (hipStream_t)stream);
   if (rc) return rc;
@@ -414,8 +457,29 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
   return EXO_OK;
 }
 
+__global__ __launch_bounds__(256) void rope_table_kernel(const float* __restrict__ inv_freq,
+                                                         float2* __restrict__ tab, int n,
+                                                         int half) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float sn, cs;
+  sincosf((float)(i / half) * inv_freq[i % half], &sn, &cs);
+  tab[i] = make_float2(cs, sn);
+}
+
+extern "C" int exo_rope_table(const float* inv_freq, float* table, int S_max, int D,
+                              exo_stream_t stream) {
+  EXO_REQUIRE(inv_freq && table && S_max > 0 && (D == 64 || D == 128),
+              "exo_rope_table: bad argument (D must be 64 or 128)");
+  const int n = S_max * (D / 2);
+  rope_table_kernel<<<dim3(exo_ceil_div(n, 256)), 256, 0, (hipStream_t)stream>>>(
+      inv_freq, reinterpret_cast<float2*>(table), n, D / 2);
+  EXO_CHECK_LAUNCH("exo_rope_table");
+  return EXO_OK;
+}
+
 extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
-                               const int32_t* pos, const float* inv_freq,
+                               const int32_t* pos, const float* inv_freq, const float* rope_table,
                                const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
                                uint16_t* out, float* workspace, float scale, int B, int Hq,
                                int Hkv, int D, int S_max, exo_stream_t stream) {
@@ -425,7 +489,8 @@ extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t*
               "exo_attn_decode: null pointer");
   SdpaParams p{nullptr, k_cache, v_cache, pos, out, workspace,
                reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
-               Hkv, S_max, pick_splits(B, Hkv, S_max), qkv, inv_freq, q_norm_w, k_norm_w, eps};
+               Hkv, S_max, pick_splits(B, Hkv, S_max), qkv, inv_freq,
+               reinterpret_cast<const float2*>(rope_table), q_norm_w, k_norm_w, eps};
   rc = (D == 64) ? launch_sdpa<64, 2>(p, (hipStream_t)stream)
                  : launch_sdpa<128, 2>(p, (hipStream_t)stream);
   if (rc) return rc;
@@ -441,7 +506,7 @@ extern "C" int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache,
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out, "exo_sdpa_prefill: null pointer");
   SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, nullptr, scale, B, T, Hq, Hkv, S_max, 1,
-               nullptr, nullptr, nullptr, nullptr, 0.f};
+               nullptr, nullptr, nullptr, nullptr, nullptr, 0.f};
   rc = (D == 64) ? launch_sdpa<64, 0>(p, (hipStream_t)stream)
                  : launch_sdpa<128, 0>(p, (hipStream_t)stream);
   if (rc) return rc;

@@ -145,6 +145,7 @@ class ShardModel:
         self.scale = cfg.head_dim ** -0.5
         self._bufs: dict[tuple[int, int], _Buffers] = {}
         self._graphs: dict[int, tuple] = {}
+        self._rope_tab: torch.Tensor | None = None
 
     # ------------------------------------------------------------------ properties
     @property
@@ -154,6 +155,12 @@ class ShardModel:
     @property
     def is_last(self) -> bool:
         return self.end_layer == self.cfg.num_hidden_layers
+
+    def _rope_table(self, n: int) -> torch.Tensor:
+        """(cos, sin) table covering n positions, built once on the device."""
+        if self._rope_tab is None or self._rope_tab.shape[0] < n:
+            self._rope_tab = ops.rope_table(self.inv_freq, n, self.cfg.head_dim)
+        return self._rope_tab
 
     def weight_bytes(self) -> int:
         n = sum(l.nbytes() for l in self.layers)
@@ -225,7 +232,8 @@ class ShardModel:
                 ops.quantized_matmul(bf.n, L.qkv, out=bf.qkv)
             if T == 1:  # rope + append + attention in one launch
                 ops.attn_decode(bf.qkv, kc, vc, pos, self.inv_freq, bf.attn, bf.sdpa_ws, self.scale,
-                                B, Hq, Hkv, D, L.q_norm, L.k_norm, c.rms_norm_eps)
+                                B, Hq, Hkv, D, L.q_norm, L.k_norm, c.rms_norm_eps,
+                                rope_tab=self._rope_table(cache.max_seq))
             else:
                 ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
                                    L.q_norm, L.k_norm, c.rms_norm_eps)

@@ -303,13 +303,24 @@ def sdpa_decode(q, k_cache, v_cache, pos, out, workspace, scale, B, Hq, Hkv, D):
     )
 
 
+def rope_table(inv_freq: torch.Tensor, S_max: int, D: int) -> torch.Tensor:
+    """float32 [S_max, D/2, 2]: (cos, sin) of position * inv_freq."""
+    lib = native.load()
+    tab = torch.empty(S_max, D // 2, 2, dtype=torch.float32, device=inv_freq.device)
+    check(lib.exo_rope_table(_ptr(inv_freq), _ptr(tab), S_max, D, _stream()), "rope_table")
+    return tab
+
+
 def attn_decode(qkv, k_cache, v_cache, pos, inv_freq, out, workspace, scale, B, Hq, Hkv, D,
-                q_norm_w=None, k_norm_w=None, eps: float = 0.0):
+                q_norm_w=None, k_norm_w=None, eps: float = 0.0, rope_tab=None):
     """rope (+ head norm) + cache append + attention for one new token per sequence."""
     lib = native.load()
+    if rope_tab is not None and rope_tab.shape[0] < k_cache.shape[2]:
+        raise ValueError("rope table shorter than the cache")
     check(
         lib.exo_attn_decode(
-            _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), _ptr(q_norm_w),
+            _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), _ptr(rope_tab),
+            _ptr(q_norm_w),
             _ptr(k_norm_w), eps, _ptr(out), _ptr(workspace), scale, B, Hq, Hkv, D,
             k_cache.shape[2], _stream(),
         ),

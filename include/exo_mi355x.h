@@ -139,13 +139,20 @@ int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* 
 /* K6+K10+K7 fused for decode: one launch per layer does what exo_rope_kv_append followed
  * by exo_sdpa_decode do for T == 1: q and k heads of the fused qkv row [B,(Hq+2Hkv)*D] are
  * (head-normalised and) rotated at position pos[b], the new k,v are appended to the
- * cache at pos[b], and attention runs over pos[b]+1 keys.  Same workspace contract as
+ * cache at pos[b], and attention runs over pos[b]+1 keys (pos[b] < S_max, and < the
+ * table's S_max when rope_table is given).  Same workspace contract as
  * exo_sdpa_decode.  No separate reference operator: it is rope + update_and_fetch +
  * scaled_dot_product_attention of one attention block. */
 int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
-                    const int32_t* pos, const float* inv_freq, const uint16_t* q_norm_w,
-                    const uint16_t* k_norm_w, float eps, uint16_t* out, float* workspace,
-                    float scale, int B, int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
+                    const int32_t* pos, const float* inv_freq, const float* rope_table,
+                    const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps, uint16_t* out,
+                    float* workspace, float scale, int B, int Hq, int Hkv, int D, int S_max,
+                    exo_stream_t stream);
+
+/* (cos, sin) of position*inv_freq[i] for every position < S_max: float [S_max, D/2, 2],
+ * the same sincosf values the RoPE kernels compute inline.  Passing it to
+ * exo_attn_decode (may be null there) replaces 8 sincosf per lane by one 64-byte load. */
+int exo_rope_table(const float* inv_freq, float* table, int S_max, int D, exo_stream_t stream);
 
 /* K7 prefill: causal attention of T new tokens per sequence (already appended to the
  * cache) over pos[b]+T keys.  q bf16 [B*T, Hq*D] -> out same shape. */

@@ -322,7 +322,8 @@ def test_norm_qmv_fused(device, bits, N, K, M):
 @pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 64, 4), (128, 4, 4)])
 @pytest.mark.parametrize("qk_norm", [False, True])
 @pytest.mark.parametrize("lens", [[1, 2], [100, 37], [513, 1000]])
-def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens):
+@pytest.mark.parametrize("table", [False, True])
+def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens, table):
     """rope + head norm + cache append + attention in one launch == the three oracle ops."""
     B, S_max = len(lens), 1024
     pos = np.array([n - 1 for n in lens], np.int32)
@@ -336,10 +337,13 @@ def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens):
     kc, vc = t_bf16(k, device), t_bf16(v, device)
     out = torch.empty(B, Hq * D, dtype=torch.bfloat16, device=device)
     ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+    inv_t = torch.from_numpy(inv).to(device)
+    tab = ops.rope_table(inv_t, S_max, D) if table else None
     for _ in range(2):  # twice: the arrival counters must be back at zero
         ops.attn_decode(t_bf16(qkv, device), kc, vc, torch.from_numpy(pos).to(device),
-                        torch.from_numpy(inv).to(device), out, ws, D ** -0.5, B, Hq, Hkv, D,
-                        t_bf16(qn, device) if qk_norm else None, t_bf16(kn, device) if qk_norm else None, 1e-6)
+                        inv_t, out, ws, D ** -0.5, B, Hq, Hkv, D,
+                        t_bf16(qn, device) if qk_norm else None, t_bf16(kn, device) if qk_norm else None, 1e-6,
+                        rope_tab=tab)
     x = qkv.reshape(B, 1, Hq + 2 * Hkv, D)
     q, kk, vv = x[:, :, :Hq], x[:, :, Hq:Hq + Hkv], x[:, :, Hq + Hkv:]
     if qk_norm:
