@@ -80,6 +80,35 @@ __device__ __forceinline__ float sumsq_word(const uint4& xv) {
          bf_lo(xv.w) * bf_lo(xv.w) + bf_hi(xv.w) * bf_hi(xv.w);
   return s;
 }
+// dot2 register order of one word's activations, with the sum of the stored values
+// (8-bit stores x and 16x) and of the plain values
+template <int BITS>
+__device__ __forceinline__ uint4 permute_word(const uint4& xv, float& stored, float& truesum) {
+  uint4 o;
+  if (BITS == 4) {
+    o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
+    o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
+    o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
+    o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
+    truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
+              (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
+    stored = truesum;
+  } else {
+    const uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);   // (x0,x2)
+    const uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u);  // (x1,x3)
+    o.x = a;
+    o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
+    o.z = c2;
+    o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
+    truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
+    stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
+  }
+  return o;
+}
+
+template <int MT, int ITERS, int NMAT>
+constexpr bool kRowsXR = (MT == 1 && ITERS <= 2 && NMAT == 1);
+
 template <int BITS>
 __device__ __forceinline__ uint4 load_word_x(const bf16_t* base, int wi) {
   if (BITS == 4) return *reinterpret_cast<const uint4*>(base + (size_t)wi * 8);
@@ -537,6 +566,12 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // Long rows: that would cost hundreds of VGPRs and the occupancy that hides HBM
   // latency, so the LDS offset is made opaque per batch and x is re-read from LDS.
   constexpr bool X_IN_REGS = ITERS * MT <= 2;
+  // XR: a single activation row whose share per lane (ITERS * 64 bytes) fits in
+  // registers.  Every wave then holds the whole row across its lanes: no LDS, no
+  // barrier, and the fused RMSNorm needs only a wave reduction.
+  constexpr bool XR = kRowsXR<MT, ITERS, NMAT>;
+  uint4 xr[XR ? ITERS : 1][4];
+  float2 sxr[XR ? ITERS : 1];
   int xlane = lane;
   uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
   asm volatile("" : "+s"(kmask));
@@ -561,7 +596,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
           float d[NMAT][MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
-            sm[m] = sx[m * CPR + j * 64 + xlane];
+            sm[m] = XR ? sxr[XR ? j : 0] : sx[m * CPR + j * 64 + xlane];
 #pragma unroll
             for (int a = 0; a < NMAT; ++a) d[a][m] = -sm[m].x;
           }
@@ -573,7 +608,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
               unpack_word_r(reinterpret_cast<const uint32_t*>(&bt.w[a][i])[t], kmask, kmagic, pr[a]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
-              const uint4 xv = xs[m * (4 * CPR) + (j * 4 + t) * 64 + xlane];
+              const uint4 xv = XR ? xr[XR ? j : 0][t] : xs[m * (4 * CPR) + (j * 4 + t) * 64 + xlane];
 #pragma unroll
               for (int a = 0; a < NMAT; ++a) {
                 d[a][m] = dot2_bf16(pr[a][0], xv.x, d[a][m]);
@@ -616,15 +651,59 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 
   // Order of the prologue: activations first (they sit in L2 and are waited for with
   // the weight loads still outstanding), then two weight batches, then the LDS staging.
-  XStage<BITS, MT, ITERS> xst;
-  stage_x_load<BITS, MT, ITERS>(p, xin, xst);
   Batch ba, bb2;
-  if (nrows > 0) issue(ba, r0);
-  if (nrows > R) issue(bb2, r0 + R);
-  __shared__ float s_red[4 * MT];
-  stage_x_store<BITS, MT, ITERS>(p, xst, xs, sx, s_red);
-  __syncthreads();
-  if (nrows <= 0) return;
+  if (XR) {
+    if (nrows <= 0) return;
+    uint4 raw[ITERS][4], nwv[ITERS][4];
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int wi = 4 * (lane + 64 * j) + t;
+        raw[j][t] = load_word_x<BITS>(xin, wi);
+        if (p.norm_w) nwv[j][t] = load_word_x<BITS>(p.norm_w, wi);
+      }
+    issue(ba, r0);
+    if (p.norm_w) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < ITERS; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ss += sumsq_word<BITS>(raw[j][t]);
+      ss = wave_sum_to_lane63(ss);
+      ss = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ss), 63));
+      const float inv = rsqrtf(ss / (float)p.K + p.eps);
+#pragma unroll
+      for (int j = 0; j < ITERS; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) norm_word<BITS>(raw[j][t], nwv[j][t], inv);
+    }
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      float stored = 0.f, truesum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float st_, ts_;
+        xr[XR ? j : 0][t] = permute_word<BITS>(raw[j][t], st_, ts_);
+        stored += st_;
+        truesum += ts_;
+      }
+      sxr[XR ? j : 0] = make_float2(128.f * stored, truesum);
+    }
+    // the second batch only now: the raw activations and norm weights are dead, so
+    // the register peak stays at what the main loop needs
+    asm volatile("" ::: "memory");
+    if (nrows > R) issue(bb2, r0 + R);
+  } else {
+    XStage<BITS, MT, ITERS> xst;
+    stage_x_load<BITS, MT, ITERS>(p, xin, xst);
+    if (nrows > 0) issue(ba, r0);
+    __shared__ float s_red[4 * MT];
+    stage_x_store<BITS, MT, ITERS>(p, xst, xs, sx, s_red);
+    __syncthreads();
+    if (nrows <= 0) return;
+    if (nrows > R) issue(bb2, r0 + R);
+  }
 
   // two register buffers in ping-pong: two batches are in flight while one is consumed,
   // without copying registers
@@ -693,7 +772,7 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
   if (grid < 1) grid = 1;
-  kern<<<dim3(grid, pairs), dim3(kThreads), pl.lds, st>>>(p);
+  kern<<<dim3(grid, pairs), dim3(kThreads), kRowsXR<MT, ITERS, NMAT> ? 0 : pl.lds, st>>>(p);
   return EXO_OK;
 }
 
