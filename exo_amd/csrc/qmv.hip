@@ -16,6 +16,7 @@
 //    per workgroup.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
+#include "qmv_internal.h"
 
 namespace {
 
@@ -910,6 +911,25 @@ extern "C" int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, floa
   if (rc) return rc;
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmv: null pointer");
   if (M == 0) return EXO_OK;
+  // two or more rows: the matrix-core GEMV streams W once per tile of up to 16 rows
+  const int cap = M >= 2 ? exo_qmv_mfma_max_rows(K, bits) : 0;
+  if (cap >= 2) {
+    int m0 = 0;
+    while (M - m0 >= 2) {
+      const int mt = (M - m0 < cap) ? (M - m0) : cap;
+      rc = exo_qmv_mfma_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases,
+                               residual ? residual + (size_t)m0 * N : nullptr, y + (size_t)m0 * N,
+                               mt, N, K, bits, (hipStream_t)stream);
+      if (rc) return rc;
+      m0 += mt;
+    }
+    EXO_CHECK_LAUNCH("exo_qmv");
+    if (m0 == M) return EXO_OK;
+    x += (size_t)m0 * K;  // a single left-over row takes the dot2 kernel below
+    y += (size_t)m0 * N;
+    if (residual) residual += (size_t)m0 * N;
+    M -= m0;
+  }
   const uint32_t* ws[1] = {w};
   const bf16_t* ss[1] = {scales};
   const bf16_t* bs[1] = {biases};
