@@ -14,6 +14,7 @@ exo's MpSender / MpReceiver satisfy both.
 
 from __future__ import annotations
 
+import logging
 import os
 import time
 from abc import ABC, abstractmethod
@@ -33,7 +34,10 @@ from .generate import (
 )
 from .loader import load_shard_weights
 from .model import ShardModel
+from .prefix_cache import KVPrefixCache, save_prefix_cache
 from .tokenizer import load_tokenizer
+logger = logging.getLogger("exo_amd")
+
 from .types import (
     BoundInstance, CancelledResponse, ErrorChunk, FinishedResponse, GenerationResponse,
     GenerationStats, GenerationTask, ModelLoadingResponse, PrefillProgressChunk,
@@ -99,6 +103,7 @@ class _Seq:
     prefill_tokens: int
     on_generation_token: Callable[[], None] | None
     stop_sequences: list[str]
+    prefix_cache_hit: str = "none"
     tokens: list[int] = field(default_factory=list)
     n_gen: int = 0
     t_first: float | None = None
@@ -114,12 +119,13 @@ class ShardBatchGenerator:
     uids.  Active rows are kept compact at the front of the pool."""
 
     def __init__(self, model: ShardModel, tokenizer, max_batch: int = EXO_MAX_CONCURRENT_REQUESTS,
-                 max_seq: int = 8192):
+                 max_seq: int = 8192, kv_prefix_cache: KVPrefixCache | None = None):
         if not (model.is_first and model.is_last):
             raise ValueError("the batch generator needs a shard that holds the whole model")
         self.model, self.tokenizer = model, tokenizer
         self.max_batch, self.max_seq = max_batch, max_seq
         self.cache: ShardKVCache = model.make_cache(max_batch, max_seq)
+        self.kv_prefix_cache = kv_prefix_cache
         self.rows: list[_Seq] = []
         self._next_uid = 0
         self._pending_input: list[int] = []  # token to feed per active row
@@ -147,7 +153,16 @@ class ShardBatchGenerator:
             if max_tokens <= 0:
                 raise ValueError(f"prompt of {len(toks)} tokens exceeds the cache ({self.max_seq})")
         row = len(self.rows)
-        self.cache.reset(rows=range(row, row + 1))
+        # prefix cache lookup (batch_generate.py:164-181): bench requests opt in
+        use_prefix = self.kv_prefix_cache is not None and (
+            not task_params.bench or task_params.use_prefix_cache)
+        matched_index, is_exact_hit, remaining = None, False, toks
+        if use_prefix:
+            _, remaining, matched_index, is_exact_hit = self.kv_prefix_cache.get_kv_cache(
+                self.cache, toks, row=row)
+        else:
+            self.cache.reset(rows=range(row, row + 1))
+        prefix_hit_length = len(toks) - len(remaining)
 
         def progress(done: int, total: int) -> None:
             if distributed_prompt_progress_callback is not None:
@@ -156,13 +171,24 @@ class ShardBatchGenerator:
                 on_prefill_progress(done, total)
 
         try:
-            tps, n = prefill(self.model, toks[:-1], self.cache, progress, row=row)
+            tps, n = prefill(self.model, remaining[:-1], self.cache, progress, row=row)
         except PrefillCancelled:
             self.cache.reset(rows=range(row, row + 1))
             raise
-        if len(toks) >= 2:
-            self.model(torch.tensor([[toks[-2]]], dtype=torch.int32), self.cache, logits="none",
-                       rows=slice(row, row + 1))
+        prefix_cache_hit = "none"
+        if matched_index is not None and prefix_hit_length > 0:
+            prefix_cache_hit = "exact" if is_exact_hit else "partial"
+            if is_exact_hit:
+                tps = self.kv_prefix_cache.prefill_tps[matched_index]
+        if use_prefix:
+            try:
+                save_prefix_cache(self.kv_prefix_cache, toks, self.cache, row, prefix_hit_length,
+                                  matched_index, prefill_tps=tps)
+            except Exception:  # a failed save never fails the request (batch_generate.py:534)
+                logger.warning("failed to save prefix cache", exc_info=True)
+        if len(remaining) >= 2:
+            self.model(torch.tensor([[remaining[-2]]], dtype=torch.int32), self.cache,
+                       logits="none", rows=slice(row, row + 1))
         gen = torch.Generator(device=self.model.device)
         gen.manual_seed(task_params.seed or 42)
         processors = [ban_token_ids(self._eos())] if task_params.bench and self._eos() else []
@@ -175,6 +201,7 @@ class ShardBatchGenerator:
                 task_params.top_k if task_params.top_k is not None else 0, gen),
             processors=processors, greedy=(temp == 0 and not processors), max_tokens=max_tokens,
             prefill_tps=tps, prefill_tokens=n, on_generation_token=on_generation_token,
+            prefix_cache_hit=prefix_cache_hit,
             stop_sequences=[task_params.stop] if isinstance(task_params.stop, str)
             else list(task_params.stop or []),
             tokens=list(toks))
@@ -236,7 +263,8 @@ class ShardBatchGenerator:
                     prompt_tps=float(seq.prefill_tps),
                     generation_tps=float((seq.n_gen - 1) / dt) if dt > 0 else 0.0,
                     prompt_tokens=len(seq.prompt_tokens), generation_tokens=seq.n_gen,
-                    peak_memory_usage=int(torch.cuda.max_memory_allocated(self.model.device)))
+                    peak_memory_usage=int(torch.cuda.max_memory_allocated(self.model.device)),
+                    prefix_cache_hit=seq.prefix_cache_hit)
                 n_p = len(seq.prompt_tokens)
                 usage = Usage(n_p, seq.n_gen, n_p + seq.n_gen)
                 finished.append(r)
@@ -300,18 +328,20 @@ class BatchGenerator(Engine):
     event_sender: Any = None
     check_for_cancel_every: int = 50
     max_seq: int = 8192
+    kv_prefix_cache: KVPrefixCache | None = None
     gen_factory: Any = None  # tests inject a fake inner generator (like the reference's FakeExoBatchGenerator)
     _cancelled_tasks: set = field(default_factory=set, init=False)
     _all_tasks: dict = field(default_factory=dict, init=False)
     _queue: deque = field(default_factory=deque, init=False)
     _active_tasks: dict = field(default_factory=dict, init=False)
+    _prefill_cache: Any = field(default=None, init=False)
 
     def __post_init__(self) -> None:
         if self.gen_factory is not None:
             self._gen = self.gen_factory()
         else:
             self._gen = ShardBatchGenerator(self.model, self.tokenizer, EXO_MAX_CONCURRENT_REQUESTS,
-                                            self.max_seq)
+                                            self.max_seq, self.kv_prefix_cache)
 
     def warmup(self) -> None:
         """generate.py:399-462: a short greedy generation on a fixed prompt; sets how
@@ -430,7 +460,19 @@ class BatchGenerator(Engine):
         self.tokenizer = None
 
     def serve_prefill(self, request, wfile) -> None:
-        raise NotImplementedError("disaggregated prefill serving is not part of this engine yet")
+        """Prefill ``request.token_ids`` and stream the KV to ``wfile`` in the reference's
+        wire format (batch_generator.py:558-572).  Runs on the engine's thread in a KV row
+        of its own, so running generations are not disturbed."""
+        from .disaggregated import run_prefill_for_request, write_cache_to_wire
+        n = len(request.token_ids)
+        if n > self.max_seq:
+            raise ValueError(f"prefill request of {n} tokens exceeds the cache ({self.max_seq})")
+        if self._prefill_cache is None:
+            self._prefill_cache = self.model.make_cache(1, self.max_seq)
+        cache = run_prefill_for_request(model=self.model, kv_prefix_cache=self.kv_prefix_cache,
+                                        request=request, cache=self._prefill_cache, row=0)
+        write_cache_to_wire(wfile, cache, row=0, request_id=request.request_id,
+                            model_id=request.model_id, start_pos=request.start_pos)
 
 
 # ----------------------------------------------------------------------- Builder
@@ -490,7 +532,8 @@ class Mi355xBuilder(Builder):
         return BatchGenerator(model=self.inference_model, tokenizer=self.tokenizer,
                               model_id=self.model_id, device_rank=0,
                               cancel_receiver=self.cancel_receiver, event_sender=self.event_sender,
-                              max_seq=self.max_seq)
+                              max_seq=self.max_seq,
+                              kv_prefix_cache=KVPrefixCache(None, self.device))  # builder.py:83
 
     def close(self) -> None:
         self.inference_model = None

@@ -136,9 +136,11 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
              on_prefill_progress: Callable[[int, int], None] | None = None,
              on_generation_token: Callable[[], None] | None = None,
              max_seq: int | None = None, eos_token_ids: list[int] | None = None,
-             ) -> Generator[GenerationResponse, None, None]:
+             kv_prefix_cache=None) -> Generator[GenerationResponse, None, None]:
     """Sequential (batch 1) generation for a full-model shard: yields one
-    GenerationResponse per token; the last carries finish_reason, stats and usage."""
+    GenerationResponse per token; the last carries finish_reason, stats and usage.
+    ``kv_prefix_cache`` (a KVPrefixCache) is consulted and updated the way the reference's
+    mlx_generate does (generate.py:577-706): bench requests only with use_prefix_cache."""
     if not (model.is_first and model.is_last):
         raise ValueError("generate() needs a shard that holds the whole model")
     seed = task.seed or 42
@@ -163,12 +165,27 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     greedy = (task.temperature == 0) and not processors
     stop_sequences = [task.stop] if isinstance(task.stop, str) else list(task.stop or [])
 
-    prefill_tps, prefill_tokens = prefill(model, prompt_tokens[:-1], cache, on_prefill_progress)
-    assert cache_length(cache) == max(n_prompt - 2, 0)
+    if task.bench and not task.use_prefix_cache:
+        kv_prefix_cache = None
+    remaining, matched_index, is_exact_hit = list(prompt_tokens), None, False
+    if kv_prefix_cache is not None:
+        _, remaining, matched_index, is_exact_hit = kv_prefix_cache.get_kv_cache(cache, prompt_tokens)
+    prefix_hit_length = n_prompt - len(remaining)
+    prefill_tps, prefill_tokens = prefill(model, remaining[:-1], cache, on_prefill_progress)
+    assert cache_length(cache) == max(n_prompt - 2, prefix_hit_length)
+    prefix_cache_hit = "none"
+    if matched_index is not None and prefix_hit_length > 0:
+        prefix_cache_hit = "exact" if is_exact_hit else "partial"
+        if is_exact_hit:
+            prefill_tps = kv_prefix_cache.prefill_tps[matched_index]
+    if kv_prefix_cache is not None:
+        from .prefix_cache import save_prefix_cache
+        save_prefix_cache(kv_prefix_cache, prompt_tokens, cache, 0, prefix_hit_length,
+                          matched_index, prefill_tps=prefill_tps)
 
     # the last two prompt tokens, one forward each (generate.py:710-733)
-    if n_prompt >= 2:
-        model(torch.tensor([[prompt_tokens[-2]]], dtype=torch.int32), cache, logits="none")
+    if len(remaining) >= 2:
+        model(torch.tensor([[remaining[-2]]], dtype=torch.int32), cache, logits="none")
     tok = int(prompt_tokens[-1])
     history = list(prompt_tokens)
     accumulated = ""
@@ -218,7 +235,8 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
             stats = GenerationStats(
                 prompt_tps=float(prefill_tps), generation_tps=float((n_gen - 1) / dt) if dt > 0 else 0.0,
                 prompt_tokens=int(prefill_tokens + min(n_prompt, 2)), generation_tokens=n_gen,
-                peak_memory_usage=int(torch.cuda.max_memory_allocated(model.device)))
+                peak_memory_usage=int(torch.cuda.max_memory_allocated(model.device)),
+                prefix_cache_hit=prefix_cache_hit)
             usage = Usage(n_prompt, n_gen, n_prompt + n_gen)
         if on_generation_token is not None:
             on_generation_token()

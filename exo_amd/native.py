@@ -38,6 +38,8 @@ SIGNATURES: dict[str, tuple] = {
     "exo_attn_decode": (_i, [_vp] * 8 + [_f, _vp, _vp, _f] + [_i] * 5 + [_vp]),
     "exo_rope_table": (_i, [_vp, _vp, _i, _i, _vp]),
     "exo_sdpa_prefill": (_i, [_vp] * 5 + [_f] + [_i] * 6 + [_vp]),
+    "exo_kv_export_nhd": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "exo_kv_import_nhd": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "exo_swiglu": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "exo_router_topk": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "exo_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

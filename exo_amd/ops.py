@@ -339,6 +339,38 @@ def sdpa_prefill(q, k_cache, v_cache, pos, out, scale, B, T, Hq, Hkv, D):
     )
 
 
+def kv_export_nhd(cache_row, start: int, n: int, out=None):
+    """Positions [start, start+n) of one layer's cache row [Hkv,S_max,D] -> [n,Hkv,D]."""
+    lib = native.load()
+    Hkv, S_max, D = cache_row.shape
+    if not cache_row.is_contiguous():
+        raise ValueError("kv_export_nhd: cache row must be contiguous")
+    if out is None:
+        out = torch.empty(n, Hkv, D, dtype=cache_row.dtype, device=cache_row.device)
+    if n == 0 and 0 <= start <= S_max:
+        return out
+    check(lib.exo_kv_export_nhd(_ptr(cache_row), _ptr(out), Hkv, S_max, D, start, n, _stream()),
+          "kv_export_nhd")
+    return out
+
+
+def kv_import_nhd(wire, cache_row, start: int):
+    """wire [n,Hkv,D] -> positions [start, start+n) of cache_row [Hkv,S_max,D] (in place)."""
+    lib = native.load()
+    Hkv, S_max, D = cache_row.shape
+    n = wire.shape[0]
+    if tuple(wire.shape[1:]) != (Hkv, D) or wire.dtype != cache_row.dtype:
+        raise ValueError(f"kv_import_nhd: wire {tuple(wire.shape)} does not fit cache row "
+                         f"{tuple(cache_row.shape)}")
+    if not (cache_row.is_contiguous() and wire.is_contiguous()):
+        raise ValueError("kv_import_nhd: tensors must be contiguous")
+    if n == 0 and 0 <= start <= S_max:
+        return cache_row
+    check(lib.exo_kv_import_nhd(_ptr(wire), _ptr(cache_row), Hkv, S_max, D, start, n, _stream()),
+          "kv_import_nhd")
+    return cache_row
+
+
 def swiglu(gate, up, out=None):
     lib = native.load()
     if out is None:

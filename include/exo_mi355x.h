@@ -160,6 +160,18 @@ int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache, const uint16_t*
                      const int32_t* pos, uint16_t* out, float scale, int B, int T, int Hq,
                      int Hkv, int D, int S_max, exo_stream_t stream);
 
+/* Disaggregated prefill, export: positions [start, start+n) of one layer's cache row
+ * ([Hkv, S_max, D] bf16) -> wire layout [n, Hkv, D] bf16, the `bhsd_to_nhd` transpose of
+ * src/exo/worker/engines/mlx/disaggregated/adapter.py:74-77,103-109.  D % 8 == 0,
+ * 16-byte aligned pointers. */
+int exo_kv_export_nhd(const uint16_t* cache_row, uint16_t* wire, int Hkv, int S_max, int D,
+                      int start, int n, exo_stream_t stream);
+
+/* Disaggregated prefill, ingest: wire [n, Hkv, D] -> positions [start, start+n) of a cache
+ * row (`nhd_to_bhsd` + `inject_kv_chunk`, adapter.py:80-83,182-201). */
+int exo_kv_import_nhd(const uint16_t* wire, uint16_t* cache_row, int Hkv, int S_max, int D,
+                      int start, int n, exo_stream_t stream);
+
 /* K8: swiglu(gate, up) = silu(gate)*up elementwise, n elements.
  * (.typings/mlx_lm/models/switch_layers.pyi:52-57) */
 int exo_swiglu(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n,

@@ -360,3 +360,35 @@ def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens, table):
         np.testing.assert_array_equal(n_f32(vc)[b, :, p], vv[b, 0])
         np.testing.assert_array_equal(n_f32(kc)[b, :, p + 1:], k[b, :, p + 1:])  # nothing else touched
         np.testing.assert_array_equal(n_f32(kc)[b, :, :p], k[b, :, :p])
+
+
+# ------------------------------------------------------------------ KV wire layout
+
+
+@pytest.mark.parametrize("Hkv,S_max,D,start,n", [(8, 64, 128, 0, 64), (4, 300, 64, 7, 201),
+                                                 (2, 16, 8, 15, 1), (3, 40, 128, 5, 0)])
+def test_kv_export_import_nhd(device, Hkv, S_max, D, start, n):
+    """Byte-exact against the transpose the reference ships
+    (engines/mlx/disaggregated/adapter.py:74-83): wire[t,h,:] = cache[h,start+t,:]."""
+    g = torch.Generator(device="cpu").manual_seed(5)
+    row = torch.randn(Hkv, S_max, D, generator=g).bfloat16().to(device)
+    wire = ops.kv_export_nhd(row, start, n)
+    want = row[:, start:start + n].permute(1, 0, 2).contiguous()
+    assert wire.shape == (n, Hkv, D) and torch.equal(wire.view(torch.int16), want.view(torch.int16))
+    dst = torch.full_like(row, 7.0)
+    ops.kv_import_nhd(wire, dst, start)
+    ref = torch.full_like(row, 7.0)
+    ref[:, start:start + n] = row[:, start:start + n]
+    assert torch.equal(dst.view(torch.int16), ref.view(torch.int16))
+
+
+def test_kv_wire_argument_errors(device):
+    row = torch.zeros(2, 16, 8, dtype=torch.bfloat16, device=device)
+    with pytest.raises(ValueError):
+        ops.kv_export_nhd(row, 10, 7)            # beyond S_max
+    with pytest.raises(ValueError):
+        ops.kv_export_nhd(row, -1, 2)
+    with pytest.raises(ValueError):
+        ops.kv_import_nhd(torch.zeros(3, 2, 4, dtype=torch.bfloat16, device=device), row, 0)
+    with pytest.raises(ValueError):
+        ops.kv_export_nhd(torch.zeros(2, 16, 12, dtype=torch.bfloat16, device=device), 0, 1)

@@ -293,3 +293,190 @@ def test_builder_engine_contract(ckpt, device):
     assert type(sender.sent[-1][1]).__name__ == "ErrorChunk" and sender.sent[-1][0] == "cmd-3"
     eng.close()
     b.close()
+
+
+def _run_requests(gm, prompts, params, pc, max_seq=2048):
+    """Submit the prompts one after the other (each runs to completion) through one
+    generator; returns the token lists and the per-request prefix-hit labels."""
+    g = ShardBatchGenerator(gm, None, max_batch=2, max_seq=max_seq, kv_prefix_cache=pc)
+    outs, hits = [], []
+    for p in prompts:
+        g.submit(params, p)
+        toks = []
+        while g.has_work:
+            for _, r in g.step():
+                toks.append(r.token)
+                if r.stats is not None:
+                    hits.append(r.stats.prefix_cache_hit)
+        outs.append(toks)
+    return outs, hits
+
+
+def test_prefix_cache_generation_invariants(ckpt, device):
+    """The generation-level invariants of the reference's prefix-cache tests
+    (src/exo/worker/tests/unittests/test_mlx/test_kv_prefix_cache.py:345-412,495-532):
+    a request stores N-2 positions; the same prompt again is an exact hit with exactly
+    the last two tokens left to feed and produces the same tokens; the stored entry is
+    not touched by the generation that used it."""
+    from exo_amd.prefix_cache import KVPrefixCache, cache_length
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    prompt = [int(t) for t in rng(61).integers(0, cfg.vocab_size, size=40)]
+    params = TextGenerationTaskParams(model="tiny", max_output_tokens=8, temperature=0.0)
+    (cold,), _ = _run_requests(gm, [prompt], params, None)
+    pc = KVPrefixCache(None, device)
+    (first, second), hits = _run_requests(gm, [prompt, prompt], params, pc)
+    assert first == cold and second == cold and hits == ["none", "exact"]
+    assert len(pc.prompts) == 2  # short prompts add entries (hit < 1000 tokens)
+    assert cache_length(pc.caches[0]) == len(prompt) - 2
+    before = [t.clone() for t in pc.caches[0].layers]
+    probe = gm.make_cache(1, 256)
+    _, remaining, idx, exact = pc.get_kv_cache(probe, prompt)
+    assert idx == 0 and exact and remaining == prompt[-2:]
+    assert all(torch.equal(a, b) for a, b in zip(before, pc.caches[0].layers))
+    # partial hit: same first 25 tokens, different tail -> same tokens as a cold run
+    other = prompt[:25] + [int(t) for t in rng(62).integers(0, cfg.vocab_size, size=9)]
+    (cold_other,), _ = _run_requests(gm, [other], params, None)
+    pc2 = KVPrefixCache(None, device)
+    (_, warm_other), hits = _run_requests(gm, [prompt, other], params, pc2)
+    assert warm_other == cold_other and hits == ["none", "partial"]
+
+
+def test_prefix_cache_long_prompt_updates_in_place(ckpt, device):
+    """test_kv_prefix_cache.py:414-493: a second prompt sharing more than 1000 tokens
+    (and more than half) with a stored one replaces that entry with the longer cache."""
+    from exo_amd.prefix_cache import KVPrefixCache, cache_length
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    base = [int(t) for t in rng(71).integers(0, cfg.vocab_size, size=1100)]
+    longer = base[:1080] + [int(t) for t in rng(72).integers(0, cfg.vocab_size, size=60)]
+    params = TextGenerationTaskParams(model="tiny", max_output_tokens=4, temperature=0.0)
+    (cold,), _ = _run_requests(gm, [longer], params, None)
+    pc = KVPrefixCache(None, device)
+    (_, warm), hits = _run_requests(gm, [base, longer], params, pc)
+    assert hits == ["none", "partial"] and len(pc.prompts) == 1
+    assert cache_length(pc.caches[0]) == len(longer) - 2 and len(pc.prompts[0]) == len(longer)
+    # the restored prefix went through the same kernels as the cold prefill's first 1080
+    # positions did only if both used the GEMM path; tokens must still agree
+    assert warm == cold
+
+
+def test_sequential_generate_with_prefix_cache(ckpt, device):
+    from exo_amd.prefix_cache import KVPrefixCache, cache_length
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    prompt = [int(t) for t in rng(81).integers(0, cfg.vocab_size, size=30)]
+    params = TextGenerationTaskParams(model="tiny", max_output_tokens=6, temperature=0.0)
+    cold = [r.token for r in generate(gm, None, params, prompt, max_seq=128)]
+    pc = KVPrefixCache(None, device)
+    first = list(generate(gm, None, params, prompt, max_seq=128, kv_prefix_cache=pc))
+    assert cache_length(pc.caches[0]) == len(prompt) - 2
+    second = list(generate(gm, None, params, prompt, max_seq=128, kv_prefix_cache=pc))
+    assert [r.token for r in first] == cold and [r.token for r in second] == cold
+    assert first[-1].stats.prefix_cache_hit == "none" and second[-1].stats.prefix_cache_hit == "exact"
+    bench = TextGenerationTaskParams(model="tiny", max_output_tokens=2, temperature=0.0, bench=True)
+    third = list(generate(gm, None, bench, prompt, max_seq=128, kv_prefix_cache=pc))
+    assert third[-1].stats.prefix_cache_hit == "none"   # bench requests opt in explicitly
+
+
+# ------------------------------------------------------- disaggregated prefill
+
+
+def test_send_and_ingest_kv_cache(ckpt, device):
+    """Port of the reference's adapter tests
+    (engines/mlx/disaggregated/tests/test_mlx_adapter.py:115-180): a cache sent and
+    ingested is bit-identical; start_pos ships only the suffix; a fill level at or below
+    start_pos ships nothing."""
+    import io
+    from exo_amd import disaggregated as D
+    gm = ckpt["model"]
+    src = gm.make_cache(2, 64)
+    for t in src.k + src.v:
+        t.copy_(torch.randn(t.shape, device=device).bfloat16())
+    src.offsets[1] = 37
+    src.sync_pos()
+    buf = io.BytesIO()
+    sent = D.write_cache_to_wire(buf, src, row=1, request_id="r", model_id="m")
+    assert sent == 37
+    buf.seek(0)
+    res = D.read_result(buf)
+    assert res.header.num_layers == len(src) and res.total_tokens == 37
+    assert sorted(res.kv_chunks) == list(range(len(src)))
+    c0 = res.kv_chunks[0][0]
+    assert c0.shape == (37, src.k[0].shape[1], src.k[0].shape[3]) and c0.dtype == "bfloat16"
+    dst = gm.make_cache(1, 48)
+    assert D.ingest_into_cache(res, dst, row=0) == 37 and dst.offsets[0] == 37
+    assert dst.pos.tolist() == [37]
+    for i in range(len(src)):
+        assert torch.equal(dst.k[i][0, :, :37], src.k[i][1, :, :37])
+        assert torch.equal(dst.v[i][0, :, :37], src.v[i][1, :, :37])
+    # suffix only
+    buf = io.BytesIO()
+    assert D.write_cache_to_wire(buf, src, row=1, start_pos=30) == 7
+    buf.seek(0)
+    res = D.read_result(buf)
+    assert res.header.start_pos == 30 and res.kv_chunks[0][0].num_tokens == 7
+    dst.k[0][0, :, 30:37].zero_()
+    assert D.ingest_into_cache(res, dst, row=0, start_pos=30) == 37
+    assert torch.equal(dst.k[0][0, :, :37], src.k[0][1, :, :37])
+    # nothing to send
+    buf = io.BytesIO()
+    assert D.write_cache_to_wire(buf, src, row=1, start_pos=40) == 0
+    buf.seek(0)
+    res = D.read_result(buf)
+    assert res.kv_chunks == {} and res.total_tokens == 0
+
+
+def test_serve_prefill_over_tcp_then_decode(ckpt, device):
+    """The engine as prefill server: a request over the TCP front is resolved by
+    Engine.serve_prefill; the KV that arrives is bit-identical to a local prefill of the
+    same tokens and a decoder continuing from it produces the local tokens.  The server
+    stops three positions short of the tokens it is given (serve.py:43-58: target n-2,
+    and the prefill routine leaves one more out), so the client asks with one padding
+    token to receive N-2 positions."""
+    from exo_amd import disaggregated as D
+    from exo_amd.engine import BatchGenerator
+    from exo_amd.prefix_cache import KVPrefixCache
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    prompt = [int(t) for t in rng(91).integers(0, cfg.vocab_size, size=45)]
+    params = TextGenerationTaskParams(model="tiny", max_output_tokens=6, temperature=0.0)
+    want = [r.token for r in generate(gm, None, params, prompt, max_seq=128)]
+    local = gm.make_cache(1, 128)
+    prefill(gm, prompt[:-1], local)
+
+    eng = BatchGenerator(model=gm, tokenizer=None, model_id="tiny", max_seq=128,
+                         kv_prefix_cache=KVPrefixCache(None, device))
+    served = []
+
+    def resolve(job, wfile):  # the runner would queue this for the engine thread
+        eng.serve_prefill(job, wfile)
+        served.append(job.request_id)
+        return True
+
+    srv = D.PrefillServer(resolve, "127.0.0.1", 0)
+    try:
+        ep = f"127.0.0.1:{srv.server_address[1]}"
+        dec = gm.make_cache(1, 128)
+        progress = []
+        tps, n = D.remote_prefill(prompt + [0], dec, lambda d, t: progress.append((d, t)),
+                                  endpoint=ep, request_id="req-1", model_id="tiny")
+        assert served == ["req-1"] and n == len(prompt) - 2 and dec.offsets[0] == n and tps > 0
+        assert progress and progress[-1][1] == len(prompt) + 1
+        for i in range(len(dec)):
+            assert torch.equal(dec.k[i][0, :, :n], local.k[i][0, :, :n])
+            assert torch.equal(dec.v[i][0, :, :n], local.v[i][0, :, :n])
+        # the same request again is served from the server's prefix cache
+        dec2 = gm.make_cache(1, 128)
+        D.remote_prefill(prompt + [0], dec2, None, endpoint=ep, request_id="req-2", model_id="tiny")
+        assert torch.equal(dec2.k[0][0, :, :n], local.k[0][0, :, :n])
+        assert len(eng.kv_prefix_cache.prompts) == 1  # hit ratio >= 0.5: updated in place
+    finally:
+        srv.stop()
+    # decode from the ingested cache: feed prompt[-2], then generate from prompt[-1]
+    gm(torch.tensor([[prompt[-2]]], dtype=torch.int32), dec, logits="none")
+    tok, got = prompt[-1], []
+    for _ in range(6):
+        bufs = gm._buffers(1, 1)
+        bufs.tokens[0] = tok
+        bufs = gm.decode_step(dec, 1)
+        tok = int(bufs.next_token[0])
+        got.append(tok)
+    assert got == want
+    eng.close()

@@ -300,7 +300,112 @@ def test_engine_prefill_cancel_and_errors():
     with pytest.raises(RuntimeError):
         e2.step()
     assert type(s2.sent[-1][1]).__name__ == "ErrorChunk" and s2.sent[-1][0] == "cmd-q"
-    with pytest.raises(NotImplementedError):
-        e2.serve_prefill(None, None)
+    from exo_amd.disaggregated import PrefillRequest
+    with pytest.raises(ValueError, match="exceeds the cache"):
+        e2.serve_prefill(PrefillRequest("r", "m", list(range(e2.max_seq + 1)), 0), None)
     with pytest.raises(PrefillCancelled):
         raise PrefillCancelled()
+
+
+# ---------------------------------------------------------------- KV prefix cache
+
+
+@pytest.mark.parametrize("a,b,want", [
+    ([1, 2, 3, 4, 5], [1, 2, 3, 4, 5], 5), ([1, 2, 3], [4, 5, 6], 0),
+    ([1, 2, 3, 4, 5], [1, 2, 3, 7, 8], 3), ([1, 2, 3, 4, 5], [1, 2, 3], 3),
+    ([1, 2, 3], [1, 2, 3, 4, 5], 3), ([1, 2, 3], [1, 5, 6], 1),
+    ([], [1, 2, 3], 0), ([1, 2, 3], [], 0), ([], [], 0)])
+def test_get_prefix_length(a, b, want):
+    """The nine cases of the reference's TestGetPrefixLength
+    (src/exo/worker/tests/unittests/test_mlx/test_kv_prefix_cache.py:33-77)."""
+    from exo_amd.prefix_cache import get_prefix_length
+    assert get_prefix_length(a, b) == want
+
+
+def _filled_cache(n_tokens, seed, layers=2, batch=2, max_seq=32):
+    from exo_amd.cache import ShardKVCache
+    c = ShardKVCache(layers, batch, 2, 8, max_seq, "cpu")
+    g = torch.Generator().manual_seed(seed)
+    for t in c.k + c.v:
+        t.copy_(torch.randn(t.shape, generator=g).bfloat16())
+    c.offsets[0] = n_tokens
+    c.sync_pos()
+    return c
+
+
+def test_prefix_cache_store_fetch_and_isolation():
+    """Exact hit leaves the last token(s) to feed, a partial hit the unmatched suffix,
+    and the stored entry is a detached copy (test_kv_prefix_cache.py:161-201,253-298)."""
+    from exo_amd.prefix_cache import KVPrefixCache, cache_length
+    pc = KVPrefixCache(None)
+    assert len(pc.prompts) == 0 and len(pc.caches) == 0
+    prompt = list(range(100, 112))                      # 12 tokens, 10 of them cached
+    src = _filled_cache(10, seed=1)
+    pc.add_kv_cache(prompt, src, row=0, prefill_tps=123.0)
+    assert len(pc.prompts) == 1 and cache_length(pc.caches[0]) == 10
+    want_k = src.k[1][0, :, :10].clone()
+    src.k[1].zero_()                                    # the live cache moves on
+    dst = _filled_cache(0, seed=2)
+    _, remaining, idx, exact = pc.get_kv_cache(dst, prompt, row=1)
+    assert idx == 0 and exact and remaining == prompt[-2:] and dst.offsets[1] == 10
+    assert torch.equal(dst.k[1][1, :, :10], want_k)
+    assert dst.pos.tolist() == [0, 10]
+    # a stored entry longer than the query is cut back to len-1
+    _, remaining, idx, exact = pc.get_kv_cache(dst, prompt[:6], row=1)
+    assert exact and remaining == prompt[5:6] and dst.offsets[1] == 5
+    # partial hit: 7 common tokens
+    other = prompt[:7] + [1, 2, 3, 4]
+    _, remaining, idx, exact = pc.get_kv_cache(dst, other, row=0)
+    assert idx == 0 and not exact and remaining == [1, 2, 3, 4] and dst.offsets[0] == 7
+    dst.k[0][0].zero_()                                 # generation mutates the row, not the entry
+    assert cache_length(pc.caches[0]) == 10 and torch.equal(pc.caches[0].layers[1][0], want_k)
+    # no common prefix: the row is reset
+    _, remaining, idx, exact = pc.get_kv_cache(dst, [9, 9, 9], row=0)
+    assert idx is None and not exact and remaining == [9, 9, 9] and dst.offsets[0] == 0
+    pc.clear()
+    assert len(pc.prompts) == 0 and len(pc.caches) == 0
+
+
+def test_prefix_cache_update_in_place_rule(monkeypatch):
+    """generator/batch_generate.py:493-535: a hit of >= min length and >= half the prompt
+    replaces the matched entry, anything else adds one."""
+    import exo_amd.prefix_cache as P
+    from exo_amd.prefix_cache import KVPrefixCache, cache_length, save_prefix_cache
+    monkeypatch.setattr(P, "get_memory_used_percentage", lambda device=None: 0.1)
+    monkeypatch.setenv("EXO_MEMORY_THRESHOLD", "0.9")
+    pc = KVPrefixCache(None)
+    c = _filled_cache(10, seed=3)
+    save_prefix_cache(pc, list(range(12)), c, 0, 0, None, min_prefix_hit_length=4)
+    c.offsets[0] = 18
+    save_prefix_cache(pc, list(range(20)), c, 0, 10, 0, min_prefix_hit_length=4)
+    assert len(pc.prompts) == 1 and cache_length(pc.caches[0]) == 18 and len(pc.prompts[0]) == 20
+    save_prefix_cache(pc, list(range(3)) + [77] * 9, c, 0, 3, 0, min_prefix_hit_length=4)
+    assert len(pc.prompts) == 2
+    save_prefix_cache(pc, list(range(5)) + [78] * 9, c, 0, 5, 0, min_prefix_hit_length=4)
+    assert len(pc.prompts) == 3                          # long enough, but under half the prompt
+
+
+def test_prefix_cache_evicts_lru_under_memory_pressure(monkeypatch):
+    """test_kv_prefix_cache.py:534-602: with usage pinned above the threshold every old
+    entry goes, least recently used first, and only the new one survives."""
+    import exo_amd.prefix_cache as P
+    monkeypatch.setenv("EXO_MEMORY_THRESHOLD", "0.9")
+    usage = {"v": 0.5}
+    monkeypatch.setattr(P, "get_memory_used_percentage", lambda device=None: usage["v"])
+    pc = P.KVPrefixCache(None)
+    for i in range(3):
+        pc.add_kv_cache([i, i, i], _filled_cache(3, seed=i))
+        pc._last_used[i] = float(i)
+    pc._last_used[2] = 100.0
+    assert len(pc.prompts) == 3
+    order = []
+    usage["v"] = 0.95
+    # record which prompts leave, in order
+    class Spy(list):
+        def pop(self, i):
+            order.append(int(self[i][0]))
+            return super().pop(i)
+    pc.prompts = Spy(pc.prompts)
+    pc.add_kv_cache([7, 7, 7, 7], _filled_cache(4, seed=9))
+    assert order == [0, 1, 2]
+    assert len(pc.prompts) == 1 and P.get_prefix_length(pc.prompts[0], [7, 7, 7, 7]) == 4
