@@ -30,7 +30,7 @@ from .cache import ShardKVCache
 from .config import ModelConfig
 from .generate import (
     DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, ban_token_ids, extract_top_logprobs,
-    make_sampler, prefill,
+    make_sampler, prefill, processors_for,
 )
 from .loader import load_shard_weights
 from .model import ShardModel
@@ -191,7 +191,7 @@ class ShardBatchGenerator:
                        logits="none", rows=slice(row, row + 1))
         gen = torch.Generator(device=self.model.device)
         gen.manual_seed(task_params.seed or 42)
-        processors = [ban_token_ids(self._eos())] if task_params.bench and self._eos() else []
+        processors = processors_for(task_params, self._eos())
         temp = task_params.temperature if task_params.temperature is not None else 0.7
         seq = _Seq(
             uid=self._next_uid, params=task_params, prompt_tokens=toks,

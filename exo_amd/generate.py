@@ -77,6 +77,79 @@ def ban_token_ids(token_ids: list[int]) -> Callable[[torch.Tensor, torch.Tensor]
     return proc
 
 
+def make_logits_processors(repetition_penalty: float | None = None,
+                           repetition_context_size: int | None = 20,
+                           presence_penalty: float | None = None,
+                           presence_context_size: int | None = 20,
+                           frequency_penalty: float | None = None,
+                           frequency_context_size: int | None = 20,
+                           ) -> list[Callable[[torch.Tensor, torch.Tensor], torch.Tensor]]:
+    """mlx_lm ``make_logits_processors`` (.typings/mlx_lm/sample_utils.pyi:47-72) as the
+    reference calls it (generate.py:599-608): each processor maps (tokens so far,
+    logits [1,V]) to logits.  Definitions as commonly stated, the library's source not
+    being at hand: repetition divides the positive / multiplies the negative logits of
+    the tokens seen in the last ``context`` positions by the penalty; presence subtracts
+    the penalty once from each token seen there; frequency subtracts it once per
+    occurrence.  A penalty of None or 0 adds no processor."""
+    procs: list[Callable[[torch.Tensor, torch.Tensor], torch.Tensor]] = []
+
+    def context(tokens: torch.Tensor, size: int | None, device) -> torch.Tensor:
+        t = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1)
+        if size is not None:
+            t = t[-size:] if size > 0 else t[:0]
+        return t.to(device)
+
+    if repetition_penalty is not None and repetition_penalty != 0:
+        if repetition_penalty < 0:
+            raise ValueError("repetition_penalty must be a non-negative float")
+
+        def repetition(tokens, logits):
+            ctx = context(tokens, repetition_context_size, logits.device)
+            if ctx.numel() == 0:
+                return logits
+            logits = logits.clone()
+            sel = logits[..., ctx]
+            logits[..., ctx] = torch.where(sel < 0, sel * repetition_penalty, sel / repetition_penalty)
+            return logits
+
+        procs.append(repetition)
+    if presence_penalty:
+        def presence(tokens, logits):
+            ctx = torch.unique(context(tokens, presence_context_size, logits.device))
+            if ctx.numel() == 0:
+                return logits
+            logits = logits.clone()
+            logits[..., ctx] -= presence_penalty
+            return logits
+
+        procs.append(presence)
+    if frequency_penalty:
+        def frequency(tokens, logits):
+            ctx = context(tokens, frequency_context_size, logits.device)
+            if ctx.numel() == 0:
+                return logits
+            counts = torch.zeros(logits.shape[-1], dtype=logits.dtype, device=logits.device)
+            counts.index_add_(0, ctx, torch.ones(ctx.numel(), dtype=logits.dtype, device=logits.device))
+            return logits - frequency_penalty * counts
+
+        procs.append(frequency)
+    return procs
+
+
+def processors_for(task: TextGenerationTaskParams, eos_token_ids) -> list:
+    """Processor list of one request: the penalties of its parameters, preceded in bench
+    mode by the EOS ban so that exactly max_tokens are produced (generate.py:599-612)."""
+    procs = make_logits_processors(
+        repetition_penalty=task.repetition_penalty,
+        repetition_context_size=task.repetition_context_size
+        if task.repetition_context_size is not None else 20,
+        presence_penalty=task.presence_penalty, frequency_penalty=task.frequency_penalty)
+    eos = list(eos_token_ids or [])
+    if task.bench and eos:
+        procs = [ban_token_ids(eos)] + procs
+    return procs
+
+
 def extract_top_logprobs(logprobs: torch.Tensor, tokenizer, top_logprobs: int,
                          selected_token: int) -> tuple[float, list[TopLogprobItem]]:
     """generate.py:483-529: the selected token's logprob and the k most likely tokens,
@@ -154,9 +227,7 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     torch.cuda.reset_peak_memory_stats(model.device)
 
     eos = list(eos_token_ids or [])
-    processors = []
-    if task.bench:
-        processors.append(ban_token_ids(eos))  # bench: exactly max_tokens are produced
+    processors = processors_for(task, eos)
     sampler = make_sampler(
         temp=task.temperature if task.temperature is not None else 0.7,
         top_p=task.top_p if task.top_p is not None else 1.0,

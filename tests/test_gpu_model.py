@@ -6,7 +6,8 @@ import pytest
 import torch
 
 from oracle import models as OM
-from tests.util import assert_close, assert_close_stat, load_checkpoint_numpy, n_f32, rng, tiny_config, t_bf16
+from tests.util import (assert_close, assert_close_stat, check_tokens as _check_tokens,
+                        load_checkpoint_numpy, n_f32, rng, tiny_config, t_bf16)
 
 pytestmark = pytest.mark.gpu
 
@@ -43,28 +44,6 @@ def ckpt(request, tmp_path_factory, device):
     # multiplies by bf16-rounded weights; the oracle mirrors that arithmetic mode.
     return dict(cfg=cfg, path=path, oracle=OM.ShardModel(ocfg, ow, gemm_rows=16),
                 model=ShardModel(cfg, w, device=device), ocfg=ocfg, ow=ow, w=w)
-
-
-def _check_tokens(got, want, om, what):
-    """Per-token statistical parity.  For MoE models a token whose k-th and (k+1)-th
-    router logits are within bf16 noise may legitimately pick another expert; such
-    tokens (and later ones, through the KV cache) are exempt when the oracle's router
-    gap shows the near-tie."""
-    got, want = got.reshape(-1, got.shape[-1]), want.reshape(-1, want.shape[-1])
-    gaps = None
-    if om.router_margins:
-        T = want.shape[0]
-        gaps = np.min(np.stack([g[-T:] for _, g in om.router_margins[-om.n_local_layers:]]), axis=0)
-    tied_before = False
-    for t in range(want.shape[0]):
-        rms = float(np.sqrt(np.mean(want[t] ** 2)))
-        rel = float(np.sqrt(np.mean((got[t] - want[t]) ** 2))) / rms
-        if gaps is not None and gaps[t] <= 2.0 ** -6 * max(1.0, rms):
-            tied_before = True
-        if rel > 2e-2:
-            assert tied_before, f"{what}: token {t} rel-rms {rel:.3e} with no router near-tie"
-            print(f"[parity] {what}: token {t} rel-rms {rel:.3e} after a router near-tie (exempt)")
-    return tied_before
 
 
 def test_prefill_and_decode_logits_match_oracle(ckpt, device):

@@ -409,3 +409,27 @@ def test_prefix_cache_evicts_lru_under_memory_pressure(monkeypatch):
     pc.add_kv_cache([7, 7, 7, 7], _filled_cache(4, seed=9))
     assert order == [0, 1, 2]
     assert len(pc.prompts) == 1 and P.get_prefix_length(pc.prompts[0], [7, 7, 7, 7]) == 4
+
+
+def test_logits_processors():
+    """Penalties as the reference requests them (generator/generate.py:599-612), checked
+    on values worked by hand."""
+    from exo_amd.generate import make_logits_processors, processors_for
+    logits = torch.tensor([[2.0, -2.0, 1.0, 0.5, -1.0]])
+    assert make_logits_processors() == []
+    assert make_logits_processors(repetition_penalty=0.0, presence_penalty=0.0, frequency_penalty=None) == []
+    (rep,) = make_logits_processors(repetition_penalty=2.0, repetition_context_size=3)
+    # context = last three tokens {1, 0, 1}; token 4 is older than the window
+    out = rep(torch.tensor([4, 1, 0, 1]), logits)
+    assert out.tolist() == [[1.0, -4.0, 1.0, 0.5, -1.0]] and logits[0, 0] == 2.0  # input untouched
+    (pres,) = make_logits_processors(presence_penalty=0.5)
+    assert pres(torch.tensor([2, 2, 3]), logits).tolist() == [[2.0, -2.0, 0.5, 0.0, -1.0]]
+    (freq,) = make_logits_processors(frequency_penalty=0.25)
+    assert freq(torch.tensor([2, 2, 3]), logits).tolist() == [[2.0, -2.0, 0.5, 0.25, -1.0]]
+    assert rep(torch.tensor([], dtype=torch.int64), logits) is logits
+    with pytest.raises(ValueError):
+        make_logits_processors(repetition_penalty=-1.0)
+    p = TextGenerationTaskParams(model="m", bench=True, repetition_penalty=1.1, frequency_penalty=0.1)
+    procs = processors_for(p, [3])
+    assert len(procs) == 3 and procs[0](None, logits)[0, 3] == -1e9
+    assert processors_for(TextGenerationTaskParams(model="m", bench=True), []) == []
