@@ -903,23 +903,25 @@ extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* sca
                       stream);
 }
 
-extern "C" int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps,
-                            const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                            const uint16_t* residual, uint16_t* y, int M, int N, int K,
-                            int bits, int group_size, exo_stream_t stream) {
+static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                         const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                         const uint16_t* residual, uint16_t* y, void* workspace, int M, int N,
+                         int K, int bits, int group_size, exo_stream_t stream) {
   int rc = check_common("exo_qmv", M, N, K, bits, group_size);
   if (rc) return rc;
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmv: null pointer");
   if (M == 0) return EXO_OK;
   // two or more rows: the matrix-core GEMV streams W once per tile of up to 16 rows
-  const int cap = M >= 2 ? exo_qmv_mfma_max_rows(K, bits) : 0;
+  // (with a workspace; without one a tile is as many rows as the LDS holds whole)
+  int cap = M >= 2 ? exo_qmv_mfma_max_rows(K, bits) : 0;
+  if (cap > 0 && workspace) cap = 16;
   if (cap >= 2) {
     int m0 = 0;
     while (M - m0 >= 2) {
       const int mt = (M - m0 < cap) ? (M - m0) : cap;
       rc = exo_qmv_mfma_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases,
                                residual ? residual + (size_t)m0 * N : nullptr, y + (size_t)m0 * N,
-                               mt, N, K, bits, (hipStream_t)stream);
+                               mt, N, K, bits, workspace, (hipStream_t)stream);
       if (rc) return rc;
       m0 += mt;
     }
@@ -938,6 +940,31 @@ extern "C" int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, floa
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_qmv");
   return EXO_OK;
+}
+
+extern "C" int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                            const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* residual, uint16_t* y, int M, int N, int K,
+                            int bits, int group_size, exo_stream_t stream) {
+  return norm_qmv_impl(x, norm_weight, eps, w, scales, biases, residual, y, nullptr, M, N, K,
+                       bits, group_size, stream);
+}
+
+extern "C" int64_t exo_qmv_workspace(int N) {
+  return N > 0 ? (int64_t)exo_qmv_mfma_workspace(N) : 0;
+}
+
+extern "C" int exo_norm_qmv_ws(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                               const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, const uint16_t* residual, uint16_t* y,
+                               void* workspace, int64_t workspace_bytes, int M, int N, int K,
+                               int bits, int group_size, exo_stream_t stream) {
+  EXO_REQUIRE(!workspace || (workspace_bytes >= exo_qmv_workspace(N) &&
+                             ((uintptr_t)workspace & 255) == 0),
+              "exo_norm_qmv_ws: workspace of %lld bytes, need %lld (256-byte aligned)",
+              (long long)workspace_bytes, (long long)exo_qmv_workspace(N));
+  return norm_qmv_impl(x, norm_weight, eps, w, scales, biases, residual, y, workspace, M, N, K,
+                       bits, group_size, stream);
 }
 
 extern "C" int exo_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,

@@ -12,17 +12,19 @@
 //  * D[m][r] of a whole group is scaled on the way out:
 //      acc += s[r,g] * (D - 128*Sx[m,g]) + b[r,g] * Sx[m,g]
 //    with the group sums Sx of the activations precomputed in LDS;
-//  * the four waves of a workgroup split K, so that 32 rows already occupy a whole CU;
-//    partial sums meet in LDS once per 32-row block.
+//  * four waves split the K range of one block of 32 rows; their partial sums meet in
+//    LDS once per block.  A workgroup holds NG such wave quartets, which share the
+//    staged activations (the staging cost per weight byte falls with NG);
+//  * with a workspace, K is also split over workgroups (blockIdx.y): 16 rows then fit
+//    the LDS at any K and a short N still fills the chip; the last workgroup of a row
+//    block to arrive adds the float32 partials in a fixed order.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 #include "qmv_internal.h"
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
-constexpr int kStepsPerSuper = 8;  // 16-byte loads in flight per lane and buffer
+constexpr int kWaves = 4;  // waves that share one block of 32 output rows (they split K)
 
 struct MfmaParams {
   const bf16_t* x;         // [M,K]
@@ -35,7 +37,18 @@ struct MfmaParams {
   float eps;
   int M, N, K, wpr, G;
   int gw;  // groups per wave (multiple of the groups per super-step)
+  // split-K: blockIdx.y owns groups [y*gc, (y+1)*gc); partial sums meet in `part`
+  int ksplit, gc;
+  float* part;    // [ksplit][M][N] float32
+  int* counters;  // [row blocks], zero between launches
 };
+
+__device__ __forceinline__ void st_dev(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_dev(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <int BITS>
 __device__ __forceinline__ uint4 load_word_x(const bf16_t* base, int wi) {
@@ -86,28 +99,86 @@ __device__ __forceinline__ uint4 permute_word(const uint4& xv, float& stored, fl
   return o;
 }
 
-// MR = D registers in use: 4 covers M <= 8, 8 covers M <= 16.
-template <int BITS, int MR>
-__global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) {
-  constexpr int WPG = 64 * BITS / 32;          // words per group: 8 / 16
-  constexpr int SPG = WPG / 8;                  // load steps per group: 1 / 2
-  constexpr int SSG = kStepsPerSuper / SPG;     // groups per super-step: 8 / 4
+// MR = D registers in use: 4 covers M <= 8, 8 covers M <= 16.  NG = wave quartets per
+// workgroup.  SPS = 16-byte loads in flight per lane and buffer (a "super-step").
+template <int BITS, int MR, int NG, int SPS>
+__global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) {
+  constexpr int kThreads = 256 * NG;
+  constexpr int WPG = 64 * BITS / 32;  // words per group: 8 / 16
+  constexpr int SPG = WPG / 8;         // load steps per group: 1 / 2
+  constexpr int SSG = SPS / SPG;       // groups per super-step
+  static_assert(SSG >= 2 && SSG <= 8, "scale vector of 2..8 bf16");
   extern __shared__ uint4 smem[];
   const int MT = p.M;
-  uint4* xs = smem;                                            // [wpr/8][4][2][MT]
-  float2* sxs = reinterpret_cast<float2*>(smem + (size_t)p.wpr * MT);  // [G][MT]
-  float* red = reinterpret_cast<float*>(sxs + (size_t)p.G * MT);        // [4][MR][64]
-  __shared__ float s_red[kWaves * 16];
+  // this workgroup's share of K: groups [gbase, gbase+Gc), words [wbase, wbase+wcount)
+  const int gbase = (int)blockIdx.y * p.gc;
+  const int Gc = min(p.gc, p.G - gbase);
+  const int wbase = gbase * WPG, wcount = Gc * WPG;
+  uint4* xs = smem;                                                         // [gc*WPG/8][4][2][MT]
+  float2* sxs = reinterpret_cast<float2*>(smem + (size_t)p.gc * WPG * MT);  // [gc][MT]
+  float* red_all = reinterpret_cast<float*>(sxs + (size_t)p.gc * MT);       // [NG][4][MR][64]
+  __shared__ float s_red[4 * NG * 16];
+  __shared__ float s_inv[16];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int quartet = wave_all >> 2, wave = wave_all & 3;
+  float* red = red_all + quartet * (kWaves * MR * 64);
   const int r = lane & 31, kq = lane >> 5;
+  const int NB = (p.N + 31) >> 5;
+
+  const int g_begin = wave * p.gw;  // this wave's share of the chunk
+  const int g_end = min(Gc, g_begin + p.gw);
+  const int n_super = p.gw / SSG;   // same for every wave of the grid
+
+  struct Buf {
+    uint4 w[SPS];
+    uint4 s, b;  // SSG scales / biases
+  };
+  // item -> (row block, super-step); loads clamp to the last valid row / group
+  auto issue = [&](Buf& bf, int blk, int ss) {
+    const int row = min(blk * 32 + r, p.N - 1);
+    const int g0 = min(g_begin + ss * SSG, Gc - SSG);
+    const uint32_t* wp = p.w + (size_t)row * p.wpr + (size_t)(gbase + g0) * WPG + kq * 4;
+#pragma unroll
+    for (int i = 0; i < SPS; ++i) {
+      // steps past the chunk end re-read its last step (never consumed)
+      const int off = min(i * 8, wcount - g0 * WPG - 8);
+      bf.w[i] = *reinterpret_cast<const uint4*>(wp + off);
+    }
+    const bf16_t* sp = p.s + (size_t)row * p.G + gbase + g0;
+    const bf16_t* bp = p.b + (size_t)row * p.G + gbase + g0;
+    if (SSG == 8) {
+      bf.s = *reinterpret_cast<const uint4*>(sp);
+      bf.b = *reinterpret_cast<const uint4*>(bp);
+    } else if (SSG == 4) {
+      const uint2 sv = *reinterpret_cast<const uint2*>(sp);
+      const uint2 bv = *reinterpret_cast<const uint2*>(bp);
+      bf.s = make_uint4(sv.x, sv.y, 0, 0);
+      bf.b = make_uint4(bv.x, bv.y, 0, 0);
+    } else {
+      bf.s = make_uint4(*reinterpret_cast<const uint32_t*>(sp), 0, 0, 0);
+      bf.b = make_uint4(*reinterpret_cast<const uint32_t*>(bp), 0, 0, 0);
+    }
+  };
+
+  // flat sequence of (row block, super-step) items; the quartets of a workgroup take
+  // neighbouring row blocks and run the same number of items (barriers are block-wide)
+  const int NBq = (NB + NG - 1) / NG;
+  const int my_blocks = (NBq - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int n_items = my_blocks * n_super;
+  if (n_items <= 0) return;
+  auto blk_of = [&](int it) {
+    return ((int)blockIdx.x + (it / n_super) * (int)gridDim.x) * NG + quartet;
+  };
+
+  Buf b0, b1;
+  // weights do not depend on x: in flight while x is staged (where registers allow)
+  constexpr bool kEarly = (MR == 4);
+  if (kEarly) issue(b0, blk_of(0), 0);
 
   // ---- stage the activations: optional RMSNorm, permute, group sums
   {
-    float inv[16];
-#pragma unroll
-    for (int m = 0; m < 16; ++m) inv[m] = 1.f;
     if (p.norm_w) {
       float ss[16];
 #pragma unroll
@@ -120,18 +191,23 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
       for (int m = 0; m < 16; ++m) {
         if (m < MT) {
           const float t = wave_sum(ss[m]);
-          if (lane == 0) s_red[wave * 16 + m] = t;
+          if (lane == 0) s_red[wave_all * 16 + m] = t;
         }
       }
       __syncthreads();
 #pragma unroll
       for (int m = 0; m < 16; ++m)
-        if (m < MT)
-          inv[m] = rsqrtf((s_red[m] + s_red[16 + m] + s_red[32 + m] + s_red[48 + m]) / (float)p.K +
-                          p.eps);
+        if (m < MT) {
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < 4 * NG; ++w) t += s_red[w * 16 + m];
+          if (tid == 0) s_inv[m] = rsqrtf(t / (float)p.K + p.eps);
+        }
+      __syncthreads();
     }
-    for (int wi = tid; wi < p.wpr; wi += kThreads) {
-      const int step = wi >> 3, q2 = (wi >> 2) & 1, t = wi & 3;
+    for (int wl = tid; wl < wcount; wl += kThreads) {
+      const int wi = wbase + wl;
+      const int step = wl >> 3, q2 = (wl >> 2) & 1, t = wl & 3;
       const int dst = ((step * 4 + t) * 2 + q2) * MT;
       uint4 nw = make_uint4(0, 0, 0, 0);
       if (p.norm_w) nw = load_word_x<BITS>(p.norm_w, wi);
@@ -139,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
       for (int m = 0; m < 16; ++m) {
         if (m < MT) {
           uint4 xv = load_word_x<BITS>(p.x + (size_t)m * p.K, wi);
-          if (p.norm_w) norm_word<BITS>(xv, nw, inv[m]);
+          if (p.norm_w) norm_word<BITS>(xv, nw, s_inv[m]);
           float stored, truesum;
           xs[dst + m] = permute_word<BITS>(xv, stored, truesum);
           // sum over the WPG consecutive words (threads) of the group
@@ -148,7 +224,7 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
             stored += __shfl_xor(stored, o, 64);
             truesum += __shfl_xor(truesum, o, 64);
           }
-          if ((wi & (WPG - 1)) == 0) sxs[(wi / WPG) * MT + m] = make_float2(128.f * stored, truesum);
+          if ((wl & (WPG - 1)) == 0) sxs[(wl / WPG) * MT + m] = make_float2(128.f * stored, truesum);
         }
       }
     }
@@ -162,49 +238,17 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
   for (int q = 0; q < MR; ++q) a_of[q] = min(8 * (q >> 2) + 4 * Rg + (q & 3), MT - 1);
   const int a_lane = min(r, MT - 1);  // A-operand row of this lane
 
-  const int NB = (p.N + 31) >> 5;
-  const int g_begin = wave * p.gw;                 // this wave's share of K
-  const int g_end = min(p.G, g_begin + p.gw);
-  const int n_super = p.gw / SSG;                  // same for every wave of the block
-
   uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
   asm volatile("" : "+s"(kmask));
   asm volatile("" : "+v"(kmagic));
 
-  struct Buf {
-    uint4 w[kStepsPerSuper];
-    uint4 s, b;  // SSG scales / biases (8-bit: only .x, .y used)
-  };
-  // item -> (row block, super-step); loads clamp to the last valid row / group
-  auto issue = [&](Buf& bf, int blk, int ss) {
-    const int row = min(blk * 32 + r, p.N - 1);
-    const int g0 = min(g_begin + ss * SSG, p.G - SSG < 0 ? 0 : p.G - SSG);
-    const uint32_t* wp = p.w + (size_t)row * p.wpr + (size_t)g0 * WPG + kq * 4;
-#pragma unroll
-    for (int i = 0; i < kStepsPerSuper; ++i) {
-      // steps past the row end re-read its last step (never consumed)
-      const int off = min(i * 8, p.wpr - g0 * WPG - 8);
-      bf.w[i] = *reinterpret_cast<const uint4*>(wp + off);
-    }
-    const bf16_t* sp = p.s + (size_t)row * p.G + g0;
-    const bf16_t* bp = p.b + (size_t)row * p.G + g0;
-    if (SSG == 8) {
-      bf.s = *reinterpret_cast<const uint4*>(sp);
-      bf.b = *reinterpret_cast<const uint4*>(bp);
-    } else {
-      const uint2 sv = *reinterpret_cast<const uint2*>(sp);
-      const uint2 bv = *reinterpret_cast<const uint2*>(bp);
-      bf.s = make_uint4(sv.x, sv.y, 0, 0);
-      bf.b = make_uint4(bv.x, bv.y, 0, 0);
-    }
-  };
-
   float acc[MR];
 #pragma unroll
   for (int q = 0; q < MR; ++q) acc[q] = 0.f;
+  if (!kEarly) issue(b0, blk_of(0), 0);
 
   auto consume = [&](const Buf& bf, int ss) {
-    const int g0 = min(g_begin + ss * SSG, p.G - SSG < 0 ? 0 : p.G - SSG);
+    const int g0 = min(g_begin + ss * SSG, Gc - SSG);
     const int g_first = g_begin + ss * SSG;  // groups [g_first, g_first+SSG) are due
     const uint32_t* sw = reinterpret_cast<const uint32_t*>(&bf.s);
     const uint32_t* bw = reinterpret_cast<const uint32_t*>(&bf.b);
@@ -246,38 +290,69 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
     }
   };
 
-  // flat sequence of (row block, super-step) items with two buffers in ping-pong
-  const int my_blocks = (NB - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-  const int n_items = my_blocks * n_super;
-  if (n_items <= 0) return;
-  auto blk_of = [&](int it) { return (int)blockIdx.x + (it / n_super) * (int)gridDim.x; };
-
   auto finish_block = [&](int blk) {
-    __syncthreads();  // wave 0 has finished reading the previous block's partials
+    __syncthreads();  // the quartet's first wave has finished reading the previous partials
 #pragma unroll
     for (int q = 0; q < MR; ++q) {
       red[(wave * MR + q) * 64 + lane] = acc[q];
       acc[q] = 0.f;
     }
     __syncthreads();
-    if (wave == 0) {
+    if (wave == 0 && blk < NB) {
       const int row = blk * 32 + r;
+      float v[MR];
 #pragma unroll
-      for (int q = 0; q < MR; ++q) {
-        const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
-        float v = red[q * 64 + lane] + red[(MR + q) * 64 + lane] + red[(2 * MR + q) * 64 + lane] +
-                  red[(3 * MR + q) * 64 + lane];
-        if (m < p.M && row < p.N) {
-          const size_t o = (size_t)m * p.N + row;
-          if (p.residual) v = bf2f(f2bf(v)) + bf2f(p.residual[o]);
-          p.y[o] = f2bf(v);
+      for (int q = 0; q < MR; ++q)
+        v[q] = red[q * 64 + lane] + red[(MR + q) * 64 + lane] + red[(2 * MR + q) * 64 + lane] +
+               red[(3 * MR + q) * 64 + lane];
+      bool write = true;
+      if (p.ksplit > 1) {
+        // partial sums go out at device scope (the merging workgroup may sit on another
+        // XCD); the last of the ksplit workgroups of this row block adds them up in a
+        // fixed order, so the result does not depend on arrival order
+#pragma unroll
+        for (int q = 0; q < MR; ++q) {
+          const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
+          if (m < p.M && row < p.N)
+            st_dev(&p.part[((size_t)blockIdx.y * p.M + m) * p.N + row], v[q]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        int last = 0;
+        if (lane == 0) {
+          const int old = __hip_atomic_fetch_add(&p.counters[blk], 1, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+          last = (old == p.ksplit - 1);
+          if (last)
+            __hip_atomic_store(&p.counters[blk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        write = __builtin_amdgcn_readfirstlane(last) != 0;
+        if (write) {
+#pragma unroll
+          for (int q = 0; q < MR; ++q) {
+            const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
+            float t = 0.f;
+            if (m < p.M && row < p.N)
+              for (int ks = 0; ks < p.ksplit; ++ks)
+                t += ld_dev(&p.part[((size_t)ks * p.M + m) * p.N + row]);
+            v[q] = t;
+          }
+        }
+      }
+      if (write) {
+#pragma unroll
+        for (int q = 0; q < MR; ++q) {
+          const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
+          if (m < p.M && row < p.N) {
+            const size_t o = (size_t)m * p.N + row;
+            float t = v[q];
+            if (p.residual) t = bf2f(f2bf(t)) + bf2f(p.residual[o]);
+            p.y[o] = f2bf(t);
+          }
         }
       }
     }
   };
 
-  Buf b0, b1;
-  issue(b0, blk_of(0), 0);
   int it = 0;
   for (;;) {
     if (it + 1 < n_items) issue(b1, blk_of(it + 1), (it + 1) % n_super);
@@ -291,41 +366,64 @@ __global__ __launch_bounds__(kThreads) void qmv_mfma_kernel(const MfmaParams p) 
   }
 }
 
-template <int BITS, int MR>
+template <int BITS, int MR, int NG, int SPS>
 int launch(const MfmaParams& p, size_t lds, hipStream_t st) {
-  auto kern = qmv_mfma_kernel<BITS, MR>;
+  auto kern = qmv_mfma_kernel<BITS, MR, NG, SPS>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048);
     if (e != hipSuccess) {
       exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
       return EXO_ERR_HIP;
     }
     attr_done = true;
   }
-  const int NB = (p.N + 31) / 32;
-  const int per_cu = lds <= 72 * 1024 ? 2 : 1;
-  int grid = NB < 256 * per_cu ? NB : 256 * per_cu;
-  kern<<<dim3(grid), dim3(kThreads), lds, st>>>(p);
+  const int NBq = ((p.N + 31) / 32 + NG - 1) / NG;
+  int per_cu = lds <= 38 * 1024 ? 4 : (lds <= 51 * 1024 ? 3 : (lds <= 78 * 1024 ? 2 : 1));
+  if (per_cu * NG > 4) per_cu = 4 / NG;  // at most 16 waves per CU
+  if (per_cu < 1) per_cu = 1;
+  int gx = 256 * per_cu / p.ksplit;
+  if (gx < 1) gx = 1;
+  if (gx > NBq) gx = NBq;
+  kern<<<dim3(gx, p.ksplit), dim3(256 * NG), lds, st>>>(p);
   return EXO_OK;
+}
+
+constexpr int kMaxSplit = 8;
+constexpr size_t kLdsBudget = 150 * 1024;
+
+size_t lds_bytes(int M, int gc, int bits, int MR, int NG) {
+  const size_t wpg = 64 * bits / 32;
+  return (size_t)gc * wpg * 16 * M + (size_t)gc * 8 * M + (size_t)NG * kWaves * MR * 64 * 4;
 }
 
 }  // namespace
 
-// rows of x that fit one launch (LDS holds their whole K), 0 if not even one
+// rows of x that fit one launch without split-K (LDS holds their whole K), 0 if the
+// kernel does not take this K at all
 int exo_qmv_mfma_max_rows(int K, int bits) {
   if (K % (bits == 4 ? 512 : 256) != 0) return 0;
   const size_t per_row = (size_t)K * bits / 32 * 16 + (size_t)(K / 64) * 8;
-  const size_t budget = 150 * 1024 - kWaves * 8 * 64 * 4;
+  const size_t budget = kLdsBudget - 4 * kWaves * 8 * 64 * 4;
   size_t m = budget / per_row;
   return m > 16 ? 16 : (int)m;
 }
 
-// y[M,N] for 2 <= M <= exo_qmv_mfma_max_rows(K, bits)
+// bytes of split-K workspace for up to 16 rows: row-block counters, then the partials.
+// The counter area has one size for every N, so that partials of one launch never land
+// where another launch (of another N, sharing the workspace) keeps its counters.
+constexpr size_t kCounterBytes = 64 * 1024;
+size_t exo_qmv_mfma_workspace(int N) {
+  return kCounterBytes + (size_t)kMaxSplit * 16 * N * 4;
+}
+
+// y[M,N] for 2 <= M <= 16.  Without a workspace M must not exceed
+// exo_qmv_mfma_max_rows(K, bits); with one, K may be split over up to kMaxSplit workgroups
+// per row block so that any M <= 16 fits and a short N still fills the chip.
 int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
                         const bf16_t* s, const bf16_t* b, const bf16_t* residual, bf16_t* y,
-                        int M, int N, int K, int bits, hipStream_t st) {
+                        int M, int N, int K, int bits, void* workspace, hipStream_t st) {
   MfmaParams p;
   p.x = x;
   p.w = w;
@@ -340,13 +438,52 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   p.K = K;
   p.wpr = K * bits / 32;
   p.G = K / 64;
-  const int ssg = bits == 4 ? 8 : 4;
-  int gw = (p.G + kWaves - 1) / kWaves;
-  gw = (gw + ssg - 1) / ssg * ssg;
-  p.gw = gw;
   const int MR = M <= 8 ? 4 : 8;
-  const size_t lds = (size_t)p.wpr * 16 * M + (size_t)p.G * 8 * M + (size_t)kWaves * MR * 64 * 4;
-  if (bits == 4)
-    return MR == 4 ? launch<4, 4>(p, lds, st) : launch<4, 8>(p, lds, st);
-  return MR == 4 ? launch<8, 4>(p, lds, st) : launch<8, 8>(p, lds, st);
+  const int NB = (N + 31) / 32;
+  // many row blocks: quartets share the staged x (2 for up to 8 rows, 4 for up to 16);
+  // few: one quartet per workgroup so that the grid stays wide
+  const int NG = NB >= 1024 ? (MR == 8 ? 3 : (M > 4 ? 2 : 1)) : 1;
+  const int sps = 4;
+  const int ssg = sps / (bits == 4 ? 1 : 2);
+  const int unit = kWaves * ssg;  // groups per chunk come in whole super-steps per wave
+  const int NBq = (NB + NG - 1) / NG;
+  int ksplit = 1;
+  if (workspace && (size_t)NB * 4 > kCounterBytes) workspace = nullptr;  // N beyond 524288
+  if (workspace) {
+    // split K until a chunk of x fits the LDS with two workgroups per CU, and further
+    // while the grid is narrower than the chip; a chunk is at least one super-step per wave
+    while (ksplit < kMaxSplit && (p.G + ksplit - 1) / ksplit > unit &&
+           (lds_bytes(M, (p.G + ksplit - 1) / ksplit, bits, MR, NG) > (NG == 1 ? 78u : 150u) * 1024 ||
+            NBq * ksplit < 256))
+      ++ksplit;
+  }
+  int gc = (p.G + ksplit - 1) / ksplit;
+  gc = (gc + unit - 1) / unit * unit;
+  if (gc > p.G) gc = p.G;
+  ksplit = (p.G + gc - 1) / gc;
+  p.ksplit = ksplit;
+  p.gc = gc;
+  int gw = (gc + kWaves - 1) / kWaves;
+  p.gw = (gw + ssg - 1) / ssg * ssg;
+  p.counters = reinterpret_cast<int*>(workspace);
+  p.part = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes)
+                     : nullptr;
+  const size_t lds = lds_bytes(M, gc, bits, MR, NG);
+  if (lds > kLdsBudget) {
+    exo_set_error("exo_qmv: %d rows of K=%d need %zu bytes of LDS", M, K, lds);
+    return EXO_ERR_ARG;
+  }
+#define EXO_MFMA_CASE(B_, MR_, NG_, SPS_) \
+  if (bits == B_ && MR == MR_ && NG == NG_) return launch<B_, MR_, NG_, SPS_>(p, lds, st);
+  EXO_MFMA_CASE(4, 4, 1, 4)
+  EXO_MFMA_CASE(4, 4, 2, 4)
+  EXO_MFMA_CASE(4, 8, 1, 4)
+  EXO_MFMA_CASE(4, 8, 3, 4)
+  EXO_MFMA_CASE(8, 4, 1, 4)
+  EXO_MFMA_CASE(8, 4, 2, 4)
+  EXO_MFMA_CASE(8, 8, 1, 4)
+  EXO_MFMA_CASE(8, 8, 3, 4)
+#undef EXO_MFMA_CASE
+  exo_set_error("exo_qmv: no kernel for bits=%d rows=%d", bits, M);
+  return EXO_ERR_ARG;
 }

@@ -130,6 +130,24 @@ def embed(ids: torch.Tensor, qw: QuantizedWeight, out: torch.Tensor | None = Non
 QMV_MAX_M = 16
 
 
+_QMV_WS: dict = {}
+
+
+def qmv_workspace(N: int, device) -> torch.Tensor:
+    """Split-K workspace for the 2..16-row GEMV, one per device (this engine issues all
+    its work in stream order), grown to the largest N seen.  A replaced buffer stays
+    alive: a captured graph may still point at it.  Zeroed once; the kernel leaves its
+    counters zero."""
+    key = torch.device(device).index or 0
+    need = native.load().exo_qmv_workspace(N)
+    cur = _QMV_WS.get(key)
+    if cur is None or cur[-1].numel() < need:
+        buf = torch.zeros(need, dtype=torch.uint8, device=device)
+        _QMV_WS.setdefault(key, []).append(buf)
+        cur = _QMV_WS[key]
+    return cur[-1]
+
+
 def quantized_matmul(
     x: torch.Tensor,
     qw: QuantizedWeight,
@@ -149,9 +167,20 @@ def quantized_matmul(
         raise ValueError(f"quantized_matmul: x has K={K}, weight has K={qw.K}")
     if out is None:
         out = torch.empty(M, qw.N, dtype=torch.bfloat16, device=x.device)
+    if norm_weight is not None and M > QMV_MAX_M:
+        raise ValueError("fused rms_norm is only available on the GEMV path (M <= 16)")
+    if 2 <= M <= QMV_MAX_M:
+        ws = qmv_workspace(qw.N, x.device)
+        check(
+            lib.exo_norm_qmv_ws(
+                _ptr(x), _ptr(norm_weight), eps, _ptr(qw.weight), _ptr(qw.scales),
+                _ptr(qw.biases), _ptr(residual), _ptr(out), _ptr(ws), ws.numel(), M, qw.N, K,
+                qw.bits, qw.group_size, _stream(),
+            ),
+            "quantized_matmul(rows 2..16)",
+        )
+        return out
     if norm_weight is not None:
-        if M > QMV_MAX_M:
-            raise ValueError("fused rms_norm is only available on the GEMV path (M <= 16)")
         check(
             lib.exo_norm_qmv(
                 _ptr(x), _ptr(norm_weight), eps, _ptr(qw.weight), _ptr(qw.scales),

@@ -72,6 +72,20 @@ int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps, cons
                  const uint16_t* scales, const uint16_t* biases, const uint16_t* residual,
                  uint16_t* y, int M, int N, int K, int bits, int group_size,
                  exo_stream_t stream);
+
+/* K1 with a workspace for 2 <= M <= 16 rows per tile: K is split over several workgroups
+ * per block of 32 output rows and the float32 partial sums meet in `workspace`, so that 16
+ * rows fit the LDS at any K and a small N still fills the chip.  exo_qmv_workspace(N)
+ * bytes, 256-byte aligned; its first 64 KiB are arrival counters, which the caller zeroes
+ * once (every launch leaves them zero; one workspace serves launches of any N up to the N
+ * it was sized for).  Launches that share a workspace must be ordered
+ * on one stream.  workspace == NULL behaves like exo_norm_qmv.  M == 1 never touches it. */
+int64_t exo_qmv_workspace(int N);
+int exo_norm_qmv_ws(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                    const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                    const uint16_t* residual, uint16_t* y, void* workspace,
+                    int64_t workspace_bytes, int M, int N, int K, int bits, int group_size,
+                    exo_stream_t stream);
 int exo_norm_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float eps,
                         const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
                         const uint32_t* wu, const uint16_t* su, const uint16_t* bu, uint16_t* y,

@@ -392,3 +392,18 @@ def test_kv_wire_argument_errors(device):
         ops.kv_import_nhd(torch.zeros(3, 2, 4, dtype=torch.bfloat16, device=device), row, 0)
     with pytest.raises(ValueError):
         ops.kv_export_nhd(torch.zeros(2, 16, 12, dtype=torch.bfloat16, device=device), 0, 1)
+
+
+def test_qmv_workspace_shared_by_launches_of_different_shapes(device):
+    """The split-K workspace is shared by all 2..16-row GEMVs of a device: a launch with a
+    short N must not leave anything where a later launch with more row blocks keeps its
+    arrival counters (the partial sums sit behind a counter area of fixed size)."""
+    for bits, M, N, K in [(4, 3, 128, 4096), (4, 16, 4096, 14336), (8, 5, 64, 2048), (8, 8, 4096, 14336),
+                          (4, 16, 4096, 14336)]:
+        trip = rand_quantized(64, K, bits, seed=N + K + bits)
+        reps = N // 64
+        trip = tuple(np.concatenate([t] * reps) for t in trip)  # N rows from 64 distinct ones
+        x = rand_bf16((M, K), seed=M + K)
+        got = n_f32(ops.quantized_matmul(t_bf16(x, device), t_qw(trip, bits, device)))
+        want = np.tile(affine.qmm(x, *(t[:64] for t in trip), 64, bits), (1, reps))
+        assert_close(got, want, what=f"qmv {M}x{N}x{K} b{bits}")
