@@ -16,6 +16,7 @@
 //          writes the output directly.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
+#include "sdpa_internal.h"
 
 namespace {
 
@@ -419,6 +420,10 @@ int launch_sdpa(const SdpaParams& p, hipStream_t st) {
   return EXO_OK;
 }
 
+// chunks of at least this many tokens take the matrix-core kernel; shorter ones the
+// one-workgroup-per-token kernel below
+constexpr int kMfmaPrefillMinT = 8;
+
 int check(const char* name, int B, int T, int Hq, int Hkv, int D, int S_max) {
   EXO_REQUIRE(B > 0 && T > 0 && Hq > 0 && Hkv > 0 && S_max > 0, "%s: non-positive size", name);
   EXO_REQUIRE(Hq % Hkv == 0, "%s: Hq=%d not a multiple of Hkv=%d", name, Hq, Hkv);
@@ -505,6 +510,13 @@ extern "C" int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache,
   int rc = check("exo_sdpa_prefill", B, T, Hq, Hkv, D, S_max);
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out, "exo_sdpa_prefill: null pointer");
+  if (T >= kMfmaPrefillMinT) {
+    rc = exo_sdpa_prefill_mfma(q, k_cache, v_cache, pos, out, scale, B, T, Hq, Hkv, D, S_max,
+                               (hipStream_t)stream);
+    if (rc) return rc;
+    EXO_CHECK_LAUNCH("exo_sdpa_prefill");
+    return EXO_OK;
+  }
   SdpaParams p{q, k_cache, v_cache, pos, out, nullptr, nullptr, scale, B, T, Hq, Hkv, S_max, 1,
                nullptr, nullptr, nullptr, nullptr, nullptr, 0.f};
   rc = (D == 64) ? launch_sdpa<64, 0>(p, (hipStream_t)stream)

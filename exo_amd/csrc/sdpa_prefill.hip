@@ -1,0 +1,236 @@
+// Causal attention for a chunk of T new tokens (prefill) on the matrix cores.
+//
+// Flash-attention recurrence with both products on v_mfma_f32_32x32x16_bf16, written
+// transposed so that every per-query quantity (running max, sum, rescale factor) is a
+// per-LANE scalar:
+//   S^T[key][query] = K . Q^T          A = K rows from LDS,      B = Q^T from registers
+//   O^T[d][query]  += V^T . P^T        A = V^T rows from LDS,    B = P^T = the S^T registers
+// The D-operand layout of the first product puts, in lane (query, half), registers that
+// are 8 consecutive keys per 16-key step once the K rows are fed in a permuted order;
+// they are rounded to bf16 and used as the B operand of the second product without any
+// data movement.  V is transposed on its way into LDS (2-byte stores), K goes in as is.
+//
+// Work split: a wave owns 32 query tokens of ONE query head; the four waves of a
+// workgroup take four consecutive (token tile, head) units of one kv head, so with GQA
+// (4, 8, 16 query heads per kv head) they share every K/V tile they stage.  Key tiles of
+// 64; the next tile's global loads are in flight while the current one is computed.
+#include "../../include/exo_mi355x.h"
+#include "common.h"
+#include "sdpa_internal.h"
+
+namespace {
+
+constexpr int kBN = 64;   // keys per tile
+constexpr int kBM = 32;   // query tokens per wave
+constexpr int kPadK = 8;  // bf16 of padding per K row / V^T row in LDS
+
+struct FaParams {
+  const bf16_t* q;    // [B*T, Hq*D] (already rotated)
+  const bf16_t* k;    // [B, Hkv, S_max, D]
+  const bf16_t* v;
+  const int32_t* pos;  // [B] tokens in the cache before this chunk
+  bf16_t* out;         // [B*T, Hq*D]
+  float scale_log2e;
+  int T, Hq, Hkv, S_max, G, units;  // units = token tiles * G
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
+  constexpr int STEPS = D / 16;  // MFMA steps over d for S^T
+  constexpr int DT = D / 32;     // 32-row tiles of O^T
+  constexpr int KS = D + kPadK;  // LDS row stride of K (bf16)
+  constexpr int VS = kBN + kPadK;  // LDS row stride of V^T (bf16)
+  constexpr int VEC = D / 8;     // 16-byte vectors per K/V row
+  constexpr int LOADS = kBN * VEC / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[kBN * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[D * VS];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, kq = lane >> 5;
+  const int kvh = blockIdx.y, b = blockIdx.z;
+  // heavy (late) token tiles first
+  const int u0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 4;
+  const int u = u0 + wave;
+  const bool active = u < p.units;
+  const int uc = active ? u : p.units - 1;
+  const int tt = uc / p.G, g = uc % p.G;
+  const int hq = kvh * p.G + g;
+  const int pos = p.pos[b];
+  const int t_lane = min(tt * kBM + n, p.T - 1);            // this lane's query token
+  const int last_w = pos + min(tt * kBM + kBM - 1, p.T - 1);  // last key any row of the wave sees
+  const int tt_max = min(u0 + 3, p.units - 1) / p.G;
+  const int last_wg = min(pos + min(tt_max * kBM + kBM - 1, p.T - 1), p.S_max - 1);
+  const int n_tiles = last_wg / kBN + 1;
+
+  // Q^T operand: lane (query n, half kq) holds d = step*16 + kq*8 .. +8 for every step
+  uint4 qreg[STEPS];
+  {
+    const bf16_t* qp = p.q + ((size_t)b * p.T + t_lane) * ((size_t)p.Hq * D) + (size_t)hq * D + kq * 8;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) qreg[s] = *reinterpret_cast<const uint4*>(qp + s * 16);
+  }
+
+  const bf16_t* kbase = p.k + ((size_t)b * p.Hkv + kvh) * (size_t)p.S_max * D;
+  const bf16_t* vbase = p.v + ((size_t)b * p.Hkv + kvh) * (size_t)p.S_max * D;
+  uint4 kreg[LOADS], vreg[LOADS];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int vi = tid + i * 256;
+      const int key_k = min(kt * kBN + vi / VEC, p.S_max - 1);  // rows past the cache end: masked
+      kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)key_k * D + (vi % VEC) * 8);
+      const int key_v = min(kt * kBN + (vi & (kBN - 1)), p.S_max - 1);
+      vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)key_v * D + (vi / kBN) * 8);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int vi = tid + i * 256;
+      *reinterpret_cast<uint4*>(&k_lds[(vi / VEC) * KS + (vi % VEC) * 8]) = kreg[i];
+      const int key = vi & (kBN - 1), c = vi / kBN;
+      const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vt_lds[(c * 8 + 2 * j) * VS + key] = (bf16_t)(w[j] & 0xFFFFu);
+        vt_lds[(c * 8 + 2 * j + 1) * VS + key] = (bf16_t)(w[j] >> 16);
+      }
+    }
+  };
+
+  // A-operand row r of a 32-key sub-tile holds this key, so that D registers 8s..8s+7
+  // of lane half kq are keys 16s + 8kq .. +8
+  const int jr = n >> 3;
+  const int key_of_row = 16 * (jr >> 1) + 8 * ((n >> 2) & 1) + 4 * (jr & 1) + (n & 3);
+
+  floatx16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  load_tile(0);
+  for (int kt = 0; kt < n_tiles; ++kt) {
+    __syncthreads();  // every wave is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (kt + 1 < n_tiles) load_tile(kt + 1);
+    const int key0 = kt * kBN;
+    if (key0 > last_w) continue;  // wave-uniform: nothing visible to this wave's rows
+
+    // ---- S^T = K Q^T for the two 32-key sub-tiles
+    floatx16 s[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[ks][e] = 0.f;
+      const bf16_t* kr = &k_lds[(ks * 32 + key_of_row) * KS + kq * 8];
+#pragma unroll
+      for (int st = 0; st < STEPS; ++st) {
+        const uint4 a = *reinterpret_cast<const uint4*>(kr + st * 16);
+        s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                        __builtin_bit_cast(bf16x8_t, qreg[st]),
+                                                        s[ks], 0, 0, 0);
+      }
+    }
+    // ---- online softmax over this lane's 32 keys (+ the partner half's 32)
+    const bool diag = key0 + kBN - 1 > pos + tt * kBM;  // some (query, key) pair is masked
+    const int vis = pos + t_lane - key0;                  // keys 0..vis of the tile are visible
+    float mx = -INFINITY;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        float x = s[ks][e] * p.scale_log2e;
+        if (diag) {
+          const int key = ks * 32 + 16 * (e >> 3) + 8 * kq + (e & 7);
+          if (key > vis) x = -INFINITY;
+        }
+        s[ks][e] = x;
+        mx = fmaxf(mx, x);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    // m_new is finite: key 0 is visible to every query, and tiles come in key order
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float sum = 0.f;
+    uint4 pb[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      float pr[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        pr[e] = __builtin_amdgcn_exp2f(s[ks][e] - m_new);
+        sum += pr[e];
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        pb[ks][st].x = pack_bf2(pr[8 * st + 0], pr[8 * st + 1]);
+        pb[ks][st].y = pack_bf2(pr[8 * st + 2], pr[8 * st + 3]);
+        pb[ks][st].z = pack_bf2(pr[8 * st + 4], pr[8 * st + 5]);
+        pb[ks][st].w = pack_bf2(pr[8 * st + 6], pr[8 * st + 7]);
+      }
+    }
+    sum += __shfl_xor(sum, 32, 64);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+    // ---- O^T = alpha * O^T + V^T P^T
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      const bf16_t* vr = &vt_lds[(dt * 32 + n) * VS + kq * 8];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const uint4 a = *reinterpret_cast<const uint4*>(vr + ks * 32 + st * 16);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                          __builtin_bit_cast(bf16x8_t, pb[ks][st]),
+                                                          o[dt], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- out[token][hq*D + d] = O^T[d][token] / l
+  if (!active || tt * kBM + n >= p.T) return;
+  const float inv = 1.f / l_run;
+  bf16_t* op = p.out + ((size_t)b * p.T + t_lane) * ((size_t)p.Hq * D) + (size_t)hq * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint2 w;
+      w.x = pack_bf2(o[dt][4 * j + 0] * inv, o[dt][4 * j + 1] * inv);
+      w.y = pack_bf2(o[dt][4 * j + 2] * inv, o[dt][4 * j + 3] * inv);
+      *reinterpret_cast<uint2*>(op + dt * 32 + 8 * j + 4 * kq) = w;
+    }
+}
+
+}  // namespace
+
+int exo_sdpa_prefill_mfma(const bf16_t* q, const bf16_t* k_cache, const bf16_t* v_cache,
+                          const int32_t* pos, bf16_t* out, float scale, int B, int T, int Hq,
+                          int Hkv, int D, int S_max, hipStream_t stream) {
+  FaParams p;
+  p.q = q;
+  p.k = k_cache;
+  p.v = v_cache;
+  p.pos = pos;
+  p.out = out;
+  p.scale_log2e = scale * 1.4426950408889634f;
+  p.T = T;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.S_max = S_max;
+  p.G = Hq / Hkv;
+  p.units = ((T + kBM - 1) / kBM) * p.G;
+  const dim3 grid((p.units + 3) / 4, Hkv, B);
+  if (D == 64)
+    fa_prefill_kernel<64><<<grid, 256, 0, stream>>>(p);
+  else
+    fa_prefill_kernel<128><<<grid, 256, 0, stream>>>(p);
+  return EXO_OK;
+}

@@ -243,11 +243,15 @@ def test_sdpa_decode(device, D, Hq, Hkv, lens):
         assert_close(n_f32(out)[b].reshape(Hq, D), want[0, :, 0], what=f"sdpa decode len {lens[b]}")
 
 
-@pytest.mark.parametrize("D,Hq,Hkv", [(64, 8, 2), (128, 8, 2)])
-def test_sdpa_prefill_causal(device, D, Hq, Hkv):
-    B, T, S_max = 2, 19, 64
-    pos = np.array([0, 30], np.int32)
-    q = rand_bf16((B * T, Hq * D), seed=D)
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 8, 2), (128, 8, 2), (128, 4, 4), (128, 4, 2), (128, 16, 2), (64, 16, 1)])
+@pytest.mark.parametrize("T,pos", [(19, (0, 30)), (5, (0, 3)), (100, (0, 77)), (64, (64, 1)), (161, (0, 200))])
+def test_sdpa_prefill_causal(device, D, Hq, Hkv, T, pos):
+    """Chunks shorter than 8 tokens run the per-token kernel, longer ones the matrix-core
+    flash kernel: 1, 2, 4, 8 and 16 query heads per kv head, chunk lengths on and off the
+    32-token tile, caches that start empty and part-filled, several key tiles."""
+    B, S_max = 2, 384
+    pos = np.array(pos, np.int32)
+    q = rand_bf16((B * T, Hq * D), seed=D + T)
     k = rand_bf16((B, Hkv, S_max, D), seed=13)
     v = rand_bf16((B, Hkv, S_max, D), seed=14)
     out = torch.empty(B * T, Hq * D, dtype=torch.bfloat16, device=device)
@@ -257,7 +261,21 @@ def test_sdpa_prefill_causal(device, D, Hq, Hkv):
         qq = q.reshape(B, T, Hq, D)[b:b + 1].transpose(0, 2, 1, 3)
         want = O.sdpa(qq, k[b:b + 1, :, :S], v[b:b + 1, :, :S], D ** -0.5, S - T)
         got = n_f32(out).reshape(B, T, Hq, D)[b].transpose(1, 0, 2)
-        assert_close(got, want[0], what="sdpa prefill")
+        assert_close(got, want[0], what=f"sdpa prefill T={T} pos={pos[b]}")
+
+
+def test_sdpa_prefill_cache_exactly_full(device):
+    """The last key tile ends at the end of the cache allocation (no reads past it)."""
+    B, T, Hq, Hkv, D, S_max = 1, 40, 8, 2, 128, 100
+    pos = np.array([60], np.int32)
+    q = rand_bf16((B * T, Hq * D), seed=3)
+    k = rand_bf16((B, Hkv, S_max, D), seed=4)
+    v = rand_bf16((B, Hkv, S_max, D), seed=5)
+    out = torch.empty(B * T, Hq * D, dtype=torch.bfloat16, device=device)
+    ops.sdpa_prefill(t_bf16(q, device), t_bf16(k, device), t_bf16(v, device), torch.from_numpy(pos).to(device), out, D ** -0.5, B, T, Hq, Hkv, D)
+    qq = q.reshape(B, T, Hq, D).transpose(0, 2, 1, 3)
+    want = O.sdpa(qq, k, v, D ** -0.5, S_max - T)
+    assert_close(n_f32(out).reshape(T, Hq, D).transpose(1, 0, 2), want[0], what="sdpa prefill full cache")
 
 
 def test_swiglu(device):

@@ -51,10 +51,10 @@ def test_prefill_and_decode_logits_match_oracle(ckpt, device):
     prompt = rng(11).integers(0, cfg.vocab_size, size=40)
     oc = OM.make_kv_cache(om.n_local_layers)
     gc = gm.make_cache(1, 128)
+    om.router_margins.clear()
     want = om(prompt[None], oc)  # [1,40,V]
     got = gm(torch.from_numpy(prompt[None].astype(np.int32)), gc)  # T=40 -> MFMA + prefill sdpa
     assert gc[0].offset == 40 and oc[0].offset == 40
-    om.router_margins.clear()
     if cfg.is_moe:
         tied = _check_tokens(n_f32(got), want, om, "prefill logits")
     else:
@@ -154,7 +154,11 @@ def test_pipeline_shards_compose(ckpt, device):
     hidden = s0(tt, c0)
     assert hidden.shape == (1, 20, cfg.hidden_size)
     o0 = OM.ShardModel(ckpt["ocfg"], ckpt["ow"], 0, k, gemm_rows=16)
-    assert_close_stat(n_f32(hidden), o0(toks, OM.make_kv_cache(k)), what="shard-0 hidden")
+    want0 = o0(toks, OM.make_kv_cache(k))
+    if cfg.is_moe:  # a router near-tie may send a token to another expert (exempt, printed)
+        _check_tokens(n_f32(hidden), want0, o0, "shard-0 hidden")
+    else:
+        assert_close_stat(n_f32(hidden), want0, what="shard-0 hidden")
     logits = s1(None, c1, input_embeddings=hidden)
     full = gm(tt, cf)
     np.testing.assert_array_equal(n_f32(logits), n_f32(full))

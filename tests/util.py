@@ -166,7 +166,9 @@ def check_tokens(got, want, om, what):
         if gaps is not None and gaps[t] <= 2.0 ** -6 * max(1.0, rms):
             tied_before = True
         if rel > 2e-2:
-            assert tied_before, f"{what}: token {t} rel-rms {rel:.3e} with no router near-tie"
+            gap = "n/a" if gaps is None else f"{float(np.min(gaps[: t + 1])):.3e}"
+            assert tied_before, (f"{what}: token {t} rel-rms {rel:.3e} with no router near-tie "
+                                 f"(smallest router gap so far {gap})")
             print(f"[parity] {what}: token {t} rel-rms {rel:.3e} after a router near-tie (exempt)")
     return tied_before
 
