@@ -1,21 +1,21 @@
 // Quantised matmul for prefill (any M): y[M,N] = x[M,K] @ dq(W)[N,K]^T.
 //
-// Matrix-core design for gfx950: a 128x128 output tile per 256-thread workgroup, one
-// 64-wide K step per iteration = exactly one quantisation group, so every packed row
-// segment needs a single (scale, bias).  Each thread dequantises 32 (4-bit) or
+// Matrix-core design for gfx950: a 256x128 (128x128 for M <= 128) output tile per
+// 256-thread workgroup, one 64-wide K step per iteration = exactly one quantisation group,
+// so every packed row segment needs a single (scale, bias).  Each thread dequantises 32 (4-bit) or
 // 2x16 (8-bit) codes to bf16 in registers - bf16(fma(s, q, b)), codes converted with
 // v_cvt_f32_ubyteN - and stores them to LDS next to the activation tile; the four
-// waves (2x2) then issue v_mfma_f32_32x32x16_bf16 on 64x64 sub-tiles with float32
-// accumulators.  Global loads of the next K step are issued before the MFMAs of the
+// waves (2x2) then issue v_mfma_f32_32x32x16_bf16 on 128x64 (64x64) sub-tiles with float32
+// accumulators: the taller tile halves both the dequantisation work and the LDS bytes
+// read per MFMA.  Global loads of the next K step are issued before the MFMAs of the
 // current one.  LDS rows are padded by 16 bytes to keep ds_read_b128 conflict-free.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row
-constexpr int kThreads = 256;
 
 struct QmmParams {
   const bf16_t* x;
@@ -37,63 +37,70 @@ __device__ __forceinline__ float ubyte_f(uint32_t v, int i) {
   return (float)((v >> (8 * i)) & 0xffu);  // v_cvt_f32_ubyteN
 }
 
-template <int BITS>
-__global__ __launch_bounds__(kThreads) void qmm_kernel(const QmmParams p) {
+// The workgroup is 2 x WN waves; a wave computes (32*MI) x 64 outputs, so the tile is
+// (64*MI) x (64*WN).  STAGES = K steps whose global loads are in flight (held in
+// registers) while the current step is multiplied.
+template <int BITS, int MI, int WN, int STAGES>
+__global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
+  constexpr int kThreads = 128 * WN;
+  constexpr int BM = 64 * MI, BN = 64 * WN;
+  constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LDS_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t ws[BN * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int wm = (wave / WN) * (32 * MI), wn = (wave % WN) * 64;
   const int G = p.K >> 6;
   const int wpr = p.K * BITS / 32;
 
-  // W: thread -> (row, part).  4-bit: 2 parts of 32 codes; 8-bit: 2 parts of 32 codes
-  // (two 16-byte loads each).
+  // W: thread -> (row, part): 2 parts of 32 codes per row and K step
   const int w_row = tid >> 1, w_part = tid & 1;
   const bool w_ok = (n0 + w_row) < p.N;
   const uint32_t* wsrc = p.w + (size_t)(n0 + (w_ok ? w_row : 0)) * wpr + w_part * (BITS);
   const bf16_t* ssrc = p.s + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
   const bf16_t* bsrc = p.b + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
 
-  uint4 xa[4];
-  WFrag<BITS> wf;
+  struct Stage {
+    uint4 xa[XR];
+    WFrag<BITS> wf;
+  };
 
-  auto load_global = [&](int k0) {
+  auto load_global = [&](Stage& st, int k0) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < XR; ++r) {
       const int id = tid + kThreads * r;
       const int row = id >> 3, kp = id & 7;
       if (m0 + row < p.M)
-        xa[r] = *reinterpret_cast<const uint4*>(p.x + (size_t)(m0 + row) * p.K + k0 + kp * 8);
+        st.xa[r] = *reinterpret_cast<const uint4*>(p.x + (size_t)(m0 + row) * p.K + k0 + kp * 8);
       else
-        xa[r] = make_uint4(0, 0, 0, 0);
+        st.xa[r] = make_uint4(0, 0, 0, 0);
     }
     const int kw = k0 * BITS / 32;  // word offset of this K step
 #pragma unroll
     for (int i = 0; i < BITS / 4; ++i)
-      wf.q[i] = *reinterpret_cast<const uint4*>(wsrc + kw + i * 4);
-    wf.s = bf2f(ssrc[k0 >> 6]);
-    wf.b = bf2f(bsrc[k0 >> 6]);
+      st.wf.q[i] = *reinterpret_cast<const uint4*>(wsrc + kw + i * 4);
+    st.wf.s = bf2f(ssrc[k0 >> 6]);
+    st.wf.b = bf2f(bsrc[k0 >> 6]);
     if (!w_ok) {
-      wf.s = 0.f;
-      wf.b = 0.f;
+      st.wf.s = 0.f;
+      st.wf.b = 0.f;
     }
   };
 
-  auto store_lds = [&]() {
+  auto store_lds = [&](const Stage& st) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < XR; ++r) {
       const int id = tid + kThreads * r;
       const int row = id >> 3, kp = id & 7;
-      *reinterpret_cast<uint4*>(&xs[row * LDS_STRIDE + kp * 8]) = xa[r];
+      *reinterpret_cast<uint4*>(&xs[row * LDS_STRIDE + kp * 8]) = st.xa[r];
     }
     bf16_t* dst = &ws[w_row * LDS_STRIDE + w_part * 32];
-    const float s = wf.s, b = wf.b;
+    const float s = st.wf.s, b = st.wf.b;
+    const uint32_t* qw = reinterpret_cast<const uint32_t*>(&st.wf.q[0]);
     if (BITS == 4) {
-      const uint32_t* qw = reinterpret_cast<const uint32_t*>(&wf.q[0]);
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {  // two 16-byte LDS stores of 8 codes... x2 words each
+      for (int h = 0; h < 2; ++h) {  // 2 words = 16 codes = two 16-byte LDS stores
         uint4 o[2];
         uint32_t* o4 = reinterpret_cast<uint32_t*>(o);
 #pragma unroll
@@ -108,7 +115,6 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(const QmmParams p) {
         *reinterpret_cast<uint4*>(dst + h * 16 + 8) = o[1];
       }
     } else {
-      const uint32_t* qw = reinterpret_cast<const uint32_t*>(&wf.q[0]);
 #pragma unroll
       for (int h = 0; h < 4; ++h) {  // 8 codes (2 words) per 16-byte LDS store
         uint4 o;
@@ -124,41 +130,56 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(const QmmParams p) {
     }
   };
 
-  floatx16 acc[2][2];
+  floatx16 acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int frow = lane & 31, fk = (lane >> 5) * 8;
-  load_global(0);
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    __syncthreads();  // previous step's LDS reads are done
-    store_lds();
-    __syncthreads();
-    if (k0 + BK < p.K) load_global(k0 + BK);
+  auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
-      bf16x8_t a[2], bq[2];
+      bf16x8_t a[MI], bq[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
         a[i] = *reinterpret_cast<const bf16x8_t*>(&xs[(wm + i * 32 + frow) * LDS_STRIDE + ks + fk]);
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         bq[j] = *reinterpret_cast<const bf16x8_t*>(&ws[(wn + j * 32 + frow) * LDS_STRIDE + ks + fk]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], bq[j], acc[i][j], 0, 0, 0);
     }
+  };
+
+  // one K step: stage `st` (loaded STAGES steps ago) goes to LDS, is refilled with the
+  // step STAGES ahead, and the tile is multiplied
+  auto step = [&](Stage& st, int k0) {
+    __syncthreads();  // previous step's LDS reads are done
+    store_lds(st);
+    __syncthreads();
+    if (k0 + STAGES * BK < p.K) load_global(st, k0 + STAGES * BK);
+    multiply();
+  };
+
+  Stage st[STAGES];
+#pragma unroll
+  for (int i = 0; i < STAGES; ++i)
+    if (i * BK < p.K) load_global(st[i], i * BK);
+  for (int k0 = 0; k0 < p.K; k0 += STAGES * BK) {
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i)
+      if (k0 + i * BK < p.K) step(st[i], k0 + i * BK);
   }
 
   // D[i][j]: column j = lane%32 (W row n), rows 8*(r/4) + 4*(lane/32) + r%4 (token m)
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int n = n0 + wn + j * 32 + (lane & 31);
@@ -175,6 +196,17 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(const QmmParams p) {
     }
 }
 
+template <int BITS>
+void launch_qmm(const QmmParams& p, hipStream_t st) {
+  const int M = p.M, N = p.N;
+  // up to 128 rows: little arithmetic per K step, so several steps' loads are kept in
+  // flight; taller inputs: 256-row tiles halve the dequantisation work per output
+  if (M <= 128)
+    qmm_kernel<BITS, 2, 2, 2><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), 256, 0, st>>>(p);
+  else
+    qmm_kernel<BITS, 4, 2, 1><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 256)), 256, 0, st>>>(p);
+}
+
 }  // namespace
 
 extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
@@ -187,12 +219,11 @@ extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* sca
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmm: null pointer");
   if (M == 0) return EXO_OK;
   QmmParams p{x, w, scales, biases, residual, y, M, N, K};
-  dim3 grid(exo_ceil_div(N, BN), exo_ceil_div(M, BM));
-  EXO_REQUIRE(grid.y <= 65535, "exo_qmm: M=%d too large", M);
+  EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm: M=%d too large", M);
   if (bits == 4)
-    qmm_kernel<4><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+    launch_qmm<4>(p, (hipStream_t)stream);
   else
-    qmm_kernel<8><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+    launch_qmm<8>(p, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_qmm");
   return EXO_OK;
 }
