@@ -36,6 +36,11 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (1..16)")
+    ap.add_argument("--shard-layers", type=int, default=None,
+                    help="run layers [0, n) as a first pipeline shard (output: hidden state)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "qmatmul_sweep"],
+                    help="decode (default, the headline) or the quantised-matmul shape sweep")
     return ap.parse_args()
 
 
@@ -197,6 +202,92 @@ def cpu_baseline(model, torch, seconds: float, context: int):
                 host_cpus=os.cpu_count(), affinity=len(os.sched_getaffinity(0)))
 
 
+def active_token_bytes(model, cfg, ctx: int, batch: int) -> int:
+    """Algorithmic HBM bytes of one decode step: every weight the step multiplies by (for
+    MoE layers the router plus top-k experts per sequence, at most all experts) once,
+    plus the K/V read of every sequence."""
+    n = 0
+    for L in model.layers:
+        n += L.qkv.nbytes + L.o.nbytes
+        if cfg.is_moe:
+            per_expert = (L.gate.nbytes + L.up.nbytes + L.down.nbytes) // cfg.num_experts
+            n += L.router.nbytes + per_expert * min(cfg.num_experts, cfg.num_experts_per_tok * batch)
+        else:
+            n += L.gate.nbytes + L.up.nbytes + L.down.nbytes
+    if model.lm_head is not None:
+        n += model.lm_head.nbytes
+    kv = 2 * len(model.layers) * cfg.num_key_value_heads * cfg.head_dim * ctx * 2 * batch
+    return n + kv
+
+
+def qmatmul_sweep(args):
+    """configs[1] of the baseline: y = x @ dq(W)^T over the listed (N, K), bits and M.
+    Weight copies rotate so that nothing is served from cache; one HIP-graph replay holds
+    one launch per copy; events on the launch stream give the average launch duration."""
+    import torch
+
+    from exo_amd import native, ops
+    from exo_amd.ops import QuantizedWeight
+
+    native.load()
+    dev = torch.device("cuda:0")
+    shapes = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)]
+    rows = []
+    g = torch.Generator(device=dev).manual_seed(4321)
+    for bits in (4, 8):
+        for (N, K) in shapes:
+            wbytes = qbytes(N, K, bits)
+            copies = max(4, min(32, int(1.5e9 // wbytes) + 1))
+            ws = []
+            for _ in range(copies):
+                w = torch.randint(-2**31, 2**31 - 1, (N, K * bits // 32), dtype=torch.int32, device=dev, generator=g)
+                sc = (torch.rand(N, K // 64, device=dev, generator=g) * 0.01).bfloat16()
+                bi = (torch.rand(N, K // 64, device=dev, generator=g) * -0.08).bfloat16()
+                ws.append(QuantizedWeight(w, sc, bi, bits))
+            for M in (1, 4, 16, 128, 2048):
+                if M >= 128 and N * M * 2 > (1 << 30):
+                    continue  # 128256 x 2048 outputs: not a shape the models produce
+                x = torch.randn(M, K, device=dev, generator=g).bfloat16()
+                y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                fns = [(lambda q=q: ops.quantized_matmul(x, q, out=y)) for q in ws]
+                for f in fns:
+                    f()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for f in fns:
+                        f()
+                gr.replay()
+                torch.cuda.synchronize()
+                reps = 10 if M <= 128 else 3
+                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                st.record()
+                for _ in range(reps):
+                    gr.replay()
+                en.record()
+                torch.cuda.synchronize()
+                us = st.elapsed_time(en) * 1e3 / (reps * copies)
+                nbytes = wbytes + 2 * M * (K + N)
+                flops = 2.0 * M * N * K
+                rows.append(dict(bits=bits, N=N, K=K, M=M, us=round(us, 2), GBps=round(nbytes / us * 1e-3, 1),
+                                 frac_hbm=round(nbytes / us * 1e-3 / 8000.0, 3),
+                                 TFLOPs=round(flops / us * 1e-6, 1), frac_mfma=round(flops / us * 1e-6 / 2500.0, 3)))
+                print(f"[sweep] b{bits} N={N} K={K} M={M}: {us:.1f} us", file=sys.stderr, flush=True)
+            del ws
+    best = max((r for r in rows if r["M"] == 1), key=lambda r: r["GBps"])
+    dom = next(r for r in rows if (r["bits"], r["N"], r["K"], r["M"]) == (4, 14336, 4096, 1))
+    print(json.dumps({
+        "metric": "qmatmul HBM GB/s (% of 8 TB/s) over the shape sweep", "value": dom["GBps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": len(rows), "warmup": 1, "ms_per_step": dom["us"] * 1e-3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: quantised matmul sweep, bits {4,8} x 5 shapes x M {1,4,16,128,2048}; "
+                               "value = 4-bit 14336x4096 at M=1"},
+        "roofline": {"bound": "hbm", "achieved": dom["GBps"], "peak": 8000.0, "unit": "GB/s",
+                     "frac": dom["GBps"] / 8000.0, "traffic": None},
+        "best_M1": best, "rows": rows, "cpu_baseline": None}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -204,6 +295,8 @@ def main():
               "supported. Multi-GPU pipeline/tensor sharding is design-only (see DESIGN.md).",
               file=sys.stderr)
         sys.exit(2)
+    if args.workload == "qmatmul_sweep":
+        return qmatmul_sweep(args)
     import torch
 
     from exo_amd import native
@@ -218,28 +311,40 @@ def main():
     cfg = named_config(args.config)
     if args.layers:
         cfg.num_hidden_layers = args.layers
+    B = args.batch
+    if not 1 <= B <= 16:
+        sys.exit("bench.py: --batch must be 1..16")
+    end = args.shard_layers or cfg.num_hidden_layers
     t0 = time.perf_counter()
-    weights = synth_weights(cfg, seed=0, device=dev)
-    model = ShardModel(cfg, weights, device=dev)
+    weights = synth_weights(cfg, 0, end, seed=0, device=dev)
+    model = ShardModel(cfg, weights, 0, end, device=dev)
     del weights
     torch.cuda.synchronize()
     t_build = time.perf_counter() - t0
+    print(f"[bench] weights ready in {t_build:.1f} s", file=sys.stderr, flush=True)
 
     g = torch.Generator().manual_seed(1234)
-    prompt = torch.randint(0, cfg.vocab_size, (args.prompt,), generator=g).tolist()
     K, W = args.steps, args.warmup
-    cache = model.make_cache(1, args.prompt + K + W + 64)
+    cache = model.make_cache(B, args.prompt + K + W + 64)
 
-    # prefill with the reference's protocol, then the last-but-one token as a GEMV step
-    tps_prefill, n_prefill = prefill(model, prompt[:-1], cache)
-    model(torch.tensor([[prompt[-2]]], dtype=torch.int32), cache, logits="none")
-    bufs = model._buffers(1, 1)
-    bufs.tokens[0] = prompt[-1]
+    # prefill with the reference's protocol (one sequence at a time, as its batch engine
+    # does), then the last-but-one prompt token of every sequence as a GEMV step
+    tps_prefill, n_prefill, last = 0.0, 0, []
+    for row in range(B):
+        prompt = torch.randint(0, cfg.vocab_size, (args.prompt,), generator=g).tolist()
+        tps, n = prefill(model, prompt[:-1], cache, row=row,
+                         faithful_extra_steps=model.is_last)
+        tps_prefill, n_prefill = tps, n
+        model(torch.tensor([[prompt[-2]]], dtype=torch.int32), cache, logits="none",
+              rows=slice(row, row + 1))
+        last.append(prompt[-1])
+        print(f"[bench] row {row}: prefill {n} tokens at {tps:.0f} tok/s", file=sys.stderr, flush=True)
+    bufs = model._buffers(B, 1)
+    bufs.tokens.copy_(torch.tensor(last, dtype=torch.int32))
 
     def step():
-        return model.decode_step(cache, 1, use_graph=not args.no_graph, feedback=True)
+        return model.decode_step(cache, B, use_graph=not args.no_graph, feedback=model.is_last)
 
-    toks = []
     for _ in range(W):
         step()
     torch.cuda.synchronize()
@@ -249,37 +354,49 @@ def main():
         step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    toks.append(int(bufs.next_token[0]))
-    tok_s = K / dt
+    last_token = int(bufs.next_token[0]) if model.is_last else None
+    tok_s = B * K / dt
+    token_bytes = active_token_bytes(model, cfg, ctx0, B)
 
-    kernels = measure_kernels(model, torch)
-    for k in kernels:
-        k["frac_of_8TBps"] = k["GBps"] / 8000.0
-        k["us_per_token"] = k["avg_us"] * k["launches_per_token"]
-    dom = max(kernels, key=lambda k: k["us_per_token"])
-    gemv_us = sum(k["us_per_token"] for k in kernels)
-    gemv_bytes = sum(k["bytes_per_launch"] * k["launches_per_token"] for k in kernels)
-    roofline = dict(bound="hbm", achieved=dom["GBps"], peak=8000.0, unit="GB/s",
-                    frac=dom["GBps"] / 8000.0, traffic=None, kernel=dom["kernel"],
-                    launch=dom["name"], avg_us=dom["avg_us"], bytes_per_launch=dom["bytes_per_launch"],
-                    all_gemv_GBps=gemv_bytes / gemv_us * 1e-3, all_gemv_us_per_token=gemv_us)
+    headline = (args.config == "llama-3.1-8b" and B == 1 and model.is_last and not cfg.is_moe)
+    if not cfg.is_moe and model.is_last and B == 1:
+        kernels = measure_kernels(model, torch)
+        for k in kernels:
+            k["frac_of_8TBps"] = k["GBps"] / 8000.0
+            k["us_per_token"] = k["avg_us"] * k["launches_per_token"]
+        dom = max(kernels, key=lambda k: k["us_per_token"])
+        gemv_us = sum(k["us_per_token"] for k in kernels)
+        gemv_bytes = sum(k["bytes_per_launch"] * k["launches_per_token"] for k in kernels)
+        roofline = dict(bound="hbm", achieved=dom["GBps"], peak=8000.0, unit="GB/s",
+                        frac=dom["GBps"] / 8000.0, traffic=None, kernel=dom["kernel"],
+                        launch=dom["name"], avg_us=dom["avg_us"], bytes_per_launch=dom["bytes_per_launch"],
+                        all_gemv_GBps=gemv_bytes / gemv_us * 1e-3, all_gemv_us_per_token=gemv_us)
+    else:
+        # no single dominant launch is isolated here: the whole step against its bytes
+        kernels = None
+        gbps = token_bytes / (dt / K) * 1e-9
+        roofline = dict(bound="hbm", achieved=gbps, peak=8000.0, unit="GB/s", frac=gbps / 8000.0,
+                        traffic=None, kernel="all launches of one decode step",
+                        bytes_per_launch=token_bytes, avg_us=dt / K * 1e6)
 
-    kv_bytes = 2 * len(model.layers) * cfg.num_key_value_heads * cfg.head_dim * ctx0 * 2
-    token_bytes = model.weight_bytes() + kv_bytes
+    what = {"llama-3.2-1b": "configs[0]", "llama-3.1-8b": "configs[2]", "qwen3-30b-a3b": "configs[3]",
+            "qwen3-235b-a22b": "configs[4]"}.get(args.config, "custom")
+    shard = "" if model.is_last else f", pipeline shard of layers [0,{end}) (output: hidden state)"
     out = {
-        "metric": "decode tok/s + qmatmul HBM GB/s (% peak), Llama-3.1-8B 4-bit g64 bs1",
+        "metric": ("decode tok/s + qmatmul HBM GB/s (% peak), Llama-3.1-8B 4-bit g64 bs1" if headline
+                   else f"decode tok/s, {args.config} {cfg.bits}-bit g64 batch {B}"),
         "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": dt / K * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"configs[2]: {args.config} architecture, MLX affine {cfg.bits}-bit g64, "
-                               f"random prompt of {args.prompt} tokens, greedy decode, batch 1",
-                   "layers": cfg.num_hidden_layers, "context_at_start": ctx0, "hip_graph": not args.no_graph},
+        "config": {"workload": f"{what}: {args.config} architecture, MLX affine {cfg.bits}-bit g64, "
+                               f"random prompt of {args.prompt} tokens, greedy decode, batch {B}{shard}",
+                   "layers": len(model.layers), "context_at_start": ctx0, "hip_graph": not args.no_graph},
         "roofline": roofline,
         "prefill_tok_s": tps_prefill, "prefill_tokens": n_prefill,
-        "token_bytes": token_bytes, "effective_GBps": token_bytes * tok_s * 1e-9,
-        "kernels": kernels, "build_s": t_build, "last_token": toks[-1],
+        "token_bytes": token_bytes, "effective_GBps": token_bytes * (K / dt) * 1e-9,
+        "kernels": kernels, "build_s": t_build, "last_token": last_token,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and kernels is not None:
         out["cpu_baseline"] = cpu_baseline(model, torch, args.cpu_seconds, ctx0)
     else:
         out["cpu_baseline"] = None

@@ -108,6 +108,7 @@ class _Buffers:
             self.router_logits = torch.empty(R, c.num_experts, **bf)
             self.act = torch.empty(R, k, Ie, **bf)
             self.expert_out = torch.empty(R, k, c.hidden_size, **bf)
+            self.gate = self.up = None
         else:
             self.act = torch.empty(R, c.intermediate_size, **bf)
             self.gate = self.up = None
@@ -211,12 +212,22 @@ class ShardModel:
             return
         ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
         idx, sc = ops.router_topk(bf.router_logits, c.num_experts_per_tok, c.norm_topk_prob)
-        step = max(1, 65535 // c.num_experts_per_tok)
-        for r0 in range(0, R, step):  # the grouped GEMV takes decode-sized row counts
-            r1 = min(R, r0 + step)
-            ops.gather_qmv_swiglu(bf.n[r0:r1], L.gate, L.up, idx[r0:r1], out=bf.act[r0:r1])
-            ops.gather_qmm(bf.act[r0:r1], L.down, idx[r0:r1], out=bf.expert_out[r0:r1])
-            ops.moe_combine(bf.expert_out[r0:r1], sc[r0:r1], residual=bf.h[r0:r1], out=bf.h[r0:r1])
+        k = c.num_experts_per_tok
+        if not gemv:  # prefill: rows sorted by expert, one MFMA GEMM per projection
+            if bf.gate is None:
+                bf.gate = torch.empty_like(bf.act)
+                bf.up = torch.empty_like(bf.act)
+            ws = ops.moe_group(idx, c.num_experts)
+            x3 = bf.n.view(R, 1, -1)
+            ops.grouped_qmm(x3, L.gate, ws, k, out=bf.gate)
+            ops.grouped_qmm(x3, L.up, ws, k, out=bf.up)
+            ops.swiglu(bf.gate, bf.up, out=bf.act)
+            ops.grouped_qmm(bf.act, L.down, ws, k, out=bf.expert_out)
+            ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
+            return
+        ops.gather_qmv_swiglu(bf.n, L.gate, L.up, idx, out=bf.act)
+        ops.gather_qmm(bf.act, L.down, idx, out=bf.expert_out)
+        ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
 
     def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
              rows: slice | None = None):

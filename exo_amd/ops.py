@@ -256,6 +256,38 @@ def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, 
     return out
 
 
+def moe_group(idx: torch.Tensor, E: int) -> torch.Tensor:
+    """Sort the (token, slot) pairs of idx int32 [T, topk] by expert; the returned workspace
+    feeds grouped_qmm for every projection that shares this routing decision."""
+    lib = native.load()
+    T, topk = idx.shape
+    assert idx.dtype == torch.int32 and idx.is_contiguous()
+    nbytes = lib.exo_moe_group_workspace(T, topk, E)
+    ws = torch.empty(nbytes // 4, dtype=torch.int32, device=idx.device)
+    check(lib.exo_moe_group(_ptr(idx), T, topk, E, _ptr(ws), nbytes, _stream()), "moe_group")
+    return ws
+
+
+def grouped_qmm(x: torch.Tensor, qw: QuantizedWeight, group_ws: torch.Tensor, topk: int, out=None):
+    """mx.gather_qmm for prefill-sized inputs on the matrix cores: x bf16 [T, R, K] (R == 1
+    or topk), routing prepared by moe_group -> bf16 [T, topk, N]."""
+    lib = native.load()
+    T, R, K = x.shape
+    E = qw.weight.shape[0]
+    if K != qw.K:
+        raise ValueError(f"grouped_qmm: x has K={K}, weight has K={qw.K}")
+    if out is None:
+        out = torch.empty(T, topk, qw.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_gather_qmm(
+            _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(group_ws), _ptr(out),
+            T, topk, R, E, qw.N, K, qw.bits, qw.group_size, _stream(),
+        ),
+        "grouped_qmm",
+    )
+    return out
+
+
 def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None):
     """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N]."""
     lib = native.load()

@@ -97,6 +97,21 @@ int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
             const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
             int K, int bits, int group_size, exo_stream_t stream);
 
+/* K3 for prefill-sized T: the same operator as exo_gather_qmv on the matrix cores.  The
+ * (token, slot) pairs are first sorted by expert (exo_moe_group, once per routing
+ * decision; its workspace of exo_moe_group_workspace(T, topk, E) bytes then serves every
+ * exo_gather_qmm of the layer), and each expert's run of rows is multiplied by that
+ * expert's matrix in tiles of 128 rows.  x bf16 [T, x_rows, K] with x_rows == 1 or topk;
+ * y bf16 [T, topk, N].  What `sorted_indices=True` asks of mx.gather_qmm
+ * (.typings/mlx/core/__init__.pyi:2957-3006; .typings/mlx_lm/models/switch_layers.pyi:10-31). */
+int64_t exo_moe_group_workspace(int T, int topk, int E);
+int exo_moe_group(const int32_t* idx, int T, int topk, int E, void* workspace,
+                  int64_t workspace_bytes, exo_stream_t stream);
+int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                   const uint16_t* biases, const void* workspace, uint16_t* y, int T, int topk,
+                   int x_rows, int E, int N, int K, int bits, int group_size,
+                   exo_stream_t stream);
+
 /* K3: mx.gather_qmm(x, w, scales, biases, rhs_indices=idx, transpose=True) as
  * QuantizedSwitchLinear calls it: w uint32 [E,N,K*bits/32]; idx int32 [T,topk];
  * x bf16 [T, x_rows, K] with x_rows == 1 (same row for every slot) or topk;

@@ -155,6 +155,34 @@ def test_gather_qmv(device, bits, x_rows):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("x_rows", ["one", "topk"])
+@pytest.mark.parametrize("E,N,K,T,topk", [(6, 96, 768, 40, 4), (128, 200, 128, 300, 8), (3, 64, 64, 1, 2)])
+def test_grouped_qmm(device, bits, x_rows, E, N, K, T, topk):
+    """Prefill-sized gather_qmm: pairs sorted by expert, one matrix-core tile row block per
+    expert run (experts with no rows, with a partial tile and with several tiles), against
+    the oracle's per-pair loop."""
+    trip = rand_quantized(N, K, bits, seed=40 + E, E=E)
+    idx = rng(41 + T).integers(0, E, size=(T, topk)).astype(np.int32)
+    if E == 128:
+        idx[: T // 2, 0] = 5  # one expert with more than a tile of rows
+    R = 1 if x_rows == "one" else topk
+    x = rand_bf16((T, R, K), seed=42)
+    it = torch.from_numpy(idx).to(device)
+    ws = ops.moe_group(it, E)
+    P = T * topk
+    sorted_pairs = ws[:P].cpu().numpy()
+    assert sorted(sorted_pairs.tolist()) == list(range(P))          # a permutation of the pairs
+    experts_in_order = idx.reshape(-1)[sorted_pairs]
+    assert np.all(np.diff(experts_in_order) >= 0)                    # grouped by expert
+    tiles = ws[P:].cpu().numpy().reshape(-1, 3)
+    used = tiles[tiles[:, 0] >= 0]
+    assert used[:, 2].sum() == P and used[:, 2].max() <= 128
+    got = n_f32(ops.grouped_qmm(t_bf16(x, device), t_qw(trip, bits, device), ws, topk))
+    want = affine.gather_qmm(x, *trip, idx, 64, bits)
+    assert_close(got, want, what="grouped_qmm")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 def test_gather_qmv_swiglu(device, bits):
     E, N, K, T, topk = 5, 64, 2048, 2, 3
     g = rand_quantized(N, K, bits, seed=50, E=E)
