@@ -148,7 +148,25 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
 }
 
 // ------------------------------------------------------------------- MoE routing
-// One wave per row; E <= 256 (4 values per lane).
+// One wave per row; E <= 256 (4 values per lane).  The k selections run on packed keys
+// (bf16 probability bits << 16 | 0xFFFF - expert): one unsigned max per selection finds
+// the largest probability and, among equals, the lowest expert id; the wave maximum is a
+// six-step DPP reduction whose result lands in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false);
+  return o > v ? o : v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = dpp_max_u32<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+  v = dpp_max_u32<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+  v = dpp_max_u32<0x141, 0xf>(v);  // row_half_mirror
+  v = dpp_max_u32<0x140, 0xf>(v);  // row_mirror: every lane holds its row-of-16 maximum
+  v = dpp_max_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_max_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 __global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* __restrict__ logits,
                                                          int32_t* __restrict__ idx,
                                                          bf16_t* __restrict__ scores, int E,
@@ -170,36 +188,26 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* __restric
     sum += v[i];
   }
   sum = wave_sum(sum);
-  // probabilities rounded to bf16; -1 marks "taken / absent"
+  // probabilities rounded to bf16 (non-negative, so their bit patterns order like the
+  // values); key 0 marks "taken / absent"
+  uint32_t key[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    v[i] = (lane + 64 * i < E) ? bf2f(f2bf(v[i] / sum)) : -1.f;
+  for (int i = 0; i < 4; ++i) {
+    const int e = lane + 64 * i;
+    key[i] = (e < E) ? (((uint32_t)f2bf(v[i] / sum) << 16) | (uint32_t)(0xFFFF - e)) : 0u;
+  }
   float sel[16];
   float tot = 0.f;
   for (int j = 0; j < k; ++j) {
-    // best (value, lowest index) over the wave
-    float bv = -1.f;
-    int bi = 0x7fffffff;
+    uint32_t best = key[0];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = lane + 64 * i;
-      if (v[i] > bv) {  // ascending e within the lane, so strict > keeps the lowest index
-        bv = v[i];
-        bi = e;
-      }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (ov > bv || (ov == bv && oi < bi)) {
-        bv = ov;
-        bi = oi;
-      }
-    }
+    for (int i = 1; i < 4; ++i) best = key[i] > best ? key[i] : best;
+    best = wave_max_u32(best);
+    const int bi = 0xFFFF - (int)(best & 0xFFFFu);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (lane + 64 * i == bi) v[i] = -1.f;
+      if (key[i] == best) key[i] = 0u;
+    const float bv = bf2f((bf16_t)(best >> 16));
     sel[j] = bv;
     tot += bv;
     if (lane == 0) idx[(size_t)row * k + j] = bi;

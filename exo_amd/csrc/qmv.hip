@@ -1020,11 +1020,13 @@ extern "C" int exo_gather_qmv(const uint16_t* x, const uint32_t* w, const uint16
   return EXO_OK;
 }
 
-extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
-                                     const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
-                                     const uint16_t* bu, const int32_t* idx, uint16_t* y, int T,
-                                     int topk, int E, int N, int K, int bits, int group_size,
-                                     exo_stream_t stream) {
+extern "C" int exo_norm_gather_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight,
+                                          float eps, const uint32_t* wg, const uint16_t* sg,
+                                          const uint16_t* bg, const uint32_t* wu,
+                                          const uint16_t* su, const uint16_t* bu,
+                                          const int32_t* idx, uint16_t* y, int T, int topk, int E,
+                                          int N, int K, int bits, int group_size,
+                                          exo_stream_t stream) {
   int rc = check_common("exo_gather_qmv_swiglu", 1, N, K, bits, group_size);
   if (rc) return rc;
   rc = check_gather("exo_gather_qmv_swiglu", T, topk, 1, E);
@@ -1042,8 +1044,17 @@ extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, cons
   ga.topk = topk;
   ga.x_rows = 1;
   rc = qmv_dispatch<2>(x, ws, ss, bs, nullptr, y, 1, N, K, bits, (hipStream_t)stream,
-                       "exo_gather_qmv_swiglu", ga);
+                       "exo_gather_qmv_swiglu", ga, norm_weight, eps);
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_gather_qmv_swiglu");
   return EXO_OK;
+}
+
+extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t* sg,
+                                     const uint16_t* bg, const uint32_t* wu, const uint16_t* su,
+                                     const uint16_t* bu, const int32_t* idx, uint16_t* y, int T,
+                                     int topk, int E, int N, int K, int bits, int group_size,
+                                     exo_stream_t stream) {
+  return exo_norm_gather_qmv_swiglu(x, nullptr, 0.f, wg, sg, bg, wu, su, bu, idx, y, T, topk, E,
+                                    N, K, bits, group_size, stream);
 }

@@ -210,7 +210,11 @@ class ShardModel:
                 ops.swiglu(bf.gate, bf.up, out=bf.act)
             ops.quantized_matmul(bf.act, L.down, residual=bf.h, out=bf.h)
             return
-        ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
+        if gemv:  # decode: the post-attention norm is fused into both consumers of it
+            ops.quantized_matmul(bf.h, L.router, out=bf.router_logits, norm_weight=L.post_norm,
+                                 eps=c.rms_norm_eps)
+        else:
+            ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
         idx, sc = ops.router_topk(bf.router_logits, c.num_experts_per_tok, c.norm_topk_prob)
         k = c.num_experts_per_tok
         if not gemv:  # prefill: rows sorted by expert, one MFMA GEMM per projection
@@ -225,7 +229,8 @@ class ShardModel:
             ops.grouped_qmm(bf.act, L.down, ws, k, out=bf.expert_out)
             ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
             return
-        ops.gather_qmv_swiglu(bf.n, L.gate, L.up, idx, out=bf.act)
+        ops.gather_qmv_swiglu(bf.h, L.gate, L.up, idx, out=bf.act, norm_weight=L.post_norm,
+                              eps=c.rms_norm_eps)
         ops.gather_qmm(bf.act, L.down, idx, out=bf.expert_out)
         ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
 
@@ -259,7 +264,7 @@ class ShardModel:
                                    L.q_norm, L.k_norm, c.rms_norm_eps)
                 ops.sdpa_prefill(bf.q, kc, vc, pos, bf.attn, self.scale, B, T, Hq, Hkv, D)
             ops.quantized_matmul(bf.attn, L.o, residual=bf.h, out=bf.h)
-            if c.is_moe or not gemv:
+            if not gemv:
                 ops.rms_norm(bf.h, L.post_norm, c.rms_norm_eps, out=bf.n)
             self._mlp(L, bf, R)
         if not self.is_last or logits_mode == "none":

@@ -288,8 +288,10 @@ def grouped_qmm(x: torch.Tensor, qw: QuantizedWeight, group_ws: torch.Tensor, to
     return out
 
 
-def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None):
-    """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N]."""
+def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None,
+                      norm_weight=None, eps: float = 0.0):
+    """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N];
+    ``norm_weight`` fuses a preceding rms_norm(x, norm_weight, eps)."""
     lib = native.load()
     T, K = x.shape
     topk = idx.shape[1]
@@ -297,10 +299,10 @@ def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=No
     if out is None:
         out = torch.empty(T, topk, gate.N, dtype=torch.bfloat16, device=x.device)
     check(
-        lib.exo_gather_qmv_swiglu(
-            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
-            _ptr(up.scales), _ptr(up.biases), _ptr(idx), _ptr(out), T, topk, E, gate.N, K,
-            gate.bits, gate.group_size, _stream(),
+        lib.exo_norm_gather_qmv_swiglu(
+            _ptr(x), _ptr(norm_weight), eps, _ptr(gate.weight), _ptr(gate.scales),
+            _ptr(gate.biases), _ptr(up.weight), _ptr(up.scales), _ptr(up.biases), _ptr(idx),
+            _ptr(out), T, topk, E, gate.N, K, gate.bits, gate.group_size, _stream(),
         ),
         "gather_qmv_swiglu",
     )

@@ -131,6 +131,15 @@ int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, const uint16_t*
                           int topk, int E, int N, int K, int bits, int group_size,
                           exo_stream_t stream);
 
+/* exo_gather_qmv_swiglu with rms_norm(x, norm_weight, eps) applied to every token row
+ * first (norm_weight == NULL: no norm), so that a MoE block's post-attention norm needs no
+ * launch of its own in decode. */
+int exo_norm_gather_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                               const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                               const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
+                               const int32_t* idx, uint16_t* y, int T, int topk, int E, int N,
+                               int K, int bits, int group_size, exo_stream_t stream);
+
 /* K5: mx.fast.rms_norm with the preceding residual add fused:
  *   h = residual ? bf16(x + residual) : x ;  h_out = h (may be null) ;
  *   n_out = bf16(h * rsqrt(mean(h^2)+eps) * weight).
