@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (1..16)")
     ap.add_argument("--shard-layers", type=int, default=None,
                     help="run layers [0, n) as a first pipeline shard (output: hidden state)")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also launch one plain 256 MiB copy kernel: the known-size dispatch that "
+                         "calibrates FETCH_SIZE / WRITE_SIZE in a rocprofv3 --pmc pass")
     ap.add_argument("--workload", default="decode", choices=["decode", "qmatmul_sweep"],
                     help="decode (default, the headline) or the quantised-matmul shape sweep")
     return ap.parse_args()
@@ -202,6 +205,23 @@ def cpu_baseline(model, torch, seconds: float, context: int):
                 host_cpus=os.cpu_count(), affinity=len(os.sched_getaffinity(0)))
 
 
+def pmc_traffic(launch: str):
+    """HBM bytes per launch of one GEMV group as measured by the committed
+    `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` passes of this command (a text summary
+    under profiles/; counters cannot be read from inside the process).  None if absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                        "decode_llama8b_4bit_bs1_pmc_traffic.md")
+    try:
+        with open(path) as fh:
+            for line in fh:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == launch:
+                    return int(parts[2])
+    except OSError:
+        pass
+    return None
+
+
 def active_token_bytes(model, cfg, ctx: int, batch: int) -> int:
     """Algorithmic HBM bytes of one decode step: every weight the step multiplies by (for
     MoE layers the router plus top-k experts per sequence, at most all experts) once,
@@ -358,6 +378,15 @@ def main():
     tok_s = B * K / dt
     token_bytes = active_token_bytes(model, cfg, ctx0, B)
 
+    if args.pmc_copy:
+        # plain 16-byte-per-lane copy of 256 MiB (the KV re-layout kernel with one head is
+        # exactly that): reads 256 MiB, writes 256 MiB
+        from exo_amd import ops
+        a = torch.zeros(1, 1 << 20, 128, dtype=torch.bfloat16, device=dev)
+        ops.kv_export_nhd(a, 0, 1 << 20)
+        torch.cuda.synchronize()
+        del a
+
     headline = (args.config == "llama-3.1-8b" and B == 1 and model.is_last and not cfg.is_moe)
     if not cfg.is_moe and model.is_last and B == 1:
         kernels = measure_kernels(model, torch)
@@ -368,7 +397,8 @@ def main():
         gemv_us = sum(k["us_per_token"] for k in kernels)
         gemv_bytes = sum(k["bytes_per_launch"] * k["launches_per_token"] for k in kernels)
         roofline = dict(bound="hbm", achieved=dom["GBps"], peak=8000.0, unit="GB/s",
-                        frac=dom["GBps"] / 8000.0, traffic=None, kernel=dom["kernel"],
+                        frac=dom["GBps"] / 8000.0,
+                        traffic=pmc_traffic(dom["name"]) if headline else None, kernel=dom["kernel"],
                         launch=dom["name"], avg_us=dom["avg_us"], bytes_per_launch=dom["bytes_per_launch"],
                         all_gemv_GBps=gemv_bytes / gemv_us * 1e-3, all_gemv_us_per_token=gemv_us)
     else:
