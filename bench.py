@@ -312,7 +312,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (per-shard forward); --gpus {args.gpus} is not "
-              "supported. Multi-GPU pipeline/tensor sharding is design-only (see DESIGN.md).",
+              "supported: every figure here is one GPU's throughput.",
               file=sys.stderr)
         sys.exit(2)
     if args.workload == "qmatmul_sweep":

@@ -1,14 +1,21 @@
 // Quantised matmul for prefill (any M): y[M,N] = x[M,K] @ dq(W)[N,K]^T.
 //
-// Matrix-core design for gfx950: a 256x128 (128x128 for M <= 128) output tile per
-// 256-thread workgroup, one 64-wide K step per iteration = exactly one quantisation group,
-// so every packed row segment needs a single (scale, bias).  Each thread dequantises 32 (4-bit) or
-// 2x16 (8-bit) codes to bf16 in registers - bf16(fma(s, q, b)), codes converted with
-// v_cvt_f32_ubyteN - and stores them to LDS next to the activation tile; the four
-// waves (2x2) then issue v_mfma_f32_32x32x16_bf16 on 128x64 (64x64) sub-tiles with float32
-// accumulators: the taller tile halves both the dequantisation work and the LDS bytes
-// read per MFMA.  Global loads of the next K step are issued before the MFMAs of the
-// current one.  LDS rows are padded by 16 bytes to keep ds_read_b128 conflict-free.
+// Matrix-core design for gfx950.  A 256-thread workgroup (2 x 2 waves) computes a
+// 256x128 output tile (128x128 for M <= 128); one 64-wide K step per iteration = exactly
+// one quantisation group, so a packed row segment needs a single (scale, bias).
+//  * Activations go through LDS (two buffers: the next tile is stored while the current
+//    one is multiplied, one barrier per K step).  LDS bandwidth, not the matrix cores, is
+//    what limits this kernel, so the weights do NOT go through LDS:
+//  * every wave loads the packed words of its own 64 weight rows straight into registers
+//    in the MFMA B-operand layout - lane (row, half) takes 16 B (4-bit) or 32 B (8-bit) =
+//    32 consecutive codes - and dequantises them there to bf16(fma(s, q, b)) with
+//    v_cvt_f32_ubyteN.  MFMA step t of a K step then covers k = 32*half + 8*t .. +8, and
+//    the A operand is read from the activation tile at that same offset, so no data is
+//    rearranged.  The two waves that share weight rows dequantise them twice; in exchange
+//    the LDS carries a third less traffic and its writes are plain copies.
+//  * v_mfma_f32_32x32x16_bf16, float32 accumulators (128x64 per wave), global loads two
+//    K steps ahead in registers.  LDS rows are padded by 16 bytes: conflict-free b128.
+//  * grouped mode (MoE prefill): blockIdx.y is a tile of one expert's sorted rows.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 
@@ -34,30 +41,50 @@ struct QmmParams {
   size_t w_stride, s_stride;  // elements between consecutive experts
 };
 
-template <int BITS>
-struct WFrag {  // one thread's share of the packed W tile for one K step
-  uint4 q[BITS / 4];  // 4-bit: 16 B = 32 codes; 8-bit: 2 x 16 B = 2 x 16 codes
-  float s, b;
-};
-
 __device__ __forceinline__ float ubyte_f(uint32_t v, int i) {
   return (float)((v >> (8 * i)) & 0xffu);  // v_cvt_f32_ubyteN
 }
 
-// The workgroup is 2 x WN waves; a wave computes (32*MI) x 64 outputs, so the tile is
-// (64*MI) x (64*WN).  STAGES = K steps whose global loads are in flight (held in
-// registers) while the current step is multiplied.
-template <int BITS, int MI, int WN, int STAGES, bool GROUPED = false>
-__global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
-  constexpr int kThreads = 128 * WN;
-  constexpr int BM = 64 * MI, BN = 64 * WN;
+// packed codes of one (weight row, half of a K step): 32 codes
+template <int BITS>
+struct WRaw {
+  uint4 q[BITS / 4];
+  bf16_t s, b;
+};
+
+// 8 codes -> the bf16x8 B operand of one MFMA step
+template <int BITS>
+__device__ __forceinline__ bf16x8_t dequant8(const WRaw<BITS>& r, int t, float s, float b) {
+  uint4 o;
+  if (BITS == 4) {
+    const uint32_t v = reinterpret_cast<const uint32_t*>(&r.q[0])[t];
+    const uint32_t ev = v & 0x0f0f0f0fu, od = (v >> 4) & 0x0f0f0f0fu;
+    o.x = pack_bf2(fmaf(s, ubyte_f(ev, 0), b), fmaf(s, ubyte_f(od, 0), b));
+    o.y = pack_bf2(fmaf(s, ubyte_f(ev, 1), b), fmaf(s, ubyte_f(od, 1), b));
+    o.z = pack_bf2(fmaf(s, ubyte_f(ev, 2), b), fmaf(s, ubyte_f(od, 2), b));
+    o.w = pack_bf2(fmaf(s, ubyte_f(ev, 3), b), fmaf(s, ubyte_f(od, 3), b));
+  } else {
+    const uint32_t v0 = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t];
+    const uint32_t v1 = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t + 1];
+    o.x = pack_bf2(fmaf(s, ubyte_f(v0, 0), b), fmaf(s, ubyte_f(v0, 1), b));
+    o.y = pack_bf2(fmaf(s, ubyte_f(v0, 2), b), fmaf(s, ubyte_f(v0, 3), b));
+    o.z = pack_bf2(fmaf(s, ubyte_f(v1, 0), b), fmaf(s, ubyte_f(v1, 1), b));
+    o.w = pack_bf2(fmaf(s, ubyte_f(v1, 2), b), fmaf(s, ubyte_f(v1, 3), b));
+  }
+  return __builtin_bit_cast(bf16x8_t, o);
+}
+
+// MI = 32-row MFMA tiles per wave along M: the workgroup tile is (64*MI) x 128.
+template <int BITS, int MI, bool GROUPED = false>
+__global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
+  constexpr int kThreads = 256;
+  constexpr int BM = 64 * MI, BN = 128;
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
-  __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t ws[BN * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * BN;
-  const int wm = (wave / WN) * (32 * MI), wn = (wave % WN) * 64;
+  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 64;
   const int G = p.K >> 6;
   const int wpr = p.K * BITS / 32;
   int m0 = blockIdx.y * BM, m_end = p.M;
@@ -75,19 +102,30 @@ __global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
     __syncthreads();
   }
 
-  // W: thread -> (row, part): 2 parts of 32 codes per row and K step
-  const int w_row = tid >> 1, w_part = tid & 1;
-  const bool w_ok = (n0 + w_row) < p.N;
-  const uint32_t* wsrc = p.w + w_off + (size_t)(n0 + (w_ok ? w_row : 0)) * wpr + w_part * (BITS);
-  const bf16_t* ssrc = p.s + s_off + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
-  const bf16_t* bsrc = p.b + s_off + (size_t)(n0 + (w_ok ? w_row : 0)) * G;
+  // weight rows of this lane: column tile j -> row n0 + wn + 32*j + lane%32, half lane/32
+  const int frow = lane & 31, kq = lane >> 5;
+  const uint32_t* wsrc[2];
+  const bf16_t* ssrc[2];
+  const bf16_t* bsrc[2];
+  bool w_ok[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn + j * 32 + frow;
+    w_ok[j] = n < p.N;
+    const size_t row = (size_t)(w_ok[j] ? n : 0);
+    wsrc[j] = p.w + w_off + row * wpr + kq * BITS;  // 32 codes = BITS words per half K step
+    ssrc[j] = p.s + s_off + row * G;
+    bsrc[j] = p.b + s_off + row * G;
+  }
 
-  struct Stage {
+  struct XStage {
     uint4 xa[XR];
-    WFrag<BITS> wf;
+  };
+  struct WStage {
+    WRaw<BITS> w[2];
   };
 
-  auto load_global = [&](Stage& st, int k0) {
+  auto load_x = [&](XStage& st, int k0) {
 #pragma unroll
     for (int r = 0; r < XR; ++r) {
       const int id = tid + kThreads * r;
@@ -95,60 +133,29 @@ __global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
       if (m0 + row < m_end) {
         const size_t src = GROUPED ? (size_t)(row_pair[row] / p.x_div) : (size_t)(m0 + row);
         st.xa[r] = *reinterpret_cast<const uint4*>(p.x + src * p.K + k0 + kp * 8);
-      } else
+      } else {
         st.xa[r] = make_uint4(0, 0, 0, 0);
+      }
     }
+  };
+  auto load_w = [&](WStage& st, int k0) {
     const int kw = k0 * BITS / 32;  // word offset of this K step
 #pragma unroll
-    for (int i = 0; i < BITS / 4; ++i)
-      st.wf.q[i] = *reinterpret_cast<const uint4*>(wsrc + kw + i * 4);
-    st.wf.s = bf2f(ssrc[k0 >> 6]);
-    st.wf.b = bf2f(bsrc[k0 >> 6]);
-    if (!w_ok) {
-      st.wf.s = 0.f;
-      st.wf.b = 0.f;
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int i = 0; i < BITS / 4; ++i)
+        st.w[j].q[i] = *reinterpret_cast<const uint4*>(wsrc[j] + kw + i * 4);
+      st.w[j].s = ssrc[j][k0 >> 6];
+      st.w[j].b = bsrc[j][k0 >> 6];
     }
   };
 
-  auto store_lds = [&](const Stage& st) {
+  auto store_x = [&](const XStage& st, int buf) {
 #pragma unroll
     for (int r = 0; r < XR; ++r) {
       const int id = tid + kThreads * r;
       const int row = id >> 3, kp = id & 7;
-      *reinterpret_cast<uint4*>(&xs[row * LDS_STRIDE + kp * 8]) = st.xa[r];
-    }
-    bf16_t* dst = &ws[w_row * LDS_STRIDE + w_part * 32];
-    const float s = st.wf.s, b = st.wf.b;
-    const uint32_t* qw = reinterpret_cast<const uint32_t*>(&st.wf.q[0]);
-    if (BITS == 4) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {  // 2 words = 16 codes = two 16-byte LDS stores
-        uint4 o[2];
-        uint32_t* o4 = reinterpret_cast<uint32_t*>(o);
-#pragma unroll
-        for (int wi = 0; wi < 2; ++wi) {
-          const uint32_t v = qw[h * 2 + wi];
-          const uint32_t ev = v & 0x0f0f0f0fu, od = (v >> 4) & 0x0f0f0f0fu;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            o4[wi * 4 + e] = pack_bf2(fmaf(s, ubyte_f(ev, e), b), fmaf(s, ubyte_f(od, e), b));
-        }
-        *reinterpret_cast<uint4*>(dst + h * 16) = o[0];
-        *reinterpret_cast<uint4*>(dst + h * 16 + 8) = o[1];
-      }
-    } else {
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {  // 8 codes (2 words) per 16-byte LDS store
-        uint4 o;
-        uint32_t* o4 = reinterpret_cast<uint32_t*>(&o);
-#pragma unroll
-        for (int wi = 0; wi < 2; ++wi) {
-          const uint32_t v = qw[h * 2 + wi];
-          o4[wi * 2] = pack_bf2(fmaf(s, ubyte_f(v, 0), b), fmaf(s, ubyte_f(v, 1), b));
-          o4[wi * 2 + 1] = pack_bf2(fmaf(s, ubyte_f(v, 2), b), fmaf(s, ubyte_f(v, 3), b));
-        }
-        *reinterpret_cast<uint4*>(dst + h * 8) = o;
-      }
+      *reinterpret_cast<uint4*>(&xs[buf][row * LDS_STRIDE + kp * 8]) = st.xa[r];
     }
   };
 
@@ -160,17 +167,23 @@ __global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int frow = lane & 31, fk = (lane >> 5) * 8;
-  auto multiply = [&]() {
+  // multiply tile `buf` by the weights held (packed) in `st`
+  auto multiply = [&](const WStage& st, int buf) {
+    float sc[2], bi[2];
 #pragma unroll
-    for (int ks = 0; ks < BK; ks += 16) {
+    for (int j = 0; j < 2; ++j) {
+      sc[j] = w_ok[j] ? bf2f(st.w[j].s) : 0.f;
+      bi[j] = w_ok[j] ? bf2f(st.w[j].b) : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {  // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step
       bf16x8_t a[MI], bq[2];
 #pragma unroll
       for (int i = 0; i < MI; ++i)
-        a[i] = *reinterpret_cast<const bf16x8_t*>(&xs[(wm + i * 32 + frow) * LDS_STRIDE + ks + fk]);
+        a[i] = *reinterpret_cast<const bf16x8_t*>(
+            &xs[buf][(wm + i * 32 + frow) * LDS_STRIDE + kq * 32 + t * 8]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        bq[j] = *reinterpret_cast<const bf16x8_t*>(&ws[(wn + j * 32 + frow) * LDS_STRIDE + ks + fk]);
+      for (int j = 0; j < 2; ++j) bq[j] = dequant8<BITS>(st.w[j], t, sc[j], bi[j]);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -179,54 +192,90 @@ __global__ __launch_bounds__(128 * WN, 2) void qmm_kernel(const QmmParams p) {
     }
   };
 
-  // one K step: stage `st` (loaded STAGES steps ago) goes to LDS, is refilled with the
-  // step STAGES ahead, and the tile is multiplied
-  auto step = [&](Stage& st, int k0) {
-    __syncthreads();  // previous step's LDS reads are done
-    store_lds(st);
+  // At K step k: the x tile of k is in LDS buffer k&1, the x tile of k+1 in registers
+  // (xr), the packed weights of k and k+1 in w0 / w1.  Per step: the next x tile goes to
+  // the other LDS buffer and its registers are refilled two steps ahead, the current tile
+  // is multiplied, the freed weight stage is refilled two steps ahead; one barrier.
+  XStage xr;
+  WStage w0, w1;
+  load_x(xr, 0);
+  load_w(w0, 0);
+  store_x(xr, 0);
+  if (BK < p.K) {
+    load_x(xr, BK);
+    load_w(w1, BK);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    if (k0 + BK < p.K) store_x(xr, buf ^ 1);
+    if (k0 + 2 * BK < p.K) load_x(xr, k0 + 2 * BK);
+    multiply(w0, buf);
+    w0 = w1;  // a few register moves keep the loop body single (no unrolled twin)
+    if (k0 + 2 * BK < p.K) load_w(w1, k0 + 2 * BK);
     __syncthreads();
-    if (k0 + STAGES * BK < p.K) load_global(st, k0 + STAGES * BK);
-    multiply();
-  };
-
-  Stage st[STAGES];
-#pragma unroll
-  for (int i = 0; i < STAGES; ++i)
-    if (i * BK < p.K) load_global(st[i], i * BK);
-  for (int k0 = 0; k0 < p.K; k0 += STAGES * BK) {
-#pragma unroll
-    for (int i = 0; i < STAGES; ++i)
-      if (k0 + i * BK < p.K) step(st[i], k0 + i * BK);
+    buf ^= 1;
   }
 
-  // D[i][j]: column j = lane%32 (W row n), rows 8*(r/4) + 4*(lane/32) + r%4 (token m)
+  // Epilogue through LDS.  D[i][j] holds column lane%32 (W row n) and rows
+  // 8*(r/4) + 4*(lane/32) + r%4 (token m): a wave first writes its (32*MI) x 64 tile as bf16
+  // into its own slice of the (now idle) activation buffers - 2-byte LDS stores at constant
+  // offsets from one base, so no address lives in registers next to the accumulators -
+  // and then copies whole rows out with 16-byte stores (residual added on the way).
+  __syncthreads();  // every wave has finished reading the last activation tile
+  constexpr int TS = 64 + 8;  // row stride of the staging tile (bf16)
+  bf16_t* stage = &xs[0][0] + (size_t)wave * (32 * MI) * TS;
+  {
+    bf16_t* sp = stage + (kq * 4) * TS + frow;
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn + j * 32 + (lane & 31);
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (m < m_end && n < p.N) {
-          const size_t o = (size_t)(GROUPED ? row_pair[m] : m) * p.N + n;
-          float v = acc[i][j][r];
-          if (p.residual) v = bf2f(f2bf(v)) + bf2f(p.residual[o]);
-          p.y[o] = f2bf(v);
-        }
+        for (int r = 0; r < 16; ++r)
+          sp[(i * 32 + (r >> 2) * 8 + (r & 3)) * TS + j * 32] = f2bf(acc[i][j][r]);
+  }
+  // the slice is private to the wave: its own LDS writes are complete before its reads
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  const bool vec_ok = (p.N & 7) == 0;
+  const int c8 = (lane & 7) * 8;  // first of this lane's 8 columns
+  for (int it = 0; it < 4 * MI; ++it) {
+    const int row = it * 8 + (lane >> 3);  // row of the wave's tile
+    const int m = m0 + wm + row, n = n0 + wn + c8;
+    if (m >= m_end || n >= p.N) continue;
+    const size_t o = (size_t)(GROUPED ? row_pair[m] : m) * p.N + n;
+    uint4 v = *reinterpret_cast<const uint4*>(stage + row * TS + c8);
+    if (vec_ok) {
+      if (p.residual) {
+        const uint4 rv = *reinterpret_cast<const uint4*>(p.residual + o);
+        v.x = pack_bf2(bf_lo(v.x) + bf_lo(rv.x), bf_hi(v.x) + bf_hi(rv.x));
+        v.y = pack_bf2(bf_lo(v.y) + bf_lo(rv.y), bf_hi(v.y) + bf_hi(rv.y));
+        v.z = pack_bf2(bf_lo(v.z) + bf_lo(rv.z), bf_hi(v.z) + bf_hi(rv.z));
+        v.w = pack_bf2(bf_lo(v.w) + bf_lo(rv.w), bf_hi(v.w) + bf_hi(rv.w));
+      }
+      *reinterpret_cast<uint4*>(p.y + o) = v;
+    } else {  // N not a multiple of 8: rows are not 16-byte aligned
+      const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (n + c >= p.N) break;
+        float f = (c & 1) ? bf_hi(w4[c >> 1]) : bf_lo(w4[c >> 1]);
+        if (p.residual) f += bf2f(p.residual[o + c]);
+        p.y[o + c] = f2bf(f);
       }
     }
+  }
 }
 
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
-  // up to 128 rows: little arithmetic per K step, so several steps' loads are kept in
-  // flight; taller inputs: 256-row tiles halve the dequantisation work per output
+  // taller inputs: 256-row tiles halve the dequantisation work and the LDS reads per output
   if (M <= 128)
-    qmm_kernel<BITS, 2, 2, 2><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), 256, 0, st>>>(p);
+    qmm_kernel<BITS, 2><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), 256, 0, st>>>(p);
   else
-    qmm_kernel<BITS, 4, 2, 1><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 256)), 256, 0, st>>>(p);
+    qmm_kernel<BITS, 4><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 256)), 256, 0, st>>>(p);
 }
 
 constexpr int kGroupBM = 128;  // rows per tile of the grouped GEMM
@@ -328,9 +377,9 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   p.s_stride = (size_t)N * (K / 64);
   const dim3 grid(exo_ceil_div(N, 128), max_tiles);
   if (bits == 4)
-    qmm_kernel<4, 2, 2, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    qmm_kernel<4, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
   else
-    qmm_kernel<8, 2, 2, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    qmm_kernel<8, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
   EXO_CHECK_LAUNCH("exo_gather_qmm");
   return EXO_OK;
 }
