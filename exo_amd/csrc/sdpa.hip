@@ -45,6 +45,9 @@ struct SdpaParams {
   const bf16_t* qn;         // [D] or null
   const bf16_t* kn;
   float eps;
+  // decode: the Hq/Hkv query heads of a kv head are handled by `hgroups` workgroups of G
+  // heads each (blockIdx.y = kv head * hgroups + group); set by the launcher
+  int hgroups;
 };
 
 // Sum over the LPK lanes of a key's lane group.  16 lanes are one DPP row: four
@@ -135,7 +138,10 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane / LPK, sl = lane % LPK;
-  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int b = blockIdx.z;
+  const int kvh = DECODE ? (int)blockIdx.y / p.hgroups : (int)blockIdx.y;
+  const int hg = DECODE ? (int)blockIdx.y % p.hgroups : 0;
+  const int h0 = kvh * (G * (DECODE ? p.hgroups : 1)) + hg * G;  // first query head of this workgroup
   const int t = DECODE ? 0 : blockIdx.x;
   const int len = min(p.pos[b] + t + 1, p.S_max);  // keys visible to this query
   int k_begin = 0, k_end = len;
@@ -202,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     const bf16_t* row = p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
 #pragma unroll
     for (int g = 0; g < G; ++g)
-      qv[g] = head_slice<D, true>(row + (size_t)(kvh * G + g) * D, sl, p.qn, p.eps, cs, sn);
+      qv[g] = head_slice<D, true>(row + (size_t)(h0 + g) * D, sl, p.qn, p.eps, cs, sn);
     if (own_new && wave == 0) {
       knew = head_slice<D, true>(row + (size_t)(p.Hq + kvh) * D, sl, p.kn, p.eps, cs, sn);
       vnew = head_slice<D, false>(row + (size_t)(p.Hq + p.Hkv + kvh) * D, sl, nullptr, 0.f, cs, sn);
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   } else {
 #pragma unroll
     for (int g = 0; g < G; ++g)
-      qv[g] = *reinterpret_cast<const uint4*>(p.q + qrow + (size_t)(kvh * G + g) * D + sl * 8);
+      qv[g] = *reinterpret_cast<const uint4*>(p.q + qrow + (size_t)(h0 + g) * D + sl * 8);
   }
 
   float m[G], l[G], o[G][8];
@@ -289,7 +295,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
       tn.v[i] = i == 0 ? vnew : make_uint4(0, 0, 0, 0);
     }
     consume(tn, len - 1, len);
-    if (sub == 0) {
+    if (sub == 0 && hg == 0) {  // one of the head groups appends to the cache
       const size_t o = head_base + (size_t)(len - 1) * D + sl * 8;
       *reinterpret_cast<uint4*>(const_cast<bf16_t*>(p.kc) + o) = knew;
       *reinterpret_cast<uint4*>(const_cast<bf16_t*>(p.vc) + o) = vnew;
@@ -338,7 +344,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
       acc += red[w][g][e] * sc;
       lsum += red[w][g][D + 1] * sc;
     }
-    const int h = kvh * G + g;
+    const int h = h0 + g;
     if (DECODE) {
       // device-scope (write-through) stores: the merging workgroup may run on another
       // XCD, whose L2 is not coherent with this one
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) {
-    int* cnt = &p.counters[b * p.Hkv + kvh];
+    int* cnt = &p.counters[b * p.Hkv * p.hgroups + blockIdx.y];
     const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = (old == p.splits - 1);
     if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -371,7 +377,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   if (!s_last) return;
   for (int idx = threadIdx.x; idx < G * D; idx += kThreads) {
     const int g = idx / D, e = idx % D;
-    const int h = kvh * G + g;
+    const int h = h0 + g;
     const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
     // all loads of all splits are issued before any is used (they miss every cache)
     constexpr int MS = max_splits(G);
@@ -399,7 +405,9 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
 }
 
 int pick_splits(int B, int Hq, int Hkv, int S_max) {
-  int s = 256 / (B * Hkv);
+  const int G = Hq / Hkv;
+  const int hgroups = (G > 4 && G % 4 == 0) ? G / 4 : 1;  // as in launch_sdpa
+  int s = 256 / (B * Hkv * hgroups);
   int cap = S_max / 64;
   if (s > cap) s = cap;
   if (s > max_splits(Hq / Hkv)) s = max_splits(Hq / Hkv);
@@ -408,9 +416,18 @@ int pick_splits(int B, int Hq, int Hkv, int S_max) {
 }
 
 template <int D, int MODE>
-int launch_sdpa(const SdpaParams& p, hipStream_t st) {
-  const int G = p.Hq / p.Hkv;
-  dim3 grid(MODE != 0 ? p.splits : p.T, p.Hkv, p.B);
+int launch_sdpa(const SdpaParams& p0, hipStream_t st) {
+  SdpaParams p = p0;
+  int G = p.Hq / p.Hkv;
+  p.hgroups = 1;
+  // decode: more than 4 query heads per kv head are spread over several workgroups (each
+  // re-reads the K/V range from L2): the per-key arithmetic of a workgroup grows with its
+  // head count, and kv-head counts of 4 would otherwise leave half the chip idle
+  if (MODE != 0 && G > 4 && G % 4 == 0) {
+    p.hgroups = G / 4;
+    G = 4;
+  }
+  dim3 grid(MODE != 0 ? p.splits : p.T, p.Hkv * p.hgroups, p.B);
   switch (G) {
     case 1: sdpa_kernel<D, 1, MODE><<<grid, kThreads, 0, st>>>(p); break;
     case 2: sdpa_kernel<D, 2, MODE><<<grid, kThreads, 0, st>>>(p); break;
