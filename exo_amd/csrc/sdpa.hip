@@ -25,7 +25,6 @@ constexpr int kWaves = 4;
 constexpr int kMaxSplits = 16;
 // More splits than 16 were slower for every head layout measured (4 and 8 kv heads): the
 // merge by the last workgroup grows with the split count.
-constexpr int max_splits(int) { return kMaxSplits; }
 constexpr int kBlk = 4;  // keys per lane group per step
 
 struct SdpaParams {
@@ -380,7 +379,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     const int h = h0 + g;
     const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
     // all loads of all splits are issued before any is used (they miss every cache)
-    constexpr int MS = max_splits(G);
+    constexpr int MS = kMaxSplits;
     float pm[MS], pl[MS], po[MS];
 #pragma unroll
     for (int sp = 0; sp < MS; ++sp) {
@@ -404,13 +403,24 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   }
 }
 
-int pick_splits(int B, int Hq, int Hkv, int S_max) {
+// Decode work split.  The G = Hq/Hkv query heads of a kv head are spread over `hgroups`
+// workgroups (each re-reads the K/V range from L2, but the per-key arithmetic, the register
+// footprint and the in-wave merge of a workgroup shrink with its head count): as many as
+// keep (sequences x kv heads x groups) within 64, so that at least 4 key splits remain at
+// about 256 workgroups in total.  Batch 1: one head per workgroup, 8 splits (measured on
+// Llama-3.1-8B and Qwen3: faster than 2 or 4 heads per workgroup; 128 and 512 workgroups
+// slower).  Batch 8 with 8 kv heads: all 4 heads in one workgroup, 4 splits.
+int pick_hgroups(int B, int Hq, int Hkv) {
   const int G = Hq / Hkv;
-  const int hgroups = G;  // as in launch_sdpa
-  int s = 256 / (B * Hkv * hgroups);  // about 256 workgroups measured best (128 and 512 slower)
+  int h = 1;
+  while (h * 2 <= G && G % (h * 2) == 0 && B * Hkv * h * 2 <= 64) h *= 2;
+  return h;
+}
+int pick_splits(int B, int Hq, int Hkv, int S_max) {
+  int s = 256 / (B * Hkv * pick_hgroups(B, Hq, Hkv));
   int cap = S_max / 64;
   if (s > cap) s = cap;
-  if (s > max_splits(Hq / Hkv)) s = max_splits(Hq / Hkv);
+  if (s > kMaxSplits) s = kMaxSplits;
   if (s < 1) s = 1;
   return s;
 }
@@ -420,14 +430,9 @@ int launch_sdpa(const SdpaParams& p0, hipStream_t st) {
   SdpaParams p = p0;
   int G = p.Hq / p.Hkv;
   p.hgroups = 1;
-  // decode: one query head per workgroup.  The G heads of a kv head re-read its K/V range
-  // (from L2), but the per-key arithmetic, the register footprint and the in-wave merge of
-  // a workgroup all shrink with its head count, and 32 heads x 8 splits fill the chip;
-  // measured on Llama-3.1-8B (4 heads per kv head) and Qwen3 (8, 16): faster than 2 or 4
-  // heads per workgroup.
-  if (MODE != 0 && G > 1) {
-    p.hgroups = G;
-    G = 1;
+  if (MODE != 0) {
+    p.hgroups = pick_hgroups(p.B, p.Hq, p.Hkv);
+    G /= p.hgroups;
   }
   dim3 grid(MODE != 0 ? p.splits : p.T, p.Hkv * p.hgroups, p.B);
   switch (G) {
