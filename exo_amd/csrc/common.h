@@ -53,6 +53,33 @@ __device__ __forceinline__ float group_sum(float v, int width) {
   return v;
 }
 
+// ---- cross-lane sums on the DPP path (no LDS traffic) ----
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+// sum over the wave; the total lands in lane 63
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_get<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+  v += dpp_get<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+  v += dpp_get<0x141, 0xf>(v);  // row_half_mirror
+  v += dpp_get<0x140, 0xf>(v);  // row_mirror: every lane holds its row-of-16 total
+  v += dpp_get<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_get<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// sum over aligned runs of W (8 or 16) lanes, in every lane of the run
+template <int W>
+__device__ __forceinline__ float run_sum(float v) {
+  v += dpp_get<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+  v += dpp_get<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+  v += dpp_get<0x141, 0xf>(v);  // row_half_mirror
+  if (W == 16) v += dpp_get<0x140, 0xf>(v);  // row_mirror
+  return v;
+}
+
 // ---- host side -------------------------------------------------------------
 #define EXO_OK 0
 #define EXO_ERR_ARG (-1)

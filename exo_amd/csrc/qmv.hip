@@ -479,22 +479,6 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
 // (u * 64>>GSHIFT elements) linearly: no per-unit address arithmetic beyond a scalar
 // add.  ITERS is a template parameter: the per-row loop, the LDS offsets of x and the
 // point where a row ends are all static.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_get(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
-}
-// sum over the wave; the total lands in lane 63
-__device__ __forceinline__ float wave_sum_to_lane63(float v) {
-  v += dpp_get<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
-  v += dpp_get<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-  v += dpp_get<0x141, 0xf>(v);  // row_half_mirror
-  v += dpp_get<0x140, 0xf>(v);  // row_mirror: every lane holds its row-of-16 total
-  v += dpp_get<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v += dpp_get<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-  return v;
-}
-
 template <int BITS, int MT, int NMAT, int ITERS>
 __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   extern __shared__ uint4 smem[];

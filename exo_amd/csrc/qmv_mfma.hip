@@ -12,9 +12,10 @@
 //  * D[m][r] of a whole group is scaled on the way out:
 //      acc += s[r,g] * (D - 128*Sx[m,g]) + b[r,g] * Sx[m,g]
 //    with the group sums Sx of the activations precomputed in LDS;
-//  * four waves split the K range of one block of 32 rows; their partial sums meet in
-//    LDS once per block.  A workgroup holds NG such wave quartets, which share the
-//    staged activations (the staging cost per weight byte falls with NG);
+//  * KW waves (4, 8 or 16) split the K range of one block of 32 rows; their partial sums
+//    meet in LDS once per block.  Few row blocks: many waves per block, so that the
+//    grid is wide without a merge through memory.  Many row blocks: KW = 4 and NG such
+//    wave teams per workgroup, which share the staged activations;
 //  * with a workspace, K is also split over workgroups (blockIdx.y): 16 rows then fit
 //    the LDS at any K and a short N still fills the chip; the last workgroup of a row
 //    block to arrive adds the float32 partials in a fixed order.
@@ -23,8 +24,6 @@
 #include "qmv_internal.h"
 
 namespace {
-
-constexpr int kWaves = 4;  // waves that share one block of 32 output rows (they split K)
 
 struct MfmaParams {
   const bf16_t* x;         // [M,K]
@@ -57,13 +56,10 @@ __device__ __forceinline__ uint4 load_word_x(const bf16_t* base, int wi) {
   return make_uint4(v.x, v.y, 0, 0);
 }
 template <int BITS>
-__device__ __forceinline__ float sumsq_word(const uint4& v) {
-  float s = bf_lo(v.x) * bf_lo(v.x) + bf_hi(v.x) * bf_hi(v.x) + bf_lo(v.y) * bf_lo(v.y) +
-            bf_hi(v.y) * bf_hi(v.y);
-  if (BITS == 4)
-    s += bf_lo(v.z) * bf_lo(v.z) + bf_hi(v.z) * bf_hi(v.z) + bf_lo(v.w) * bf_lo(v.w) +
-         bf_hi(v.w) * bf_hi(v.w);
-  return s;
+__device__ __forceinline__ float sumsq_word(const uint4& v, float acc) {
+  acc = dot2_bf16(v.x, v.x, dot2_bf16(v.y, v.y, acc));
+  if (BITS == 4) acc = dot2_bf16(v.z, v.z, dot2_bf16(v.w, v.w, acc));
+  return acc;
 }
 template <int BITS>
 __device__ __forceinline__ void norm_word(uint4& xv, const uint4& wv, float inv) {
@@ -74,18 +70,20 @@ __device__ __forceinline__ void norm_word(uint4& xv, const uint4& wv, float inv)
     xv.w = pack_bf2(bf_lo(xv.w) * inv * bf_lo(wv.w), bf_hi(xv.w) * inv * bf_hi(wv.w));
   }
 }
-// activations of one packed word in the register order of the unpacked nibble pairs
+// activations of one packed word in the register order of the unpacked nibble pairs;
+// `sum` = sum of the word's activations.  (8-bit: the operand holds every activation twice,
+// as x against the low nibble and 16x against the high one, so the sum of the stored
+// values is exactly 17 times the sum of the activations.)
 template <int BITS>
-__device__ __forceinline__ uint4 permute_word(const uint4& xv, float& stored, float& truesum) {
+__device__ __forceinline__ uint4 permute_word(const uint4& xv, float& sum) {
+  constexpr uint32_t kOnes = 0x3F803F80u;  // bf16 (1, 1)
   uint4 o;
   if (BITS == 4) {
     o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
     o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
     o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
     o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
-    truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
-              (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
-    stored = truesum;
+    sum = dot2_bf16(o.x, kOnes, dot2_bf16(o.y, kOnes, dot2_bf16(o.z, kOnes, dot2_bf16(o.w, kOnes, 0.f))));
   } else {  // byte codes as two nibbles against (x, 16x)
     const uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);   // (x0,x2)
     const uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u);  // (x1,x3)
@@ -93,37 +91,42 @@ __device__ __forceinline__ uint4 permute_word(const uint4& xv, float& stored, fl
     o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
     o.z = c2;
     o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
-    truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
-    stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
+    sum = dot2_bf16(a, kOnes, dot2_bf16(c2, kOnes, 0.f));
   }
   return o;
 }
 
-// MR = D registers in use: 4 covers M <= 8, 8 covers M <= 16.  NG = wave quartets per
-// workgroup.  SPS = 16-byte loads in flight per lane and buffer (a "super-step").
-template <int BITS, int MR, int NG, int SPS>
-__global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) {
-  constexpr int kThreads = 256 * NG;
+// MR = D registers in use: 4 covers M <= 8, 8 covers M <= 16.  KW = waves that split K
+// for one row block, NG = such wave teams per workgroup.  SPS = 16-byte loads in flight
+// per lane and buffer (a "super-step").
+template <int BITS, int MR, int KW, int NG, int SPS>
+__global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams p) {
+  constexpr int kThreads = 64 * KW * NG;
   constexpr int WPG = 64 * BITS / 32;  // words per group: 8 / 16
   constexpr int SPG = WPG / 8;         // load steps per group: 1 / 2
   constexpr int SSG = SPS / SPG;       // groups per super-step
   static_assert(SSG >= 2 && SSG <= 8, "scale vector of 2..8 bf16");
   extern __shared__ uint4 smem[];
   const int MT = p.M;
+  constexpr int MROWS = MR * 2;  // activation rows this instantiation covers
   // this workgroup's share of K: groups [gbase, gbase+Gc), words [wbase, wbase+wcount)
   const int gbase = (int)blockIdx.y * p.gc;
   const int Gc = min(p.gc, p.G - gbase);
   const int wbase = gbase * WPG, wcount = Gc * WPG;
-  uint4* xs = smem;                                                         // [gc*WPG/8][4][2][MT]
-  float2* sxs = reinterpret_cast<float2*>(smem + (size_t)p.gc * WPG * MT);  // [gc][MT]
-  float* red_all = reinterpret_cast<float*>(sxs + (size_t)p.gc * MT);       // [NG][4][MR][64]
-  __shared__ float s_red[4 * NG * 16];
+  // activations by row, slot (step, t, kq) inside; the row stride is padded by two slots
+  // so that the rows a wave reads together (same slot, rows 0..MT-1) fall into different
+  // banks, while the staging threads of one row write consecutive slots
+  const int XS = p.gc * WPG + 2;
+  uint4* xs = smem;                                                   // [MT][XS]
+  float2* sxs = reinterpret_cast<float2*>(smem + (size_t)XS * MT);    // [gc][MT]
+  float* red_all = reinterpret_cast<float*>(sxs + (size_t)p.gc * MT);       // [NG][KW][MR][64]
+  __shared__ float s_red[KW * NG * 16];
   __shared__ float s_inv[16];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int quartet = wave_all >> 2, wave = wave_all & 3;
-  float* red = red_all + quartet * (kWaves * MR * 64);
+  const int quartet = wave_all / KW, wave = wave_all % KW;
+  float* red = red_all + quartet * (KW * MR * 64);
   const int r = lane & 31, kq = lane >> 5;
   const int NB = (p.N + 31) >> 5;
 
@@ -179,52 +182,84 @@ __global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) 
 
   // ---- stage the activations: optional RMSNorm, permute, group sums
   {
+    // one pass over x when every thread sees at most one word of the row and the
+    // workgroup stages the whole row: the words read for the norm stay in registers
+    const bool keep = p.norm_w && p.ksplit == 1 && p.wpr <= kThreads;
+    uint4 xkeep[MROWS];
+    uint4 nwkeep = make_uint4(0, 0, 0, 0);
+    if (keep && tid < p.wpr) nwkeep = load_word_x<BITS>(p.norm_w, tid);
     if (p.norm_w) {
-      float ss[16];
+      // rows are loaded in batches of 4 (clamped to the last real row) so that the loads
+      // of a batch are in flight together instead of one latency per row
+      float ss[MROWS];
 #pragma unroll
-      for (int m = 0; m < 16; ++m) ss[m] = 0.f;
+      for (int m = 0; m < MROWS; ++m) ss[m] = 0.f;
       for (int wi = tid; wi < p.wpr; wi += kThreads)
 #pragma unroll
-        for (int m = 0; m < 16; ++m)
-          if (m < MT) ss[m] += sumsq_word<BITS>(load_word_x<BITS>(p.x + (size_t)m * p.K, wi));
+        for (int m0 = 0; m0 < MROWS; m0 += 4) {
+          if (m0 < MT) {
+            uint4 xv[4];
 #pragma unroll
-      for (int m = 0; m < 16; ++m) {
-        if (m < MT) {
-          const float t = wave_sum(ss[m]);
-          if (lane == 0) s_red[wave_all * 16 + m] = t;
+            for (int j = 0; j < 4; ++j)
+              xv[j] = load_word_x<BITS>(p.x + (size_t)min(m0 + j, MT - 1) * p.K, wi);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              ss[m0 + j] = sumsq_word<BITS>(xv[j], ss[m0 + j]);
+              if (keep) xkeep[m0 + j] = xv[j];
+            }
+          }
         }
+#pragma unroll
+      for (int m = 0; m < MROWS; ++m) {
+        const float t = wave_sum_to_lane63(ss[m]);
+        if (lane == 63) s_red[wave_all * 16 + m] = t;
       }
       __syncthreads();
+      if (tid < MROWS) {
+        float t = 0.f;
 #pragma unroll
-      for (int m = 0; m < 16; ++m)
-        if (m < MT) {
-          float t = 0.f;
-#pragma unroll
-          for (int w = 0; w < 4 * NG; ++w) t += s_red[w * 16 + m];
-          if (tid == 0) s_inv[m] = rsqrtf(t / (float)p.K + p.eps);
-        }
+        for (int w = 0; w < KW * NG; ++w) t += s_red[w * 16 + tid];
+        s_inv[tid] = rsqrtf(t / (float)p.K + p.eps);
+      }
       __syncthreads();
     }
     for (int wl = tid; wl < wcount; wl += kThreads) {
       const int wi = wbase + wl;
       const int step = wl >> 3, q2 = (wl >> 2) & 1, t = wl & 3;
-      const int dst = ((step * 4 + t) * 2 + q2) * MT;
+      const int dst = (step * 4 + t) * 2 + q2;
       uint4 nw = make_uint4(0, 0, 0, 0);
-      if (p.norm_w) nw = load_word_x<BITS>(p.norm_w, wi);
+      if (keep)
+        nw = nwkeep;
+      else if (p.norm_w)
+        nw = load_word_x<BITS>(p.norm_w, wi);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) {
-        if (m < MT) {
-          uint4 xv = load_word_x<BITS>(p.x + (size_t)m * p.K, wi);
-          if (p.norm_w) norm_word<BITS>(xv, nw, s_inv[m]);
-          float stored, truesum;
-          xs[dst + m] = permute_word<BITS>(xv, stored, truesum);
-          // sum over the WPG consecutive words (threads) of the group
+      for (int m0 = 0; m0 < MROWS; m0 += 4) {
+        if (m0 < MT) {
+          uint4 xr[4];
+          if (keep) {
 #pragma unroll
-          for (int o = 1; o < WPG; o <<= 1) {
-            stored += __shfl_xor(stored, o, 64);
-            truesum += __shfl_xor(truesum, o, 64);
+            for (int j = 0; j < 4; ++j) xr[j] = xkeep[m0 + j];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              xr[j] = load_word_x<BITS>(p.x + (size_t)min(m0 + j, MT - 1) * p.K, wi);
           }
-          if ((wl & (WPG - 1)) == 0) sxs[(wl / WPG) * MT + m] = make_float2(128.f * stored, truesum);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int m = m0 + j;
+            uint4 xv = xr[j];
+            if (p.norm_w) norm_word<BITS>(xv, nw, s_inv[m]);
+            float sum;
+            const uint4 pw = permute_word<BITS>(xv, sum);
+            // the WPG consecutive words (lanes) of a group: wcount is a multiple of WPG,
+            // so a run of WPG lanes is active or idle as a whole
+            sum = run_sum<WPG>(sum);
+            if (m < MT) {
+              xs[m * XS + dst] = pw;
+              if ((wl & (WPG - 1)) == 0)
+                sxs[(wl / WPG) * MT + m] = make_float2((BITS == 4 ? 128.f : 128.f * 17.f) * sum, sum);
+            }
+          }
         }
       }
     }
@@ -236,7 +271,7 @@ __global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) 
   int a_of[MR];
 #pragma unroll
   for (int q = 0; q < MR; ++q) a_of[q] = min(8 * (q >> 2) + 4 * Rg + (q & 3), MT - 1);
-  const int a_lane = min(r, MT - 1);  // A-operand row of this lane
+  const uint4* xa = xs + min(r, MT - 1) * XS + kq;  // A-operand row of this lane
 
   uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
   asm volatile("" : "+s"(kmask));
@@ -272,7 +307,7 @@ __global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) 
             bq.y = ((wd[t] >> 4) & kmask) | kmagic;
             bq.z = ((wd[t] >> 8) & kmask) | kmagic;
             bq.w = ((wd[t] >> 12) & kmask) | kmagic;
-            const uint4 av = xs[((step * 4 + t) * 2 + kq) * MT + a_lane];
+            const uint4 av = xa[(step * 4 + t) * 2];
             d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
                                                         __builtin_bit_cast(bf16x8_t, bq), d, 0, 0, 0);
           }
@@ -302,9 +337,13 @@ __global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) 
       const int row = blk * 32 + r;
       float v[MR];
 #pragma unroll
-      for (int q = 0; q < MR; ++q)
-        v[q] = red[q * 64 + lane] + red[(MR + q) * 64 + lane] + red[(2 * MR + q) * 64 + lane] +
-               red[(3 * MR + q) * 64 + lane];
+      for (int q = 0; q < MR; ++q) v[q] = 0.f;
+#pragma unroll 1
+      for (int w0 = 0; w0 < KW; w0 += 4)
+#pragma unroll
+        for (int q = 0; q < MR; ++q)
+          v[q] += (red[(w0 * MR + q) * 64 + lane] + red[((w0 + 1) * MR + q) * 64 + lane]) +
+                  (red[((w0 + 2) * MR + q) * 64 + lane] + red[((w0 + 3) * MR + q) * 64 + lane]);
       bool write = true;
       if (p.ksplit > 1) {
         // partial sums go out at device scope (the merging workgroup may sit on another
@@ -366,9 +405,9 @@ __global__ __launch_bounds__(256 * NG) void qmv_mfma_kernel(const MfmaParams p) 
   }
 }
 
-template <int BITS, int MR, int NG, int SPS>
+template <int BITS, int MR, int KW, int NG, int SPS>
 int launch(const MfmaParams& p, size_t lds, hipStream_t st) {
-  auto kern = qmv_mfma_kernel<BITS, MR, NG, SPS>;
+  auto kern = qmv_mfma_kernel<BITS, MR, KW, NG, SPS>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -381,21 +420,21 @@ int launch(const MfmaParams& p, size_t lds, hipStream_t st) {
   }
   const int NBq = ((p.N + 31) / 32 + NG - 1) / NG;
   int per_cu = lds <= 38 * 1024 ? 4 : (lds <= 51 * 1024 ? 3 : (lds <= 78 * 1024 ? 2 : 1));
-  if (per_cu * NG > 4) per_cu = 4 / NG;  // at most 16 waves per CU
+  if (per_cu * KW * NG > 16) per_cu = 16 / (KW * NG);  // at most 16 waves per CU
   if (per_cu < 1) per_cu = 1;
   int gx = 256 * per_cu / p.ksplit;
   if (gx < 1) gx = 1;
   if (gx > NBq) gx = NBq;
-  kern<<<dim3(gx, p.ksplit), dim3(256 * NG), lds, st>>>(p);
+  kern<<<dim3(gx, p.ksplit), dim3(64 * KW * NG), lds, st>>>(p);
   return EXO_OK;
 }
 
 constexpr int kMaxSplit = 8;
 constexpr size_t kLdsBudget = 150 * 1024;
 
-size_t lds_bytes(int M, int gc, int bits, int MR, int NG) {
+size_t lds_bytes(int M, int gc, int bits, int MR, int KW, int NG) {
   const size_t wpg = 64 * bits / 32;
-  return (size_t)gc * wpg * 16 * M + (size_t)gc * 8 * M + (size_t)NG * kWaves * MR * 64 * 4;
+  return (size_t)(gc * wpg + 2) * 16 * M + (size_t)gc * 8 * M + (size_t)NG * KW * MR * 64 * 4;
 }
 
 }  // namespace
@@ -404,8 +443,8 @@ size_t lds_bytes(int M, int gc, int bits, int MR, int NG) {
 // kernel does not take this K at all
 int exo_qmv_mfma_max_rows(int K, int bits) {
   if (K % (bits == 4 ? 512 : 256) != 0) return 0;
-  const size_t per_row = (size_t)K * bits / 32 * 16 + (size_t)(K / 64) * 8;
-  const size_t budget = kLdsBudget - 4 * kWaves * 8 * 64 * 4;
+  const size_t per_row = ((size_t)K * bits / 32 + 2) * 16 + (size_t)(K / 64) * 8;
+  const size_t budget = kLdsBudget - 4 * 4 * 8 * 64 * 4;
   size_t m = budget / per_row;
   return m > 16 ? 16 : (int)m;
 }
@@ -440,49 +479,63 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   p.G = K / 64;
   const int MR = M <= 8 ? 4 : 8;
   const int NB = (N + 31) / 32;
-  // many row blocks: quartets share the staged x (2 for up to 8 rows, 4 for up to 16);
-  // few: one quartet per workgroup so that the grid stays wide
-  const int NG = NB >= 1024 ? (MR == 8 ? 3 : (M > 4 ? 2 : 1)) : 1;
   const int sps = 4;
   const int ssg = sps / (bits == 4 ? 1 : 2);
-  const int unit = kWaves * ssg;  // groups per chunk come in whole super-steps per wave
+  const int n_steps = p.G / ssg;  // super-steps along K
+  // waves per row block: as many as keep the whole grid at about 4096 waves with at
+  // least two super-steps each (16 needs the 128-register kernels: M <= 8 only)
+  int KW = 4;
+  if (MR == 4) {
+    while (KW < 16 && NB * KW * 2 <= 4096 && n_steps >= KW * 2) KW *= 2;
+  } else if (NB <= 128 && n_steps <= 16) {
+    KW = 8;  // more registers per wave: 8 waves, and only where both N and K are short
+  }
+  // many row blocks: teams of 4 waves share the staged x (2 teams for up to 8 rows, 3 for
+  // up to 16)
+  const int NG = (KW == 4 && NB >= 1024) ? (MR == 8 ? 3 : (M > 4 ? 2 : 1)) : 1;
   const int NBq = (NB + NG - 1) / NG;
+  // LDS the activations of a chunk may take: two workgroups per CU while a workgroup is
+  // 4 or 8 waves, one beyond
+  const size_t lds_cap = (KW * NG <= 8 ? 78u : 150u) * 1024;
   int ksplit = 1;
   if (workspace && (size_t)NB * 4 > kCounterBytes) workspace = nullptr;  // N beyond 524288
   if (workspace) {
-    // split K until a chunk of x fits the LDS with two workgroups per CU, and further
-    // while the grid is narrower than the chip; a chunk is at least one super-step per wave
-    while (ksplit < kMaxSplit && (p.G + ksplit - 1) / ksplit > unit &&
-           (lds_bytes(M, (p.G + ksplit - 1) / ksplit, bits, MR, NG) > (NG == 1 ? 78u : 150u) * 1024 ||
+    // split K until a chunk of x fits the LDS, and further while the grid is narrower
+    // than the chip; a chunk is at least one super-step per wave
+    while (ksplit < kMaxSplit && (p.G + ksplit - 1) / ksplit > KW * ssg &&
+           (lds_bytes(M, (p.G + ksplit - 1) / ksplit, bits, MR, KW, NG) > lds_cap ||
             NBq * ksplit < 256))
       ++ksplit;
   }
   int gc = (p.G + ksplit - 1) / ksplit;
-  gc = (gc + unit - 1) / unit * unit;
+  gc = (gc + ssg - 1) / ssg * ssg;  // chunks in whole super-steps
   if (gc > p.G) gc = p.G;
   ksplit = (p.G + gc - 1) / gc;
   p.ksplit = ksplit;
   p.gc = gc;
-  int gw = (gc + kWaves - 1) / kWaves;
+  int gw = (gc + KW - 1) / KW;
   p.gw = (gw + ssg - 1) / ssg * ssg;
   p.counters = reinterpret_cast<int*>(workspace);
   p.part = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes)
                      : nullptr;
-  const size_t lds = lds_bytes(M, gc, bits, MR, NG);
+  const size_t lds = lds_bytes(M, gc, bits, MR, KW, NG);
   if (lds > kLdsBudget) {
     exo_set_error("exo_qmv: %d rows of K=%d need %zu bytes of LDS", M, K, lds);
     return EXO_ERR_ARG;
   }
-#define EXO_MFMA_CASE(B_, MR_, NG_, SPS_) \
-  if (bits == B_ && MR == MR_ && NG == NG_) return launch<B_, MR_, NG_, SPS_>(p, lds, st);
-  EXO_MFMA_CASE(4, 4, 1, 4)
-  EXO_MFMA_CASE(4, 4, 2, 4)
-  EXO_MFMA_CASE(4, 8, 1, 4)
-  EXO_MFMA_CASE(4, 8, 3, 4)
-  EXO_MFMA_CASE(8, 4, 1, 4)
-  EXO_MFMA_CASE(8, 4, 2, 4)
-  EXO_MFMA_CASE(8, 8, 1, 4)
-  EXO_MFMA_CASE(8, 8, 3, 4)
+#define EXO_MFMA_CASE(B_, MR_, KW_, NG_) \
+  if (bits == B_ && MR == MR_ && KW == KW_ && NG == NG_) return launch<B_, MR_, KW_, NG_, 4>(p, lds, st);
+#define EXO_MFMA_BITS(B_)    \
+  EXO_MFMA_CASE(B_, 4, 4, 1)  \
+  EXO_MFMA_CASE(B_, 4, 4, 2)  \
+  EXO_MFMA_CASE(B_, 4, 8, 1)  \
+  EXO_MFMA_CASE(B_, 4, 16, 1) \
+  EXO_MFMA_CASE(B_, 8, 4, 1)  \
+  EXO_MFMA_CASE(B_, 8, 4, 3)  \
+  EXO_MFMA_CASE(B_, 8, 8, 1)
+  EXO_MFMA_BITS(4)
+  EXO_MFMA_BITS(8)
+#undef EXO_MFMA_BITS
 #undef EXO_MFMA_CASE
   exo_set_error("exo_qmv: no kernel for bits=%d rows=%d", bits, M);
   return EXO_ERR_ARG;
