@@ -41,8 +41,22 @@ struct QmmParams {
   size_t w_stride, s_stride;  // elements between consecutive experts
 };
 
-__device__ __forceinline__ float ubyte_f(uint32_t v, int i) {
-  return (float)((v >> (8 * i)) & 0xffu);  // v_cvt_f32_ubyteN
+// byte I of v as float.  Written as the instruction: the compiler otherwise extracts
+// bytes 1 and 2 with a v_bfe_u32 first.
+template <int I>
+__device__ __forceinline__ float ubyte_f(uint32_t v) {
+  float f;
+  if (I == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+  if (I == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+  if (I == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+  if (I == 3) asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+  return f;
+}
+
+// buffer descriptor over memory that starts at `base`: raw (stride 0) 32-bit data, no
+// range check (every offset the kernel forms is in range by construction)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
 }
 
 // packed codes of one (weight row, half of a K step): 32 codes
@@ -59,23 +73,27 @@ __device__ __forceinline__ bf16x8_t dequant8(const WRaw<BITS>& r, int t, float s
   if (BITS == 4) {
     const uint32_t v = reinterpret_cast<const uint32_t*>(&r.q[0])[t];
     const uint32_t ev = v & 0x0f0f0f0fu, od = (v >> 4) & 0x0f0f0f0fu;
-    o.x = pack_bf2(fmaf(s, ubyte_f(ev, 0), b), fmaf(s, ubyte_f(od, 0), b));
-    o.y = pack_bf2(fmaf(s, ubyte_f(ev, 1), b), fmaf(s, ubyte_f(od, 1), b));
-    o.z = pack_bf2(fmaf(s, ubyte_f(ev, 2), b), fmaf(s, ubyte_f(od, 2), b));
-    o.w = pack_bf2(fmaf(s, ubyte_f(ev, 3), b), fmaf(s, ubyte_f(od, 3), b));
+    o.x = pack_bf2(fmaf(s, ubyte_f<0>(ev), b), fmaf(s, ubyte_f<0>(od), b));
+    o.y = pack_bf2(fmaf(s, ubyte_f<1>(ev), b), fmaf(s, ubyte_f<1>(od), b));
+    o.z = pack_bf2(fmaf(s, ubyte_f<2>(ev), b), fmaf(s, ubyte_f<2>(od), b));
+    o.w = pack_bf2(fmaf(s, ubyte_f<3>(ev), b), fmaf(s, ubyte_f<3>(od), b));
   } else {
     const uint32_t v0 = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t];
     const uint32_t v1 = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t + 1];
-    o.x = pack_bf2(fmaf(s, ubyte_f(v0, 0), b), fmaf(s, ubyte_f(v0, 1), b));
-    o.y = pack_bf2(fmaf(s, ubyte_f(v0, 2), b), fmaf(s, ubyte_f(v0, 3), b));
-    o.z = pack_bf2(fmaf(s, ubyte_f(v1, 0), b), fmaf(s, ubyte_f(v1, 1), b));
-    o.w = pack_bf2(fmaf(s, ubyte_f(v1, 2), b), fmaf(s, ubyte_f(v1, 3), b));
+    o.x = pack_bf2(fmaf(s, ubyte_f<0>(v0), b), fmaf(s, ubyte_f<1>(v0), b));
+    o.y = pack_bf2(fmaf(s, ubyte_f<2>(v0), b), fmaf(s, ubyte_f<3>(v0), b));
+    o.z = pack_bf2(fmaf(s, ubyte_f<0>(v1), b), fmaf(s, ubyte_f<1>(v1), b));
+    o.w = pack_bf2(fmaf(s, ubyte_f<2>(v1), b), fmaf(s, ubyte_f<3>(v1), b));
   }
   return __builtin_bit_cast(bf16x8_t, o);
 }
 
 // MI = 32-row MFMA tiles per wave along M: the workgroup tile is (64*MI) x 128.
-template <int BITS, int MI, bool GROUPED = false>
+// SB4: rows of scales / biases are 8-byte aligned (K a multiple of 256), so the (scale,
+// bias) of four consecutive K steps come in one 8-byte load each instead of four 2-byte
+// ones - a 2-byte load that touches 32 rows costs the memory pipeline as much as a
+// 16-byte one.
+template <int BITS, int MI, bool GROUPED = false, bool SB4 = false>
 __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   constexpr int kThreads = 256;
   constexpr int BM = 64 * MI, BN = 128;
@@ -102,20 +120,36 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     __syncthreads();
   }
 
-  // weight rows of this lane: column tile j -> row n0 + wn + 32*j + lane%32, half lane/32
+  // weight rows of this lane: column tile j -> row n0 + wn + 32*j + lane%32, half lane/32.
+  // Addresses are a workgroup-uniform base plus a 32-bit lane offset (the tile spans at
+  // most 128 rows), so the loop carries no 64-bit address arithmetic.
   const int frow = lane & 31, kq = lane >> 5;
-  const uint32_t* wsrc[2];
-  const bf16_t* ssrc[2];
-  const bf16_t* bsrc[2];
+  const uint32_t* wbase = p.w + w_off + (size_t)n0 * wpr;
+  const bf16_t* sbase = p.s + s_off + (size_t)n0 * G;
+  const bf16_t* bbase = p.b + s_off + (size_t)n0 * G;
+  uint32_t woff[2], soff[2];
   bool w_ok[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int n = n0 + wn + j * 32 + frow;
     w_ok[j] = n < p.N;
-    const size_t row = (size_t)(w_ok[j] ? n : 0);
-    wsrc[j] = p.w + w_off + row * wpr + kq * BITS;  // 32 codes = BITS words per half K step
-    ssrc[j] = p.s + s_off + row * G;
-    bsrc[j] = p.b + s_off + row * G;
+    const uint32_t rel = (uint32_t)(min(n, p.N - 1) - n0);  // rows past N re-read the last one
+    woff[j] = (rel * (uint32_t)wpr + kq * BITS) * 4;  // bytes; 32 codes = BITS words per half K step
+    soff[j] = rel * (uint32_t)G * 2;
+  }
+  // Loads go through buffer instructions: a workgroup-uniform descriptor, a 32-bit lane
+  // offset that never changes, and the K step as the scalar offset.
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x), rw = make_rsrc(wbase), rs = make_rsrc(sbase),
+                               rb = make_rsrc(bbase);
+  // activation rows of this thread: rows past the end re-read the last valid row (their
+  // products are never written)
+  uint32_t xoff[XR];
+#pragma unroll
+  for (int r = 0; r < XR; ++r) {
+    const int id = tid + kThreads * r;
+    const int row = min(id >> 3, m_end - 1 - m0), kp = id & 7;
+    const uint32_t src = GROUPED ? (uint32_t)(row_pair[row] / p.x_div) : (uint32_t)(m0 + row);
+    xoff[r] = (src * (uint32_t)p.K + kp * 8) * 2;  // bytes
   }
 
   struct XStage {
@@ -127,27 +161,36 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 
   auto load_x = [&](XStage& st, int k0) {
 #pragma unroll
-    for (int r = 0; r < XR; ++r) {
-      const int id = tid + kThreads * r;
-      const int row = id >> 3, kp = id & 7;
-      if (m0 + row < m_end) {
-        const size_t src = GROUPED ? (size_t)(row_pair[row] / p.x_div) : (size_t)(m0 + row);
-        st.xa[r] = *reinterpret_cast<const uint4*>(p.x + src * p.K + k0 + kp * 8);
-      } else {
-        st.xa[r] = make_uint4(0, 0, 0, 0);
-      }
-    }
+    for (int r = 0; r < XR; ++r)
+      st.xa[r] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[r], k0 * 2, 0));
   };
   auto load_w = [&](WStage& st, int k0) {
-    const int kw = k0 * BITS / 32;  // word offset of this K step
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int i = 0; i < BITS / 4; ++i)
-        st.w[j].q[i] = *reinterpret_cast<const uint4*>(wsrc[j] + kw + i * 4);
-      st.w[j].s = ssrc[j][k0 >> 6];
-      st.w[j].b = bsrc[j][k0 >> 6];
+        st.w[j].q[i] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(rw, woff[j] + i * 16, k0 * BITS / 8, 0));
+      if (!SB4) {
+        st.w[j].s = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, soff[j], (k0 >> 6) * 2, 0);
+        st.w[j].b = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rb, soff[j], (k0 >> 6) * 2, 0);
+      }
     }
+  };
+  // SB4: (scale, bias) of K steps [4*blk, 4*blk+4) for both column tiles
+  struct SBlock {
+    uint2 s[2], b[2];
+  };
+  auto load_sb = [&](SBlock& sb, int blk) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      sb.s[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs, soff[j], blk * 8, 0));
+      sb.b[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rb, soff[j], blk * 8, 0));
+    }
+  };
+  auto pick = [&](const uint2& v, int e) {  // element e (uniform) of four bf16
+    const uint32_t w = (e & 2) ? v.y : v.x;
+    return (e & 1) ? bf_hi(w) : bf_lo(w);
   };
 
   auto store_x = [&](const XStage& st, int buf) {
@@ -168,27 +211,37 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // multiply tile `buf` by the weights held (packed) in `st`
-  auto multiply = [&](const WStage& st, int buf) {
+  auto multiply = [&](const WStage& st, int buf, const SBlock& sb, int e) {
     float sc[2], bi[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      sc[j] = w_ok[j] ? bf2f(st.w[j].s) : 0.f;
-      bi[j] = w_ok[j] ? bf2f(st.w[j].b) : 0.f;
+      sc[j] = SB4 ? pick(sb.s[j], e) : bf2f(st.w[j].s);
+      bi[j] = SB4 ? pick(sb.b[j], e) : bf2f(st.w[j].b);
+      if (!w_ok[j]) sc[j] = bi[j] = 0.f;
     }
+    // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step.  The A operands of step t+1
+    // are requested before the products of step t, so their LDS latency hides behind them.
+    const bf16_t* arow = &xs[buf][(wm + frow) * LDS_STRIDE + kq * 32];
+    bf16x8_t a[2][MI];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {  // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step
-      bf16x8_t a[MI], bq[2];
+    for (int i = 0; i < MI; ++i)
+      a[0][i] = *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * LDS_STRIDE);
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
-        a[i] = *reinterpret_cast<const bf16x8_t*>(
-            &xs[buf][(wm + i * 32 + frow) * LDS_STRIDE + kq * 32 + t * 8]);
+    for (int t = 0; t < 4; ++t) {
+      bf16x8_t bq[2];
+      if (t < 3) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+          a[(t + 1) & 1][i] =
+              *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * LDS_STRIDE + (t + 1) * 8);
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) bq[j] = dequant8<BITS>(st.w[j], t, sc[j], bi[j]);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], bq[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1][i], bq[j], acc[i][j], 0, 0, 0);
     }
   };
 
@@ -198,6 +251,11 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // is multiplied, the freed weight stage is refilled two steps ahead; one barrier.
   XStage xr;
   WStage w0, w1;
+  SBlock sb0, sb1;  // current block of four K steps, next block
+  if (SB4) {
+    load_sb(sb0, 0);
+    sb1 = sb0;
+  }
   load_x(xr, 0);
   load_w(w0, 0);
   store_x(xr, 0);
@@ -208,9 +266,14 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   __syncthreads();
   int buf = 0;
   for (int k0 = 0; k0 < p.K; k0 += BK) {
+    const int ks = k0 >> 6;
+    if (SB4 && (ks & 3) == 0) {  // a new block: its values arrived during the previous one
+      sb0 = sb1;
+      if (k0 + 4 * BK < p.K) load_sb(sb1, (ks >> 2) + 1);
+    }
     if (k0 + BK < p.K) store_x(xr, buf ^ 1);
     if (k0 + 2 * BK < p.K) load_x(xr, k0 + 2 * BK);
-    multiply(w0, buf);
+    multiply(w0, buf, sb0, ks & 3);
     w0 = w1;  // a few register moves keep the loop body single (no unrolled twin)
     if (k0 + 2 * BK < p.K) load_w(w1, k0 + 2 * BK);
     __syncthreads();
@@ -272,10 +335,27 @@ template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
   // taller inputs: 256-row tiles halve the dequantisation work and the LDS reads per output
-  if (M <= 128)
-    qmm_kernel<BITS, 2><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), 256, 0, st>>>(p);
+  const dim3 g2(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), g4(exo_ceil_div(N, 128), exo_ceil_div(M, 256));
+  const bool sb4 = p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0;
+  if (M <= 128) {
+    if (sb4)
+      qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 2, false, false><<<g2, 256, 0, st>>>(p);
+  } else {
+    if (sb4)
+      qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 4, false, false><<<g4, 256, 0, st>>>(p);
+  }
+}
+
+template <int BITS>
+void launch_grouped(const QmmParams& p, dim3 grid, hipStream_t st) {
+  if (p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0)
+    qmm_kernel<BITS, 2, true, true><<<grid, 256, 0, st>>>(p);
   else
-    qmm_kernel<BITS, 4><<<dim3(exo_ceil_div(N, 128), exo_ceil_div(M, 256)), 256, 0, st>>>(p);
+    qmm_kernel<BITS, 2, true, false><<<grid, 256, 0, st>>>(p);
 }
 
 constexpr int kGroupBM = 128;  // rows per tile of the grouped GEMM
@@ -369,6 +449,9 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   const int P = T * topk;
   const int max_tiles = group_max_tiles(P, E);
   EXO_REQUIRE(max_tiles <= 65535, "exo_gather_qmm: %d row tiles exceed the grid limit", max_tiles);
+  EXO_REQUIRE((int64_t)T * topk * K < (1ll << 31),
+              "exo_gather_qmm: T*topk*K=%lld exceeds 32-bit byte offsets",
+              (long long)T * topk * K);
   QmmParams p{x, w, scales, biases, nullptr, y, P, N, K};
   p.sorted = reinterpret_cast<const int32_t*>(workspace);
   p.tiles = p.sorted + P;
@@ -377,9 +460,9 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   p.s_stride = (size_t)N * (K / 64);
   const dim3 grid(exo_ceil_div(N, 128), max_tiles);
   if (bits == 4)
-    qmm_kernel<4, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    launch_grouped<4>(p, grid, (hipStream_t)stream);
   else
-    qmm_kernel<8, 2, true><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    launch_grouped<8>(p, grid, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_gather_qmm");
   return EXO_OK;
 }
@@ -399,6 +482,8 @@ extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* sca
   p.x_div = 1;
   p.w_stride = p.s_stride = 0;
   EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm: M=%d too large", M);
+  EXO_REQUIRE((int64_t)M * K < (1ll << 31), "exo_qmm: M*K=%lld exceeds 32-bit byte offsets",
+              (long long)M * K);
   if (bits == 4)
     launch_qmm<4>(p, (hipStream_t)stream);
   else

@@ -903,7 +903,8 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
     int m0 = 0;
     while (M - m0 >= 2) {
       const int mt = (M - m0 < cap) ? (M - m0) : cap;
-      rc = exo_qmv_mfma_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases,
+      rc = exo_qmv_mfma_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases, nullptr,
+                               nullptr, nullptr,
                                residual ? residual + (size_t)m0 * N : nullptr, y + (size_t)m0 * N,
                                mt, N, K, bits, workspace, (hipStream_t)stream);
       if (rc) return rc;
@@ -964,10 +965,41 @@ extern "C" int exo_norm_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weigh
                                    const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
                                    uint16_t* y, int M, int N, int K, int bits, int group_size,
                                    exo_stream_t stream) {
+  return exo_norm_qmv_swiglu_ws(x, norm_weight, eps, wg, sg, bg, wu, su, bu, y, nullptr, 0, M, N,
+                                K, bits, group_size, stream);
+}
+
+extern "C" int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                                      const uint32_t* wg, const uint16_t* sg,
+                                      const uint16_t* bg, const uint32_t* wu,
+                                      const uint16_t* su, const uint16_t* bu, uint16_t* y,
+                                      void* workspace, int64_t workspace_bytes, int M, int N,
+                                      int K, int bits, int group_size, exo_stream_t stream) {
   int rc = check_common("exo_qmv_swiglu", M, N, K, bits, group_size);
   if (rc) return rc;
   EXO_REQUIRE(x && wg && sg && bg && wu && su && bu && y, "exo_qmv_swiglu: null pointer");
+  EXO_REQUIRE(!workspace || (workspace_bytes >= exo_qmv_workspace(2 * N) &&
+                             ((uintptr_t)workspace & 255) == 0),
+              "exo_norm_qmv_swiglu_ws: workspace of %lld bytes, need %lld (256-byte aligned)",
+              (long long)workspace_bytes, (long long)exo_qmv_workspace(2 * N));
   if (M == 0) return EXO_OK;
+  // two or more rows: both projections in one matrix-core launch per tile of up to 16 rows
+  if (workspace && M >= 2 && exo_qmv_mfma_max_rows(K, bits) > 0) {
+    int m0 = 0;
+    while (M - m0 >= 2) {
+      const int mt = (M - m0 < 16) ? (M - m0) : 16;
+      rc = exo_qmv_mfma_launch(x + (size_t)m0 * K, norm_weight, eps, wg, sg, bg, wu, su, bu,
+                               nullptr, y + (size_t)m0 * N, mt, N, K, bits, workspace,
+                               (hipStream_t)stream);
+      if (rc) return rc;
+      m0 += mt;
+    }
+    EXO_CHECK_LAUNCH("exo_qmv_swiglu");
+    if (m0 == M) return EXO_OK;
+    x += (size_t)m0 * K;  // a single left-over row takes the dot2 kernel below
+    y += (size_t)m0 * N;
+    M -= m0;
+  }
   const uint32_t* ws[2] = {wg, wu};
   const bf16_t* ss[2] = {sg, su};
   const bf16_t* bs[2] = {bg, bu};

@@ -11,5 +11,6 @@
 int exo_qmv_mfma_max_rows(int K, int bits);
 size_t exo_qmv_mfma_workspace(int N);
 int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
-                        const bf16_t* s, const bf16_t* b, const bf16_t* residual, bf16_t* y,
-                        int M, int N, int K, int bits, void* workspace, hipStream_t st);
+                        const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
+                        const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
+                        int bits, void* workspace, hipStream_t st);

@@ -30,6 +30,10 @@ struct MfmaParams {
   const uint32_t* w;       // [N, wpr]
   const bf16_t* s;         // [N, K/64]
   const bf16_t* b;
+  // second matrix of the (gate, up) pair with the SwiGLU epilogue, or null
+  const uint32_t* w2;
+  const bf16_t* s2;
+  const bf16_t* b2;
   const bf16_t* residual;  // [M,N] or null
   bf16_t* y;               // [M,N]
   const bf16_t* norm_w;    // [K] or null (fused RMSNorm of x)
@@ -38,7 +42,7 @@ struct MfmaParams {
   int gw;  // groups per wave (multiple of the groups per super-step)
   // split-K: blockIdx.y owns groups [y*gc, (y+1)*gc); partial sums meet in `part`
   int ksplit, gc;
-  float* part;    // [ksplit][M][N] float32
+  float* part;    // [ksplit][1 or 2 matrices][M][N] float32
   int* counters;  // [row blocks], zero between launches
 };
 
@@ -139,18 +143,18 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
     uint4 s, b;  // SSG scales / biases
   };
   // item -> (row block, super-step); loads clamp to the last valid row / group
-  auto issue = [&](Buf& bf, int blk, int ss) {
+  auto issue = [&](Buf& bf, int blk, int mat, int ss) {
     const int row = min(blk * 32 + r, p.N - 1);
     const int g0 = min(g_begin + ss * SSG, Gc - SSG);
-    const uint32_t* wp = p.w + (size_t)row * p.wpr + (size_t)(gbase + g0) * WPG + kq * 4;
+    const uint32_t* wp = (mat ? p.w2 : p.w) + (size_t)row * p.wpr + (size_t)(gbase + g0) * WPG + kq * 4;
 #pragma unroll
     for (int i = 0; i < SPS; ++i) {
       // steps past the chunk end re-read its last step (never consumed)
       const int off = min(i * 8, wcount - g0 * WPG - 8);
       bf.w[i] = *reinterpret_cast<const uint4*>(wp + off);
     }
-    const bf16_t* sp = p.s + (size_t)row * p.G + gbase + g0;
-    const bf16_t* bp = p.b + (size_t)row * p.G + gbase + g0;
+    const bf16_t* sp = (mat ? p.s2 : p.s) + (size_t)row * p.G + gbase + g0;
+    const bf16_t* bp = (mat ? p.b2 : p.b) + (size_t)row * p.G + gbase + g0;
     if (SSG == 8) {
       bf.s = *reinterpret_cast<const uint4*>(sp);
       bf.b = *reinterpret_cast<const uint4*>(bp);
@@ -165,20 +169,22 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
     }
   };
 
-  // flat sequence of (row block, super-step) items; the quartets of a workgroup take
+  // flat sequence of (row block, matrix, super-step) items; the teams of a workgroup take
   // neighbouring row blocks and run the same number of items (barriers are block-wide)
+  const int nmat = p.w2 ? 2 : 1;
   const int NBq = (NB + NG - 1) / NG;
   const int my_blocks = (NBq - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-  const int n_items = my_blocks * n_super;
+  const int n_items = my_blocks * nmat * n_super;
   if (n_items <= 0) return;
   auto blk_of = [&](int it) {
-    return ((int)blockIdx.x + (it / n_super) * (int)gridDim.x) * NG + quartet;
+    return ((int)blockIdx.x + (it / (nmat * n_super)) * (int)gridDim.x) * NG + quartet;
   };
+  auto mat_of = [&](int it) { return (it / n_super) & (nmat - 1); };
 
   Buf b0, b1;
   // weights do not depend on x: in flight while x is staged (where registers allow)
   constexpr bool kEarly = (MR == 4);
-  if (kEarly) issue(b0, blk_of(0), 0);
+  if (kEarly) issue(b0, blk_of(0), 0, 0);
 
   // ---- stage the activations: optional RMSNorm, permute, group sums
   {
@@ -280,7 +286,7 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
   float acc[MR];
 #pragma unroll
   for (int q = 0; q < MR; ++q) acc[q] = 0.f;
-  if (!kEarly) issue(b0, blk_of(0), 0);
+  if (!kEarly) issue(b0, blk_of(0), 0, 0);
 
   auto consume = [&](const Buf& bf, int ss) {
     const int g0 = min(g_begin + ss * SSG, Gc - SSG);
@@ -325,8 +331,12 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
     }
   };
 
-  auto finish_block = [&](int blk) {
-    __syncthreads();  // the quartet's first wave has finished reading the previous partials
+  float vg[MR];  // the gate sums of this row block while the up matrix is under way
+#pragma unroll
+  for (int q = 0; q < MR; ++q) vg[q] = 0.f;
+
+  auto finish_block = [&](int blk, int mat) {
+    __syncthreads();  // the team's first wave has finished reading the previous partials
 #pragma unroll
     for (int q = 0; q < MR; ++q) {
       red[(wave * MR + q) * 64 + lane] = acc[q];
@@ -344,7 +354,8 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
         for (int q = 0; q < MR; ++q)
           v[q] += (red[(w0 * MR + q) * 64 + lane] + red[((w0 + 1) * MR + q) * 64 + lane]) +
                   (red[((w0 + 2) * MR + q) * 64 + lane] + red[((w0 + 3) * MR + q) * 64 + lane]);
-      bool write = true;
+      const bool pair_open = nmat == 2 && mat == 0;  // the up matrix is still to come
+      bool write = !pair_open;
       if (p.ksplit > 1) {
         // partial sums go out at device scope (the merging workgroup may sit on another
         // XCD); the last of the ksplit workgroups of this row block adds them up in a
@@ -353,29 +364,37 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
         for (int q = 0; q < MR; ++q) {
           const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
           if (m < p.M && row < p.N)
-            st_dev(&p.part[((size_t)blockIdx.y * p.M + m) * p.N + row], v[q]);
+            st_dev(&p.part[(((size_t)blockIdx.y * nmat + mat) * p.M + m) * p.N + row], v[q]);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        int last = 0;
-        if (lane == 0) {
-          const int old = __hip_atomic_fetch_add(&p.counters[blk], 1, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT);
-          last = (old == p.ksplit - 1);
-          if (last)
-            __hip_atomic_store(&p.counters[blk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        write = __builtin_amdgcn_readfirstlane(last) != 0;
-        if (write) {
+        if (!pair_open) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          int last = 0;
+          if (lane == 0) {
+            const int old = __hip_atomic_fetch_add(&p.counters[blk], 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            last = (old == p.ksplit - 1);
+            if (last)
+              __hip_atomic_store(&p.counters[blk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          write = __builtin_amdgcn_readfirstlane(last) != 0;
+          if (write) {
 #pragma unroll
-          for (int q = 0; q < MR; ++q) {
-            const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
-            float t = 0.f;
-            if (m < p.M && row < p.N)
-              for (int ks = 0; ks < p.ksplit; ++ks)
-                t += ld_dev(&p.part[((size_t)ks * p.M + m) * p.N + row]);
-            v[q] = t;
+            for (int q = 0; q < MR; ++q) {
+              const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
+              float t = 0.f, tg = 0.f;
+              if (m < p.M && row < p.N)
+                for (int ks = 0; ks < p.ksplit; ++ks) {
+                  t += ld_dev(&p.part[(((size_t)ks * nmat + mat) * p.M + m) * p.N + row]);
+                  if (nmat == 2) tg += ld_dev(&p.part[((size_t)ks * nmat * p.M + m) * p.N + row]);
+                }
+              v[q] = t;
+              vg[q] = tg;
+            }
           }
         }
+      } else if (pair_open) {
+#pragma unroll
+        for (int q = 0; q < MR; ++q) vg[q] = v[q];
       }
       if (write) {
 #pragma unroll
@@ -384,7 +403,12 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
           if (m < p.M && row < p.N) {
             const size_t o = (size_t)m * p.N + row;
             float t = v[q];
-            if (p.residual) t = bf2f(f2bf(t)) + bf2f(p.residual[o]);
+            if (nmat == 2) {  // SwiGLU on the bf16-rounded projections
+              const float g = bf2f(f2bf(vg[q])), up = bf2f(f2bf(t));
+              t = g / (1.f + __expf(-g)) * up;
+            } else if (p.residual) {
+              t = bf2f(f2bf(t)) + bf2f(p.residual[o]);
+            }
             p.y[o] = f2bf(t);
           }
         }
@@ -394,13 +418,13 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
 
   int it = 0;
   for (;;) {
-    if (it + 1 < n_items) issue(b1, blk_of(it + 1), (it + 1) % n_super);
+    if (it + 1 < n_items) issue(b1, blk_of(it + 1), mat_of(it + 1), (it + 1) % n_super);
     consume(b0, it % n_super);
-    if (it % n_super == n_super - 1) finish_block(blk_of(it));
+    if (it % n_super == n_super - 1) finish_block(blk_of(it), mat_of(it));
     if (++it >= n_items) break;
-    if (it + 1 < n_items) issue(b0, blk_of(it + 1), (it + 1) % n_super);
+    if (it + 1 < n_items) issue(b0, blk_of(it + 1), mat_of(it + 1), (it + 1) % n_super);
     consume(b1, it % n_super);
-    if (it % n_super == n_super - 1) finish_block(blk_of(it));
+    if (it % n_super == n_super - 1) finish_block(blk_of(it), mat_of(it));
     if (++it >= n_items) break;
   }
 }
@@ -457,17 +481,24 @@ size_t exo_qmv_mfma_workspace(int N) {
   return kCounterBytes + (size_t)kMaxSplit * 16 * N * 4;
 }
 
-// y[M,N] for 2 <= M <= 16.  Without a workspace M must not exceed
+// y[M,N] for 2 <= M <= 16; with a second matrix (w2, s2, b2: the up projection, w being
+// the gate) y = silu(x W^T) * (x W2^T) and the workspace is sized for 2N rows.  Without a
+// workspace M must not exceed
 // exo_qmv_mfma_max_rows(K, bits); with one, K may be split over up to kMaxSplit workgroups
 // per row block so that any M <= 16 fits and a short N still fills the chip.
 int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
-                        const bf16_t* s, const bf16_t* b, const bf16_t* residual, bf16_t* y,
-                        int M, int N, int K, int bits, void* workspace, hipStream_t st) {
+                        const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
+                        const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
+                        int bits, void* workspace, hipStream_t st) {
   MfmaParams p;
   p.x = x;
   p.w = w;
   p.s = s;
   p.b = b;
+  p.w2 = w2;
+  p.s2 = s2;
+  p.b2 = b2;
+  const int nmat = w2 ? 2 : 1;
   p.residual = residual;
   p.y = y;
   p.norm_w = norm_w;
@@ -486,7 +517,7 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   // least two super-steps each (16 needs the 128-register kernels: M <= 8 only)
   int KW = 4;
   if (MR == 4) {
-    while (KW < 16 && NB * KW * 2 <= 4096 && n_steps >= KW * 2) KW *= 2;
+    while (KW < 16 && NB * nmat * KW * 2 <= 4096 && n_steps >= KW * 2) KW *= 2;
   } else if (NB <= 128 && n_steps <= 16) {
     KW = 8;  // more registers per wave: 8 waves, and only where both N and K are short
   }

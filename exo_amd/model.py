@@ -189,18 +189,9 @@ class ShardModel:
         c = self.cfg
         gemv = R <= GEMV_MAX_ROWS
         if not c.is_moe:
-            if R == 1:  # post-attention norm fused into the gate/up GEMV pair
+            if gemv:  # post-attention norm and SwiGLU fused into the gate/up GEMV pair
                 ops.qmv_swiglu(bf.h, L.gate, L.up, out=bf.act, norm_weight=L.post_norm,
                                eps=c.rms_norm_eps)
-            elif gemv:  # a few rows: matrix-core GEMV per projection (norm fused), then swiglu
-                if bf.gate is None:
-                    bf.gate = torch.empty_like(bf.act)
-                    bf.up = torch.empty_like(bf.act)
-                ops.quantized_matmul(bf.h, L.gate, out=bf.gate, norm_weight=L.post_norm,
-                                     eps=c.rms_norm_eps)
-                ops.quantized_matmul(bf.h, L.up, out=bf.up, norm_weight=L.post_norm,
-                                     eps=c.rms_norm_eps)
-                ops.swiglu(bf.gate, bf.up, out=bf.act)
             else:
                 if bf.gate is None:
                     bf.gate = torch.empty_like(bf.act)

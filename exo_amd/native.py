@@ -30,6 +30,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_qmv_workspace": (_i64, [_i]),
     "exo_norm_qmv_ws": (_i, [_vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "exo_norm_qmv_swiglu": (_i, [_vp, _vp, _f] + [_vp] * 7 + [_i, _i, _i, _i, _i, _vp]),
+    "exo_norm_qmv_swiglu_ws": (_i, [_vp, _vp, _f] + [_vp] * 8 + [_i64, _i, _i, _i, _i, _i, _vp]),
     "exo_moe_group_workspace": (_i64, [_i, _i, _i]),
     "exo_moe_group": (_i, [_vp, _i, _i, _i, _vp, _i64, _vp]),
     "exo_gather_qmm": (_i, [_vp] * 6 + [_i] * 8 + [_vp]),

@@ -225,6 +225,17 @@ def qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None, norm_wei
     assert gate.N == up.N and gate.K == up.K == K and gate.bits == up.bits
     if out is None:
         out = torch.empty(M, gate.N, dtype=torch.bfloat16, device=x.device)
+    if 2 <= M <= QMV_MAX_M:
+        ws = qmv_workspace(2 * gate.N, x.device)
+        check(
+            lib.exo_norm_qmv_swiglu_ws(
+                _ptr(x), _ptr(norm_weight), eps, _ptr(gate.weight), _ptr(gate.scales),
+                _ptr(gate.biases), _ptr(up.weight), _ptr(up.scales), _ptr(up.biases), _ptr(out),
+                _ptr(ws), ws.numel(), M, gate.N, K, gate.bits, gate.group_size, _stream(),
+            ),
+            "qmv_swiglu(rows 2..16)",
+        )
+        return out
     check(
         lib.exo_norm_qmv_swiglu(
             _ptr(x), _ptr(norm_weight), eps, _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),

@@ -90,6 +90,15 @@ int exo_norm_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float ep
                         const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
                         const uint32_t* wu, const uint16_t* su, const uint16_t* bu, uint16_t* y,
                         int M, int N, int K, int bits, int group_size, exo_stream_t stream);
+/* exo_norm_qmv_swiglu with the workspace of exo_norm_qmv_ws, sized for both matrices:
+ * exo_qmv_workspace(2 * N) bytes.  For 2 <= M <= 16 rows both projections and the
+ * SwiGLU (.typings/mlx_lm/models/switch_layers.pyi:52-57) run as one matrix-core launch.
+ * workspace == NULL behaves like exo_norm_qmv_swiglu. */
+int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                           const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                           const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
+                           uint16_t* y, void* workspace, int64_t workspace_bytes, int M, int N,
+                           int K, int bits, int group_size, exo_stream_t stream);
 
 /* K2: the same operator for any M (prefill): weights are dequantised to bf16 in
  * LDS and multiplied on the matrix cores, float32 accumulation, bf16 out. */

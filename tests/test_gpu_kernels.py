@@ -110,7 +110,7 @@ def test_qmv_residual(device, bits):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("M", [1, 4])
+@pytest.mark.parametrize("M", [1, 4, 9, 16])
 def test_qmv_swiglu(device, bits, M):
     N, K = 320, 2048
     g = rand_quantized(N, K, bits, seed=31)
@@ -119,6 +119,27 @@ def test_qmv_swiglu(device, bits, M):
     got = n_f32(ops.qmv_swiglu(t_bf16(x, device), t_qw(g, bits, device), t_qw(u, bits, device)))
     want = O.swiglu(affine.qmm(x, *g, 64, bits), affine.qmm(x, *u, 64, bits))
     assert_close(got, want, what="qmv_swiglu")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(8, 1000, 4096), (3, 96, 14336), (16, 2080, 2048), (5, 14336, 512)])
+def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
+    """The one-launch (gate, up, SwiGLU) of 2..16 rows rounds each projection to bf16
+    before the SwiGLU, so it equals the two GEMVs followed by the elementwise kernel bit
+    for bit; with and without the fused RMSNorm, with K split over workgroups (short N)
+    and not."""
+    g = t_qw(rand_quantized(N, K, bits, seed=N + 1), bits, device)
+    u = t_qw(rand_quantized(N, K, bits, seed=N + 2), bits, device)
+    x = t_bf16(rand_bf16((M, K), seed=M + K, scale=2.0), device)
+    w = t_bf16(affine.bf16_round(rand_bf16((K,), seed=6) * 0.1 + 1.0), device)
+    for nw in (None, w):
+        fused = ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
+        sep = ops.swiglu(ops.quantized_matmul(x, g, norm_weight=nw, eps=1e-5),
+                         ops.quantized_matmul(x, u, norm_weight=nw, eps=1e-5))
+        assert torch.equal(fused.view(torch.int16), sep.view(torch.int16))
+    # the shared workspace is left clean for a launch of another shape
+    y = ops.quantized_matmul(x[:2], g)
+    assert torch.equal(y.view(torch.int16), ops.quantized_matmul(x[:2], g).view(torch.int16))
 
 
 @pytest.mark.parametrize("bits", [4, 8])
