@@ -180,6 +180,31 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
   }
 }
 
+// Which 16-byte chunk of a row a lane takes in unit j of the row-streaming kernel.  Units
+// come in pairs (2d, 2d+1) that interleave their quantisation groups: the lanes of a
+// group own the groups 2g and 2g+1 of the pair, one in each unit, so the (scale, bias) of
+// both units sit next to each other and come in ONE 32-bit load instead of two 16-bit
+// ones.  A wave instruction of a pair still covers whole 64-byte pieces of every 128-byte
+// line of the 2 KiB span.  An odd last unit keeps the linear order.
+template <int BITS, int ITERS>
+__device__ __forceinline__ int chunk_of(int j, int lane) {
+  constexpr int LG = BITS == 4 ? 2 : 4;  // lanes (chunks) per group
+  if ((ITERS & 1) && j == ITERS - 1) return 64 * j + lane;
+  return 128 * (j >> 1) + 2 * LG * (lane / LG) + LG * (j & 1) + (lane % LG);
+}
+template <int BITS, int ITERS>
+__device__ __forceinline__ void unit_lane_of(int c, int& j, int& lane) {
+  constexpr int LG = BITS == 4 ? 2 : 4;
+  if ((ITERS & 1) && c >= 64 * (ITERS - 1)) {
+    j = ITERS - 1;
+    lane = c - 64 * (ITERS - 1);
+    return;
+  }
+  const int r = c & 127;
+  j = 2 * (c >> 7) + ((r / LG) & 1);
+  lane = (r / (2 * LG)) * LG + (r % LG);
+}
+
 // Two-phase staging for the row-streaming kernel (wpr == 256*ITERS, so every thread
 // owns exactly ITERS words per activation row): the global loads are issued first and
 // consumed after the first weight batches are in flight.
@@ -228,7 +253,8 @@ __device__ __forceinline__ void stage_x_store(const QmvParams& p, XStage<BITS, M
   for (int it = 0; it < ITERS; ++it) {
     const int wi = threadIdx.x + it * kThreads;
     const int c = wi >> 2, t = wi & 3;
-    const int j = c >> 6, sl = c & 63;
+    int j, sl;
+    unit_lane_of<BITS, ITERS>(c, j, sl);
     const int dst = (((j << 2) + t) << 6) + sl;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -258,7 +284,7 @@ __device__ __forceinline__ void stage_x_store(const QmvParams& p, XStage<BITS, M
       truesum += __shfl_xor(truesum, 1, 64);
       stored += __shfl_xor(stored, 2, 64);
       truesum += __shfl_xor(truesum, 2, 64);
-      if (t == 0) sx[m * CPR + c] = make_float2(128.f * stored, truesum);
+      if (t == 0) sx[m * CPR + j * 64 + sl] = make_float2(128.f * stored, truesum);
     }
   }
 }
@@ -486,7 +512,12 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   float2* sx = reinterpret_cast<float2*>(smem + (size_t)MT * p.wpr);
   constexpr int GSHIFT = (BITS == 4) ? 1 : 2;
   constexpr int UG = 64 >> GSHIFT;  // scale elements per unit
-  constexpr int R0 = 8 / (ITERS * NMAT);
+  // NBUF register buffers of one batch each.  The (gate, up) pair on short rows takes four
+  // batches of one row instead of two of two: the arithmetic on a batch then starts when a
+  // quarter of the wave's loads has landed (measured: 1.5 us off the 14336x4096 pair; for a
+  // single matrix the extra live registers cost more than the finer batches gain)
+  constexpr int NBUF = (NMAT == 2 && ITERS <= 2) ? 4 : 2;
+  constexpr int R0 = (16 / NBUF) / (ITERS * NMAT);
   constexpr int R = R0 < 1 ? 1 : R0;  // rows per batch
   constexpr int UB = R * ITERS;       // units per batch and matrix
   constexpr int CPR = 64 * ITERS;
@@ -524,12 +555,11 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     sb[a] = reinterpret_cast<const char*>(p.s[a] + eg);
     bb[a] = reinterpret_cast<const char*>(p.b[a] + eg);
   }
-  const uint32_t lw = lane * 16;               // byte offset of the lane inside a unit
-  const uint32_t ls = (lane >> GSHIFT) * 2;    // byte offset of the lane's scale
-
   struct Batch {
     uint4 w[NMAT][UB];
-    bf16_t s[NMAT][UB], b[NMAT][UB];
+    // (scale, bias) words: a unit pair shares the word of its even unit (low half: even
+    // unit, high half: odd unit); an unpaired last unit holds its value in the low half
+    uint32_t s[NMAT][UB], b[NMAT][UB];
   };
 
   auto issue = [&](Batch& bt, int row_first) {
@@ -537,12 +567,23 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     for (int i = 0; i < UB; ++i) {
       // rows past the end of the range re-read its last row (results are dropped)
       const int row = min(row_first + i / ITERS, r1 - 1);
-      const uint32_t u = (uint32_t)row * ITERS + (i % ITERS);
+      const int j = i % ITERS;
+      const bool paired = !((ITERS & 1) && j == ITERS - 1);
+      const size_t wofs = (size_t)row * (ITERS * 1024) + chunk_of<BITS, ITERS>(j, lane) * 16;
 #pragma unroll
       for (int a = 0; a < NMAT; ++a) {
-        bt.w[a][i] = *reinterpret_cast<const uint4*>(wb[a] + (size_t)u * 1024 + lw);
-        bt.s[a][i] = *reinterpret_cast<const bf16_t*>(sb[a] + (size_t)u * (UG * 2) + ls);
-        bt.b[a][i] = *reinterpret_cast<const bf16_t*>(bb[a] + (size_t)u * (UG * 2) + ls);
+        bt.w[a][i] = *reinterpret_cast<const uint4*>(wb[a] + wofs);
+        if (paired) {
+          if ((j & 1) == 0) {
+            const size_t sofs = ((size_t)row * G + UG * j) * 2 + (lane >> GSHIFT) * 4;
+            bt.s[a][i] = *reinterpret_cast<const uint32_t*>(sb[a] + sofs);
+            bt.b[a][i] = *reinterpret_cast<const uint32_t*>(bb[a] + sofs);
+          }
+        } else {
+          const size_t sofs = ((size_t)row * G + UG * j + (lane >> GSHIFT)) * 2;
+          bt.s[a][i] = *reinterpret_cast<const bf16_t*>(sb[a] + sofs);
+          bt.b[a][i] = *reinterpret_cast<const bf16_t*>(bb[a] + sofs);
+        }
       }
     }
   };
@@ -607,8 +648,13 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
           for (int m = 0; m < MT; ++m) {
 #pragma unroll
             for (int a = 0; a < NMAT; ++a) {
-              acc[a][m] = fmaf(bf2f(bt.s[a][i]), d[a][m], acc[a][m]);
-              acc[a][m] = fmaf(bf2f(bt.b[a][i]), sm[m].y, acc[a][m]);
+              // odd unit of a pair: high half of the even unit's word
+              const bool hi = (j & 1) && !((ITERS & 1) && j == ITERS - 1);
+              const int is = hi ? i - 1 : i;
+              const float sc = hi ? bf_hi(bt.s[a][is]) : bf_lo(bt.s[a][is]);
+              const float bi = hi ? bf_hi(bt.b[a][is]) : bf_lo(bt.b[a][is]);
+              acc[a][m] = fmaf(sc, d[a][m], acc[a][m]);
+              acc[a][m] = fmaf(bi, sm[m].y, acc[a][m]);
             }
           }
         }
@@ -636,7 +682,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 
   // Order of the prologue: activations first (they sit in L2 and are waited for with
   // the weight loads still outstanding), then two weight batches, then the LDS staging.
-  Batch ba, bb2;
+  Batch buf[NBUF];
   if (XR) {
     if (nrows <= 0) return;
     uint4 raw[ITERS][4], nwv[ITERS][4];
@@ -644,11 +690,11 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     for (int j = 0; j < ITERS; ++j)
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int wi = 4 * (lane + 64 * j) + t;
+        const int wi = 4 * chunk_of<BITS, ITERS>(j, lane) + t;
         raw[j][t] = load_word_x<BITS>(xin, wi);
         if (p.norm_w) nwv[j][t] = load_word_x<BITS>(p.norm_w, wi);
       }
-    issue(ba, r0);
+    issue(buf[0], r0);
     if (p.norm_w) {
       float ss = 0.f;
 #pragma unroll
@@ -678,30 +724,44 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     // the second batch only now: the raw activations and norm weights are dead, so
     // the register peak stays at what the main loop needs
     asm volatile("" ::: "memory");
-    if (nrows > R) issue(bb2, r0 + R);
+    if (nrows > R) issue(buf[1], r0 + R);
   } else {
     XStage<BITS, MT, ITERS> xst;
     stage_x_load<BITS, MT, ITERS>(p, xin, xst);
-    if (nrows > 0) issue(ba, r0);
+    if (nrows > 0) issue(buf[0], r0);
     __shared__ float s_red[4 * MT];
     stage_x_store<BITS, MT, ITERS>(p, xst, xs, sx, s_red);
     __syncthreads();
     if (nrows <= 0) return;
-    if (nrows > R) issue(bb2, r0 + R);
+#pragma unroll
+    for (int b = 1; b < NBUF; ++b)
+      if (nrows > b * R) issue(buf[b], r0 + b * R);
   }
 
-  // two register buffers in ping-pong: two batches are in flight while one is consumed,
-  // without copying registers
+  // the register buffers in rotation: NBUF - 1 batches are in flight while one is
+  // consumed, without copying registers
   int rb = r0;
-  for (;;) {
-    compute(ba, rb);
-    rb += R;
-    if (rb >= r1) break;
-    if (rb + R < r1) issue(ba, rb + R);
-    compute(bb2, rb);
-    rb += R;
-    if (rb >= r1) break;
-    if (rb + R < r1) issue(bb2, rb + R);
+  if (NBUF == 2) {
+    for (;;) {
+      compute(buf[0], rb);
+      rb += R;
+      if (rb >= r1) break;
+      if (rb + R < r1) issue(buf[0], rb + R);
+      compute(buf[1], rb);
+      rb += R;
+      if (rb >= r1) break;
+      if (rb + R < r1) issue(buf[1], rb + R);
+    }
+  } else {
+    for (;;) {
+#pragma unroll
+      for (int b = 0; b < NBUF; ++b) {
+        compute(buf[b], rb);
+        rb += R;
+        if (rb >= r1) return;
+        if (rb + (NBUF - 1) * R < r1) issue(buf[b], rb + (NBUF - 1) * R);
+      }
+    }
   }
 }
 
