@@ -765,6 +765,133 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Long rows (4 or more KiB-units per row, one activation row, no fused norm): the NW
+// waves of a workgroup split K.  Wave w owns unit w of every row of the workgroup's row
+// range, so its share of x (16 registers) never leaves the wave: no LDS staging of the
+// activations and no barrier before the first product.  The partial sums of a batch of
+// rows meet in LDS (one barrier per batch, two partial-sum buffers in alternation) and
+// are added in wave order, so the result does not depend on timing.
+template <int BITS, int NW>
+__global__ __launch_bounds__(64 * NW) void qmv_ksplit_kernel(const QmvParams p) {
+  constexpr int GSHIFT = (BITS == 4) ? 1 : 2;
+  constexpr int UG = 64 >> GSHIFT;  // scale elements per unit
+  constexpr int R = 4;              // rows per batch
+  __shared__ float red[2][R][NW];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int G = p.K >> 6;
+
+  // balanced contiguous row range of this workgroup
+  const int base = p.N / (int)gridDim.x, rem = p.N - base * (int)gridDim.x;
+  const int r0 = (int)blockIdx.x * base + min((int)blockIdx.x, rem);
+  const int r1 = r0 + base + ((int)blockIdx.x < rem ? 1 : 0);
+  if (r0 >= r1) return;
+
+  const char* wb = reinterpret_cast<const char*>(p.w[0]) + (size_t)wave * 1024 + lane * 16;
+  const char* sb = reinterpret_cast<const char*>(p.s[0]) + ((size_t)wave * UG + (lane >> GSHIFT)) * 2;
+  const char* bb = reinterpret_cast<const char*>(p.b[0]) + ((size_t)wave * UG + (lane >> GSHIFT)) * 2;
+
+  struct Batch {
+    uint4 w[R];
+    bf16_t s[R], b[R];
+  };
+  auto issue = [&](Batch& bt, int row_first) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int row = min(row_first + i, r1 - 1);  // rows past the end: dropped later
+      bt.w[i] = *reinterpret_cast<const uint4*>(wb + (size_t)row * (NW * 1024));
+      bt.s[i] = *reinterpret_cast<const bf16_t*>(sb + (size_t)row * G * 2);
+      bt.b[i] = *reinterpret_cast<const bf16_t*>(bb + (size_t)row * G * 2);
+    }
+  };
+
+  // this lane's 16-byte chunk of x (unit `wave`, chunk `lane`), in dot2 register order
+  uint4 xr[4];
+  float2 sxr;
+  {
+    uint4 raw[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) raw[t] = load_word_x<BITS>(p.x, 4 * (64 * wave + lane) + t);
+    float stored = 0.f, truesum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float st_, ts_;
+      xr[t] = permute_word<BITS>(raw[t], st_, ts_);
+      stored += st_;
+      truesum += ts_;
+    }
+    sxr = make_float2(128.f * stored, truesum);
+  }
+  uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
+  asm volatile("" : "+s"(kmask));
+  asm volatile("" : "+v"(kmagic));
+
+  auto compute = [&](const Batch& bt, int rb, int parity) {
+    float acc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      float d = -sxr.x;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        uint32_t pr[4];
+        unpack_word_r(reinterpret_cast<const uint32_t*>(&bt.w[i])[t], kmask, kmagic, pr);
+        d = dot2_bf16(pr[0], xr[t].x, d);
+        d = dot2_bf16(pr[1], xr[t].y, d);
+        d = dot2_bf16(pr[2], xr[t].z, d);
+        d = dot2_bf16(pr[3], xr[t].w, d);
+      }
+      acc[i] = fmaf(bf2f(bt.s[i]), d, bf2f(bt.b[i]) * sxr.y);
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const float t = wave_sum_to_lane63(acc[i]);
+      if (lane == 63) red[parity][i][wave] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x < R) {
+      const int row = rb + (int)threadIdx.x;
+      if (row < r1) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) t += red[parity][threadIdx.x][w];
+        if (p.residual) t = bf2f(f2bf(t)) + bf2f(p.residual[row]);
+        p.y[row] = f2bf(t);
+      }
+    }
+  };
+
+  Batch ba, bb2;
+  issue(ba, r0);
+  if (r0 + R < r1) issue(bb2, r0 + R);
+  int rb = r0, parity = 0;
+  for (;;) {
+    compute(ba, rb, parity);
+    rb += R;
+    parity ^= 1;
+    if (rb >= r1) break;
+    if (rb + R < r1) issue(ba, rb + R);
+    compute(bb2, rb, parity);
+    rb += R;
+    parity ^= 1;
+    if (rb >= r1) break;
+    if (rb + R < r1) issue(bb2, rb + R);
+  }
+}
+
+template <int BITS, int NW>
+int launch_ksplit(const QmvParams& p, hipStream_t st) {
+  // 16 waves per CU; at least one batch of four rows per workgroup
+  const int per_cu = 16 / NW < 1 ? 1 : 16 / NW;
+  int grid = 256 * per_cu;
+  const int max_grid = (p.N + 3) / 4;
+  if (grid > max_grid) grid = max_grid;
+  qmv_ksplit_kernel<BITS, NW><<<dim3(grid), dim3(64 * NW), 0, st>>>(p);
+  return EXO_OK;
+}
+
 struct Plan {
   int lpr_log2, iters, slots, spw, grid, ragged;
   size_t lds;
@@ -823,6 +950,11 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
 
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
+  if (MT == 1 && NMAT == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.norm_w && !p.idx && p.M == 1) {
+    // measured against the row kernel: ahead at 14 units per row (8-bit, K = 14336: 17.0
+    // vs 18.3 us for 4096 rows), level at 7 and 8, behind at 4
+    if (pl.iters == 14) return launch_ksplit<BITS, 14>(p, st);
+  }
   if (MT <= 2 && pl.lpr_log2 == 6 && !pl.ragged) {
     constexpr int MTR = MT <= 2 ? MT : 1;  // (no instantiation for larger tiles)
     switch (pl.iters) {
