@@ -39,6 +39,10 @@ struct QmmParams {
   const int32_t* tiles;   // [max_tiles][3] = expert (-1: unused), start, rows
   int x_div;
   size_t w_stride, s_stride;  // elements between consecutive experts
+  // split-K (few row tiles): blockIdx.z owns K steps [z*kc, (z+1)*kc) and writes a
+  // float32 partial tile; qmm_reduce_kernel adds them
+  int ksplit, kc;
+  float* part;  // [ksplit][M][N]
 };
 
 // byte I of v as float.  Written as the instruction: the compiler otherwise extracts
@@ -57,6 +61,11 @@ __device__ __forceinline__ float ubyte_f(uint32_t v) {
 // range check (every offset the kernel forms is in range by construction)
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
+}
+
+// elements between the partial tiles of consecutive K ranges (16-byte aligned rows of 4)
+__host__ __device__ inline size_t part_stride(int M, int N) {
+  return ((size_t)M * N + 3) / 4 * 4;
 }
 
 // packed codes of one (weight row, half of a K step): 32 codes
@@ -249,35 +258,56 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // (xr), the packed weights of k and k+1 in w0 / w1.  Per step: the next x tile goes to
   // the other LDS buffer and its registers are refilled two steps ahead, the current tile
   // is multiplied, the freed weight stage is refilled two steps ahead; one barrier.
+  // this workgroup's K range (all of K unless split; a multiple of four K steps)
+  const int kb = GROUPED ? 0 : (int)blockIdx.z * p.kc;
+  const int ke = GROUPED ? p.K : min(p.K, kb + p.kc);
   XStage xr;
   WStage w0, w1;
   SBlock sb0, sb1;  // current block of four K steps, next block
   if (SB4) {
-    load_sb(sb0, 0);
+    load_sb(sb0, kb >> 8);
     sb1 = sb0;
   }
-  load_x(xr, 0);
-  load_w(w0, 0);
+  load_x(xr, kb);
+  load_w(w0, kb);
   store_x(xr, 0);
-  if (BK < p.K) {
-    load_x(xr, BK);
-    load_w(w1, BK);
+  if (kb + BK < ke) {
+    load_x(xr, kb + BK);
+    load_w(w1, kb + BK);
   }
   __syncthreads();
   int buf = 0;
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
+  for (int k0 = kb; k0 < ke; k0 += BK) {
     const int ks = k0 >> 6;
     if (SB4 && (ks & 3) == 0) {  // a new block: its values arrived during the previous one
       sb0 = sb1;
-      if (k0 + 4 * BK < p.K) load_sb(sb1, (ks >> 2) + 1);
+      if (k0 + 4 * BK < ke) load_sb(sb1, (ks >> 2) + 1);
     }
-    if (k0 + BK < p.K) store_x(xr, buf ^ 1);
-    if (k0 + 2 * BK < p.K) load_x(xr, k0 + 2 * BK);
+    if (k0 + BK < ke) store_x(xr, buf ^ 1);
+    if (k0 + 2 * BK < ke) load_x(xr, k0 + 2 * BK);
     multiply(w0, buf, sb0, ks & 3);
     w0 = w1;  // a few register moves keep the loop body single (no unrolled twin)
-    if (k0 + 2 * BK < p.K) load_w(w1, k0 + 2 * BK);
+    if (k0 + 2 * BK < ke) load_w(w1, k0 + 2 * BK);
     __syncthreads();
     buf ^= 1;
+  }
+
+  if (!GROUPED && p.ksplit > 1) {
+    // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
+    // small launch adds the ranges in a fixed order (qmm_reduce_kernel)
+    float* mine = p.part + (size_t)blockIdx.z * part_stride(p.M, p.N);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int n = n0 + wn + j * 32 + frow;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+          if (m < m_end && n < p.N) mine[(size_t)m * p.N + n] = acc[i][j][r];
+        }
+      }
+    return;
   }
 
   // Epilogue through LDS.  D[i][j] holds column lane%32 (W row n) and rows
@@ -331,17 +361,88 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   }
 }
 
+constexpr int kQmmMaxSplit = 8;
+
+// y = bf16(sum over the K ranges, in order) (+ residual): four outputs per thread
+__global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict__ part,
+                                                         const bf16_t* __restrict__ residual,
+                                                         bf16_t* __restrict__ y, int64_t total,
+                                                         int64_t stride, int ksplit, int vec_ok) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  if (vec_ok && i + 4 <= total) {
+    float4 v[kQmmMaxSplit];
+#pragma unroll
+    for (int z = 0; z < kQmmMaxSplit; ++z)
+      if (z < ksplit) v[z] = *reinterpret_cast<const float4*>(part + (size_t)z * stride + i);
+    float4 t = v[0];
+#pragma unroll
+    for (int z = 1; z < kQmmMaxSplit; ++z)
+      if (z < ksplit) {
+        t.x += v[z].x;
+        t.y += v[z].y;
+        t.z += v[z].z;
+        t.w += v[z].w;
+      }
+    float o[4] = {bf2f(f2bf(t.x)), bf2f(f2bf(t.y)), bf2f(f2bf(t.z)), bf2f(f2bf(t.w))};
+    if (residual) {
+      const uint2 rv = *reinterpret_cast<const uint2*>(residual + i);
+      o[0] += bf_lo(rv.x);
+      o[1] += bf_hi(rv.x);
+      o[2] += bf_lo(rv.y);
+      o[3] += bf_hi(rv.y);
+    }
+    uint2 w;
+    w.x = pack_bf2(o[0], o[1]);
+    w.y = pack_bf2(o[2], o[3]);
+    *reinterpret_cast<uint2*>(y + i) = w;
+  } else {
+    for (int64_t e = i; e < min(i + 4, total); ++e) {
+      float t = 0.f;
+      for (int z = 0; z < ksplit; ++z) t += part[(size_t)z * stride + e];
+      t = bf2f(f2bf(t));
+      if (residual) t += bf2f(residual[e]);
+      y[e] = f2bf(t);
+    }
+  }
+}
+
+// K split of a launch: only for up to 128 rows (one row tile) when the column tiles alone
+// cover less than the chip; chunks of whole blocks of four K steps, at least two blocks
+void plan_split(int M, int N, int K, bool have_ws, int* ksplit, int* kc) {
+  *ksplit = 1;
+  *kc = K;
+  if (!have_ws || M > 128 || K % 256 != 0) return;
+  const int tiles = exo_ceil_div(N, 128);
+  int ks = 1;
+  while (ks < kQmmMaxSplit && tiles * ks < 256 && K / (ks * 2) >= 512) ks *= 2;
+  if (ks == 1) return;
+  int c = exo_ceil_div(K, ks);
+  c = (c + 255) / 256 * 256;
+  *kc = c;
+  *ksplit = exo_ceil_div(K, c);
+}
+
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
   // taller inputs: 256-row tiles halve the dequantisation work and the LDS reads per output
-  const dim3 g2(exo_ceil_div(N, 128), exo_ceil_div(M, 128)), g4(exo_ceil_div(N, 128), exo_ceil_div(M, 256));
+  const dim3 g2(exo_ceil_div(N, 128), exo_ceil_div(M, 128), p.ksplit), g4(exo_ceil_div(N, 128), exo_ceil_div(M, 256));
   const bool sb4 = p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0;
-  if (M <= 128) {
+  // a grid of fewer than 128 of the tall tiles leaves most CUs idle: twice as many
+  // 128-row tiles are faster there (1024x4096 at 2046 rows: 89 -> 70 us), not beyond
+  const bool small_grid = (int64_t)g4.x * g4.y < 128;
+  if (M <= 128 || small_grid) {
     if (sb4)
       qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, false, false><<<g2, 256, 0, st>>>(p);
+    if (p.ksplit > 1) {
+      const int64_t total = (int64_t)M * N;
+      const int vec_ok = (((uintptr_t)p.y | (uintptr_t)p.residual) & 7) == 0;
+      qmm_reduce_kernel<<<dim3(exo_ceil_div(exo_ceil_div(total, 4), 256)), 256, 0, st>>>(
+          p.part, p.residual, p.y, total, (int64_t)part_stride(M, N), p.ksplit, vec_ok);
+    }
   } else {
     if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
@@ -458,6 +559,9 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   p.x_div = x_rows == 1 ? topk : 1;
   p.w_stride = (size_t)N * (K * bits / 32);
   p.s_stride = (size_t)N * (K / 64);
+  p.ksplit = 1;
+  p.kc = K;
+  p.part = nullptr;
   const dim3 grid(exo_ceil_div(N, 128), max_tiles);
   if (bits == 4)
     launch_grouped<4>(p, grid, (hipStream_t)stream);
@@ -467,20 +571,40 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   return EXO_OK;
 }
 
+extern "C" int64_t exo_qmm_workspace(int M, int N) {
+  if (M <= 0 || N <= 0 || M > 128) return 0;
+  return (int64_t)kQmmMaxSplit * (int64_t)part_stride(M, N) * 4;
+}
+
 extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M,
                        int N, int K, int bits, int group_size, exo_stream_t stream) {
+  return exo_qmm_ws(x, w, scales, biases, residual, y, nullptr, 0, M, N, K, bits, group_size,
+                    stream);
+}
+
+extern "C" int exo_qmm_ws(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, const uint16_t* residual, uint16_t* y,
+                          void* workspace, int64_t workspace_bytes, int M, int N, int K,
+                          int bits, int group_size, exo_stream_t stream) {
   EXO_REQUIRE(bits == 4 || bits == 8, "exo_qmm: bits must be 4 or 8, got %d", bits);
   EXO_REQUIRE(group_size == 64, "exo_qmm: group_size must be 64, got %d", group_size);
   EXO_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 64 == 0, "exo_qmm: bad shape M=%d N=%d K=%d", M, N,
               K);
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmm: null pointer");
   if (M == 0) return EXO_OK;
+  if (exo_qmm_workspace(M, N) == 0) workspace = nullptr;
+  EXO_REQUIRE(!workspace || (workspace_bytes >= exo_qmm_workspace(M, N) &&
+                             ((uintptr_t)workspace & 255) == 0),
+              "exo_qmm_ws: workspace of %lld bytes, need %lld (256-byte aligned)",
+              (long long)workspace_bytes, (long long)exo_qmm_workspace(M, N));
   QmmParams p{x, w, scales, biases, residual, y, M, N, K};
   p.sorted = nullptr;
   p.tiles = nullptr;
   p.x_div = 1;
   p.w_stride = p.s_stride = 0;
+  plan_split(M, N, K, workspace != nullptr, &p.ksplit, &p.kc);
+  p.part = reinterpret_cast<float*>(workspace);
   EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm: M=%d too large", M);
   EXO_REQUIRE((int64_t)M * K < (1ll << 31), "exo_qmm: M*K=%lld exceeds 32-bit byte offsets",
               (long long)M * K);

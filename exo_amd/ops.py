@@ -148,6 +148,25 @@ def qmv_workspace(N: int, device) -> torch.Tensor:
     return cur[-1]
 
 
+_QMM_WS: dict[int, list[torch.Tensor]] = {}
+
+
+def qmm_workspace(M: int, N: int, device) -> torch.Tensor | None:
+    """Split-K workspace of the GEMM for inputs of up to 128 rows (None above), one per
+    device, grown on demand; a replaced buffer stays alive (a captured graph may still
+    point at it)."""
+    need = native.load().exo_qmm_workspace(M, N)
+    if need == 0:
+        return None
+    key = torch.device(device).index or 0
+    cur = _QMM_WS.get(key)
+    if cur is None or cur[-1].numel() < need:
+        buf = torch.empty(need, dtype=torch.uint8, device=device)
+        _QMM_WS.setdefault(key, []).append(buf)
+        cur = _QMM_WS[key]
+    return cur[-1]
+
+
 def quantized_matmul(
     x: torch.Tensor,
     qw: QuantizedWeight,
@@ -190,9 +209,19 @@ def quantized_matmul(
             "quantized_matmul(norm)",
         )
         return out
-    fn = lib.exo_qmv if M <= QMV_MAX_M else lib.exo_qmm
+    if M > QMV_MAX_M:
+        ws = qmm_workspace(M, qw.N, x.device)
+        check(
+            lib.exo_qmm_ws(
+                _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(residual),
+                _ptr(out), _ptr(ws), 0 if ws is None else ws.numel(), M, qw.N, K, qw.bits,
+                qw.group_size, _stream(),
+            ),
+            "quantized_matmul(gemm)",
+        )
+        return out
     check(
-        fn(
+        lib.exo_qmv(
             _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(residual), _ptr(out),
             M, qw.N, K, qw.bits, qw.group_size, _stream(),
         ),

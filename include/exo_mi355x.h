@@ -101,10 +101,22 @@ int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_weight, float
                            int K, int bits, int group_size, exo_stream_t stream);
 
 /* K2: the same operator for any M (prefill): weights are dequantised to bf16 in
- * LDS and multiplied on the matrix cores, float32 accumulation, bf16 out. */
+ * registers and multiplied on the matrix cores, float32 accumulation, bf16 out.
+ * (.typings/mlx/core/__init__.pyi:4198-4234) */
 int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
             const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
             int K, int bits, int group_size, exo_stream_t stream);
+/* exo_qmm with a workspace for short inputs (M <= 128, e.g. a short prompt): one row
+ * tile has too few column tiles to fill the chip, so K is split over up to 8 workgroups
+ * per tile, the float32 partial tiles go to `workspace` and a second small launch adds
+ * them in a fixed order.  exo_qmm_workspace(M, N) bytes (0: this M never splits),
+ * 256-byte aligned, no initialisation needed.  Launches that share a workspace must be
+ * ordered on one stream.  workspace == NULL behaves like exo_qmm. */
+int64_t exo_qmm_workspace(int M, int N);
+int exo_qmm_ws(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+               const uint16_t* biases, const uint16_t* residual, uint16_t* y, void* workspace,
+               int64_t workspace_bytes, int M, int N, int K, int bits, int group_size,
+               exo_stream_t stream);
 
 /* K3 for prefill-sized T: the same operator as exo_gather_qmv on the matrix cores.  The
  * (token, slot) pairs are first sorted by expert (exo_moe_group, once per routing

@@ -152,6 +152,27 @@ def test_qmm_mfma(device, bits, M, N, K):
     assert_close(got, want, what=f"qmm {M}x{N}x{K} b{bits}")
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024)])
+def test_qmm_split_k(device, bits, M, N, K):
+    """Up to 128 rows and few column tiles: K is split over workgroups and the float32
+    partial tiles are merged by the last arrival.  Against the oracle, against the
+    unsplit kernel (same products, another summation order: a few bf16 ulps at most),
+    with the residual, and twice in a row (the counters return to zero)."""
+    trip = rand_quantized(N, K, bits, seed=M + N)
+    x = rand_bf16((M, K), seed=M * 3 + 1)
+    r = rand_bf16((M, N), seed=M + 5)
+    qw, xt, rt = t_qw(trip, bits, device), t_bf16(x, device), t_bf16(r, device)
+    want = affine.qmm(x, *trip, 64, bits)
+    for _ in range(2):
+        got = ops.quantized_matmul(xt, qw)
+        assert_close(n_f32(got), want, what=f"qmm split-K {M}x{N}x{K} b{bits}")
+    unsplit = ops.qmm(xt, qw)
+    assert_close(n_f32(got), n_f32(unsplit), rtol=1e-2, what="split vs unsplit")
+    got_r = n_f32(ops.quantized_matmul(xt, qw, residual=rt))
+    assert_close(got_r, affine.bf16_round(affine.bf16_round(want) + r), what="qmm split-K + residual")
+
+
 def test_qmm_residual_and_dispatch(device):
     M, N, K, bits = 40, 192, 256, 4
     trip = rand_quantized(N, K, bits, seed=5)
