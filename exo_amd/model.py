@@ -144,6 +144,9 @@ class ShardModel:
                 cfg.bits, cfg.group_size)
         self.inv_freq = rope_inv_freq(cfg).to(self.device)
         self.scale = cfg.head_dim ** -0.5
+        # inputs of up to this many rows take the GEMV family with fused norms; 8-bit
+        # weights switch to the GEMM (separate norm launch) above 8 rows, where it is faster
+        self.gemv_rows = GEMV_MAX_ROWS if cfg.bits == 4 else 8
         self._bufs: dict[tuple[int, int], _Buffers] = {}
         self._graphs: dict[int, tuple] = {}
         self._rope_tab: torch.Tensor | None = None
@@ -187,7 +190,7 @@ class ShardModel:
     def _mlp(self, L: _Layer, bf: _Buffers, R: int) -> None:
         """h <- h + mlp(post_norm(h)) in place; bf.n holds the normed input."""
         c = self.cfg
-        gemv = R <= GEMV_MAX_ROWS
+        gemv = R <= (GEMV_MAX_ROWS if c.is_moe else self.gemv_rows)
         if not c.is_moe:
             if gemv:  # post-attention norm and SwiGLU fused into the gate/up GEMV pair
                 ops.qmv_swiglu(bf.h, L.gate, L.up, out=bf.act, norm_weight=L.post_norm,
@@ -237,7 +240,8 @@ class ShardModel:
         pos = cache.pos[rsl]
         if self.is_first:
             ops.embed(bf.tokens, self.embed_tokens, out=bf.h)
-        gemv = R <= GEMV_MAX_ROWS
+        gemv = R <= self.gemv_rows                                       # qkv, o, lm_head
+        mlp_gemv = R <= (GEMV_MAX_ROWS if c.is_moe else self.gemv_rows)  # see _mlp
         for li, L in enumerate(self.layers):
             kc, vc = cache.k[li][rsl], cache.v[li][rsl]
             if gemv:  # input norm fused into the q|k|v GEMV
@@ -255,7 +259,7 @@ class ShardModel:
                                    L.q_norm, L.k_norm, c.rms_norm_eps)
                 ops.sdpa_prefill(bf.q, kc, vc, pos, bf.attn, self.scale, B, T, Hq, Hkv, D)
             ops.quantized_matmul(bf.attn, L.o, residual=bf.h, out=bf.h)
-            if not gemv:
+            if not mlp_gemv:
                 ops.rms_norm(bf.h, L.post_norm, c.rms_norm_eps, out=bf.n)
             self._mlp(L, bf, R)
         if not self.is_last or logits_mode == "none":
@@ -264,7 +268,7 @@ class ShardModel:
         rows = hl.shape[0]
         if bf.logits is None or bf.logits.shape[0] != rows:
             bf.logits = torch.empty(rows, c.vocab_size, dtype=torch.bfloat16, device=self.device)
-        if rows <= GEMV_MAX_ROWS:  # final norm fused into the lm_head GEMV
+        if rows <= self.gemv_rows:  # final norm fused into the lm_head GEMV
             ops.quantized_matmul(hl, self.lm_head, out=bf.logits, norm_weight=self.norm,
                                  eps=c.rms_norm_eps)
         else:

@@ -188,7 +188,10 @@ def quantized_matmul(
         out = torch.empty(M, qw.N, dtype=torch.bfloat16, device=x.device)
     if norm_weight is not None and M > QMV_MAX_M:
         raise ValueError("fused rms_norm is only available on the GEMV path (M <= 16)")
-    if 2 <= M <= QMV_MAX_M:
+    # 9..16 rows: the matrix-core GEMV needs its 16-row variant there, which the split-K
+    # GEMM beats for 8-bit weights and for long rows (measured on the Llama-8B shapes)
+    gemm_rows = M > 8 and norm_weight is None and (qw.bits == 8 or K >= 8192)
+    if 2 <= M <= QMV_MAX_M and not gemm_rows:
         ws = qmv_workspace(qw.N, x.device)
         check(
             lib.exo_norm_qmv_ws(
@@ -209,7 +212,7 @@ def quantized_matmul(
             "quantized_matmul(norm)",
         )
         return out
-    if M > QMV_MAX_M:
+    if M > QMV_MAX_M or gemm_rows:
         ws = qmm_workspace(M, qw.N, x.device)
         check(
             lib.exo_qmm_ws(

@@ -136,7 +136,11 @@ def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
         fused = ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
         sep = ops.swiglu(ops.quantized_matmul(x, g, norm_weight=nw, eps=1e-5),
                          ops.quantized_matmul(x, u, norm_weight=nw, eps=1e-5))
-        assert torch.equal(fused.view(torch.int16), sep.view(torch.int16))
+        if nw is None and M > 8 and (bits == 8 or K >= 8192):
+            # these single projections take the split-K GEMM (another summation order)
+            assert_close(n_f32(fused), n_f32(sep), what="fused pair vs GEMM projections")
+        else:
+            assert torch.equal(fused.view(torch.int16), sep.view(torch.int16))
     # the shared workspace is left clean for a launch of another shape
     y = ops.quantized_matmul(x[:2], g)
     assert torch.equal(y.view(torch.int16), ops.quantized_matmul(x[:2], g).view(torch.int16))
@@ -153,7 +157,8 @@ def test_qmm_mfma(device, bits, M, N, K):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024)])
+@pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024),
+                                   (12, 256, 8192), (9, 96, 1024)])
 def test_qmm_split_k(device, bits, M, N, K):
     """Up to 128 rows and few column tiles: K is split over workgroups and the float32
     partial tiles are merged by the last arrival.  Against the oracle, against the

@@ -1,6 +1,8 @@
 """End-to-end parity of the shard forward and the generation protocol on the GPU
 against the CPU oracle, on tiny random-weight checkpoints shared through safetensors."""
 
+import time
+
 import numpy as np
 import pytest
 import torch
@@ -440,6 +442,10 @@ def test_serve_prefill_over_tcp_then_decode(ckpt, device):
         progress = []
         tps, n = D.remote_prefill(prompt + [0], dec, lambda d, t: progress.append((d, t)),
                                   endpoint=ep, request_id="req-1", model_id="tiny")
+        for _ in range(500):  # the handler thread notes the job after the client has its reply
+            if served:
+                break
+            time.sleep(0.01)
         assert served == ["req-1"] and n == len(prompt) - 2 and dec.offsets[0] == n and tps > 0
         assert progress and progress[-1][1] == len(prompt) + 1
         for i in range(len(dec)):
