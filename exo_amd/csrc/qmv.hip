@@ -560,9 +560,16 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     // (scale, bias) words: a unit pair shares the word of its even unit (low half: even
     // unit, high half: odd unit); an unpaired last unit holds its value in the low half
     uint32_t s[NMAT][UB], b[NMAT][UB];
+    // residual of row i of the batch in lane i (single activation row only): requested
+    // with the weights, so that the epilogue of a row does not wait for it
+    bf16_t res;
   };
 
   auto issue = [&](Batch& bt, int row_first) {
+    if (MT == 1 && NMAT == 1) {
+      bt.res = 0;
+      if (p.residual && lane < R) bt.res = p.residual[min(row_first + lane, r1 - 1)];
+    }
 #pragma unroll
     for (int i = 0; i < UB; ++i) {
       // rows past the end of the range re-read its last row (results are dropped)
@@ -663,6 +670,9 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
           float rsum[NMAT];
 #pragma unroll
           for (int a = 0; a < NMAT; ++a) rsum[a] = wave_sum_to_lane63(acc[a][m]);
+          float resv = 0.f;
+          if (MT == 1 && NMAT == 1)
+            resv = bf2f((bf16_t)__builtin_amdgcn_readlane((int)bt.res, r));
           if (lane == 63 && m < p.M) {
             const size_t o = (size_t)m * p.N + row;
             float out;
@@ -671,7 +681,8 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
               out = g / (1.f + __expf(-g)) * up;
             } else {
               out = rsum[0];
-              if (p.residual) out = bf2f(f2bf(out)) + bf2f(p.residual[o]);
+              if (p.residual)
+                out = bf2f(f2bf(out)) + ((MT == 1 && NMAT == 1) ? resv : bf2f(p.residual[o]));
             }
             yout[o] = f2bf(out);
           }
