@@ -3,19 +3,27 @@
 // Matrix-core design for gfx950.  A 256-thread workgroup (2 x 2 waves) computes a
 // 256x128 output tile (128x128 for M <= 128); one 64-wide K step per iteration = exactly
 // one quantisation group, so a packed row segment needs a single (scale, bias).
-//  * Activations go through LDS (two buffers: the next tile is stored while the current
-//    one is multiplied, one barrier per K step).  LDS bandwidth, not the matrix cores, is
-//    what limits this kernel, so the weights do NOT go through LDS:
+//  * Activations go from global memory straight into LDS (buffer_load_dwordx4 ... lds: no
+//    registers, no LDS store instructions), two tile buffers, one barrier per K step.  The
+//    tile rows are 128 bytes apart without padding (the loads write in lane order); chunk c
+//    of row r sits at slot c ^ (r % 8), so the operand reads of 16 rows spread over the
+//    banks.  LDS bandwidth, not the matrix cores, limited the first version of this kernel,
+//    so the weights do NOT go through LDS:
 //  * every wave loads the packed words of its own 64 weight rows straight into registers
 //    in the MFMA B-operand layout - lane (row, half) takes 16 B (4-bit) or 32 B (8-bit) =
 //    32 consecutive codes - and dequantises them there to bf16(fma(s, q, b)) with
 //    v_cvt_f32_ubyteN.  MFMA step t of a K step then covers k = 32*half + 8*t .. +8, and
-//    the A operand is read from the activation tile at that same offset, so no data is
-//    rearranged.  The two waves that share weight rows dequantise them twice; in exchange
-//    the LDS carries a third less traffic and its writes are plain copies.
-//  * v_mfma_f32_32x32x16_bf16, float32 accumulators (128x64 per wave), global loads two
-//    K steps ahead in registers.  LDS rows are padded by 16 bytes: conflict-free b128.
+//    the A operand is read from the activation tile at that same offset.  The two waves
+//    that share weight rows dequantise them twice; in exchange the LDS carries a third less
+//    traffic.
+//  * All global loads are buffer loads: workgroup-uniform descriptors, 32-bit lane offsets
+//    that never change, the K step as the scalar offset - no address arithmetic in the
+//    loop.  (scale, bias) of four K steps come in one 8-byte load when K % 256 == 0.
+//  * v_mfma_f32_32x32x16_bf16, float32 accumulators (128x64 per wave); the tile and the
+//    weights of the next K step are requested before the current one is multiplied.
 //  * grouped mode (MoE prefill): blockIdx.y is a tile of one expert's sorted rows.
+//  * up to 128 rows and few column tiles: blockIdx.z splits K; float32 partial tiles and a
+//    small reduce launch.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 
@@ -61,6 +69,14 @@ __device__ __forceinline__ float ubyte_f(uint32_t v) {
 // range check (every offset the kernel forms is in range by construction)
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
+}
+
+// 16 bytes per lane from a buffer straight into LDS: lane l of the wave writes
+// lds_base + 16*l (buffer_load_dwordx4 ... lds); completion is counted by vmcnt
+__device__ __forceinline__ void load_to_lds16(__amdgpu_buffer_rsrc_t rsrc, void* lds_base,
+                                              uint32_t voffset, uint32_t soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(
+      rsrc, (__attribute__((address_space(3))) void*)lds_base, 16, voffset, soffset, 0, 0);
 }
 
 // elements between the partial tiles of consecutive K ranges (16-byte aligned rows of 4)
@@ -109,7 +125,8 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LDS_STRIDE];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * BN;
   const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 64;
   const int G = p.K >> 6;
@@ -155,23 +172,29 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   uint32_t xoff[XR];
 #pragma unroll
   for (int r = 0; r < XR; ++r) {
+    // 16-byte chunk `id` of the LDS tile (row id/8, slot id%8) holds chunk slot ^ (row%8) of
+    // that activation row: rows are 128 bytes apart without padding (the loads write LDS in
+    // lane order), and the XOR keeps the operand reads of 16 rows off each other's banks
     const int id = tid + kThreads * r;
-    const int row = min(id >> 3, m_end - 1 - m0), kp = id & 7;
+    const int trow = id >> 3, kp = (id & 7) ^ (trow & 7);
+    const int row = min(trow, m_end - 1 - m0);
     const uint32_t src = GROUPED ? (uint32_t)(row_pair[row] / p.x_div) : (uint32_t)(m0 + row);
     xoff[r] = (src * (uint32_t)p.K + kp * 8) * 2;  // bytes
   }
 
-  struct XStage {
-    uint4 xa[XR];
-  };
   struct WStage {
     WRaw<BITS> w[2];
   };
 
-  auto load_x = [&](XStage& st, int k0) {
+  // the activation tile goes from global memory straight into LDS (no registers, no LDS
+  // store instructions): wave instruction r writes chunks [wave*64 + 256*r, +64) in lane
+  // order.  Completion is counted by vmcnt.
+  char* const tiles = reinterpret_cast<char*>(&xs[0][0]);
+  constexpr int TILE_BYTES = BM * 128;
+  auto load_x = [&](int buf, int k0) {
 #pragma unroll
     for (int r = 0; r < XR; ++r)
-      st.xa[r] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[r], k0 * 2, 0));
+      load_to_lds16(rx, tiles + buf * TILE_BYTES + (wave * 64 + kThreads * r) * 16, xoff[r], k0 * 2);
   };
   auto load_w = [&](WStage& st, int k0) {
 #pragma unroll
@@ -202,14 +225,10 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     return (e & 1) ? bf_hi(w) : bf_lo(w);
   };
 
-  auto store_x = [&](const XStage& st, int buf) {
+  // byte offset of this lane's operand chunk of MFMA step t inside its tile row
+  int aoff[4];
 #pragma unroll
-    for (int r = 0; r < XR; ++r) {
-      const int id = tid + kThreads * r;
-      const int row = id >> 3, kp = id & 7;
-      *reinterpret_cast<uint4*>(&xs[buf][row * LDS_STRIDE + kp * 8]) = st.xa[r];
-    }
-  };
+  for (int t = 0; t < 4; ++t) aoff[t] = ((kq * 4 + t) ^ (frow & 7)) * 16;
 
   floatx16 acc[MI][2];
 #pragma unroll
@@ -230,11 +249,11 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     }
     // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step.  The A operands of step t+1
     // are requested before the products of step t, so their LDS latency hides behind them.
-    const bf16_t* arow = &xs[buf][(wm + frow) * LDS_STRIDE + kq * 32];
+    const char* arow = tiles + buf * TILE_BYTES + (wm + frow) * 128;
     bf16x8_t a[2][MI];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
-      a[0][i] = *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * LDS_STRIDE);
+      a[0][i] = *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * 128 + aoff[0]);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       bf16x8_t bq[2];
@@ -242,7 +261,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
           a[(t + 1) & 1][i] =
-              *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * LDS_STRIDE + (t + 1) * 8);
+              *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * 128 + aoff[t + 1]);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) bq[j] = dequant8<BITS>(st.w[j], t, sc[j], bi[j]);
@@ -261,21 +280,19 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // this workgroup's K range (all of K unless split; a multiple of four K steps)
   const int kb = GROUPED ? 0 : (int)blockIdx.z * p.kc;
   const int ke = GROUPED ? p.K : min(p.K, kb + p.kc);
-  XStage xr;
   WStage w0, w1;
   SBlock sb0, sb1;  // current block of four K steps, next block
   if (SB4) {
     load_sb(sb0, kb >> 8);
     sb1 = sb0;
   }
-  load_x(xr, kb);
+  load_x(0, kb);
   load_w(w0, kb);
-  store_x(xr, 0);
-  if (kb + BK < ke) {
-    load_x(xr, kb + BK);
-    load_w(w1, kb + BK);
-  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile is in LDS
   __syncthreads();
+  // At K step k: the x tile of k is in LDS buffer k&1 and the packed weights of k in w0.
+  // The tile and the weights of k+1 are requested first, then tile k is multiplied; every
+  // load of the step has landed before the one barrier that ends it.
   int buf = 0;
   for (int k0 = kb; k0 < ke; k0 += BK) {
     const int ks = k0 >> 6;
@@ -283,11 +300,13 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
       sb0 = sb1;
       if (k0 + 4 * BK < ke) load_sb(sb1, (ks >> 2) + 1);
     }
-    if (k0 + BK < ke) store_x(xr, buf ^ 1);
-    if (k0 + 2 * BK < ke) load_x(xr, k0 + 2 * BK);
+    if (k0 + BK < ke) {
+      load_x(buf ^ 1, k0 + BK);
+      load_w(w1, k0 + BK);
+    }
     multiply(w0, buf, sb0, ks & 3);
-    w0 = w1;  // a few register moves keep the loop body single (no unrolled twin)
-    if (k0 + 2 * BK < ke) load_w(w1, k0 + 2 * BK);
+    w0 = w1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     buf ^= 1;
   }
