@@ -903,6 +903,146 @@ int launch_ksplit(const QmvParams& p, hipStream_t st) {
   return EXO_OK;
 }
 
+
+// ---------------------------------------------------------------------------
+// Decode-side SwitchGLU down projection fused with the weighted sum over the token's
+// top-k experts and the residual (mx.gather_qmm + the `(y * scores[..., None]).sum(-2)`
+// of the MoE block + `h + r`):
+//   out[t,n] = bf16( bf16( sum_j bf16( bf16(W[e_j][n,:] . x[t,j,:]) * score[t,j] ) ) + res[t,n] )
+// - the same rounding points as exo_gather_qmv followed by exo_moe_combine.
+// blockIdx.y = token; a workgroup has one wave per expert slot.  Wave j stages ITS
+// activation row x[t,j,:], multiplies kDownRW sets of 64/LPR rows of expert e_j (all its
+// loads in flight from the start) and leaves bf16(bf16(dot) * score_j) in LDS; the first
+// wave adds the k contributions in slot order.  The launch is latency-bound, hence the
+// many short waves.
+struct DownCombineParams {
+  const bf16_t* x;       // [T, topk, K]
+  const uint32_t* w;     // [E, N, wpr]
+  const bf16_t* s;       // [E, N, K/64]
+  const bf16_t* b;
+  const int32_t* idx;    // [T, topk]
+  const bf16_t* scores;  // [T, topk]
+  const bf16_t* residual;  // [T, N] or null
+  bf16_t* out;           // [T, N]
+  int topk, E, N, K, wpr, lpr_log2, iters;
+};
+
+constexpr int kDownMaxIters = 4;  // 16-byte chunks per lane and expert row
+constexpr int kDownMaxTopk = 8;
+constexpr int kDownRW = 2;        // row sets per wave
+
+template <int BITS>
+__global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
+    const DownCombineParams p) {
+  extern __shared__ uint4 smem[];
+  constexpr int GSHIFT = (BITS == 4) ? 1 : 2;
+  const int cpr = p.wpr >> 2;
+  const int lane = threadIdx.x & 63;
+  const int slot = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // one wave per slot
+  uint4* xs = smem + (size_t)slot * p.wpr;                                                // [wpr]
+  float2* sx = reinterpret_cast<float2*>(smem + (size_t)p.topk * p.wpr) + (size_t)slot * cpr;  // [cpr]
+  __shared__ float contrib[kDownMaxTopk][kDownRW * 64];
+
+  const int lpr = 1 << p.lpr_log2;
+  const int rpwi = 64 >> p.lpr_log2;
+  const int sl = lane & (lpr - 1), sub = lane >> p.lpr_log2;
+  const int G = p.K >> 6;
+  const int t = blockIdx.y;
+  const int row0 = (int)blockIdx.x * (kDownRW * rpwi);
+
+  int e = p.idx[(size_t)t * p.topk + slot];
+  e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+  const float score = bf2f(p.scores[(size_t)t * p.topk + slot]);
+
+  // every weight load of this wave goes out first
+  uint4 wv[kDownRW][kDownMaxIters];
+  bf16_t sv[kDownRW][kDownMaxIters], bv[kDownRW][kDownMaxIters];
+#pragma unroll
+  for (int i = 0; i < kDownRW; ++i) {
+    const int row = min(row0 + i * rpwi + sub, p.N - 1);  // rows past N: not stored
+    const size_t r = (size_t)e * p.N + row;
+    const uint32_t* wp = p.w + r * p.wpr + sl * 4;
+    const bf16_t* sp = p.s + r * G + (sl >> GSHIFT);
+    const bf16_t* bp = p.b + r * G + (sl >> GSHIFT);
+#pragma unroll
+    for (int j = 0; j < kDownMaxIters; ++j)
+      if (j < p.iters) {
+        wv[i][j] = *reinterpret_cast<const uint4*>(wp + (size_t)j * lpr * 4);
+        sv[i][j] = sp[j * (lpr >> GSHIFT)];
+        bv[i][j] = bp[j * (lpr >> GSHIFT)];
+      }
+  }
+
+  // stage this slot's activation row: word wi -> xs[(j*4 + w4) * LPR + sl] in dot2 order,
+  // per-chunk sums to sx[chunk]; four consecutive lanes hold one chunk
+  {
+    const bf16_t* xt = p.x + ((size_t)t * p.topk + slot) * p.K;
+    for (int base = 0; base < p.wpr; base += 64 * 4) {
+      uint4 raw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        raw[u] = load_word_x<BITS>(xt, min(base + u * 64 + lane, p.wpr - 1));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int wi = base + u * 64 + lane;
+        const int c = wi >> 2, w4 = wi & 3;
+        const int j = c >> p.lpr_log2, csl = c & (lpr - 1);
+        float stored, truesum;
+        const uint4 o = permute_word<BITS>(raw[u], stored, truesum);
+        stored += __shfl_xor(stored, 1, 64);
+        truesum += __shfl_xor(truesum, 1, 64);
+        stored += __shfl_xor(stored, 2, 64);
+        truesum += __shfl_xor(truesum, 2, 64);
+        if (wi < p.wpr) {
+          xs[(((j << 2) + w4) << p.lpr_log2) + csl] = o;
+          if (w4 == 0) sx[c] = make_float2(128.f * stored, truesum);
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
+  asm volatile("" : "+s"(kmask));
+  asm volatile("" : "+v"(kmagic));
+#pragma unroll
+  for (int i = 0; i < kDownRW; ++i) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < kDownMaxIters; ++j)
+      if (j < p.iters) {
+        const float2 sm = sx[(j << p.lpr_log2) + sl];
+        float d = -sm.x;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+          uint32_t pr[4];
+          unpack_word_r(reinterpret_cast<const uint32_t*>(&wv[i][j])[w4], kmask, kmagic, pr);
+          const uint4 xv = xs[(((j << 2) + w4) << p.lpr_log2) + sl];
+          d = dot2_bf16(pr[0], xv.x, d);
+          d = dot2_bf16(pr[1], xv.y, d);
+          d = dot2_bf16(pr[2], xv.z, d);
+          d = dot2_bf16(pr[3], xv.w, d);
+        }
+        acc = fmaf(bf2f(sv[i][j]), d, acc);
+        acc = fmaf(bf2f(bv[i][j]), sm.y, acc);
+      }
+    acc = group_sum(acc, lpr);
+    if (sl == 0) contrib[slot][i * rpwi + sub] = bf2f(f2bf(bf2f(f2bf(acc)) * score));
+  }
+  __syncthreads();
+
+  if (slot == 0 && lane < kDownRW * rpwi) {
+    const int row = row0 + lane;  // lane = i * rpwi + sub
+    if (row < p.N) {
+      float total = 0.f;
+      for (int j = 0; j < p.topk; ++j) total += contrib[j][lane];
+      float o = bf2f(f2bf(total));
+      if (p.residual) o += bf2f(p.residual[(size_t)t * p.N + row]);
+      p.out[(size_t)t * p.N + row] = f2bf(o);
+    }
+  }
+}
+
 struct Plan {
   int lpr_log2, iters, slots, spw, grid, ragged;
   size_t lds;
@@ -1276,4 +1416,53 @@ extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, cons
                                      exo_stream_t stream) {
   return exo_norm_gather_qmv_swiglu(x, nullptr, 0.f, wg, sg, bg, wu, su, bu, idx, y, T, topk, E,
                                     N, K, bits, group_size, stream);
+}
+
+extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                                      const uint16_t* biases, const int32_t* idx,
+                                      const uint16_t* scores, const uint16_t* residual,
+                                      uint16_t* out, uint16_t* scratch, int T, int topk, int E,
+                                      int N, int K, int bits, int group_size,
+                                      exo_stream_t stream) {
+  int rc = check_common("exo_gather_qmv_combine", 1, N, K, bits, group_size);
+  if (rc) return rc;
+  rc = check_gather("exo_gather_qmv_combine", T, topk, topk, E);
+  if (rc) return rc;
+  EXO_REQUIRE(x && w && scales && biases && idx && scores && out,
+              "exo_gather_qmv_combine: null pointer");
+  Plan pl;
+  const bool fused = make_plan(N, K, bits, 1, &pl) && pl.iters <= kDownMaxIters &&
+                     topk <= kDownMaxTopk && T <= 65535;
+  if (!fused) {
+    EXO_REQUIRE(scratch, "exo_gather_qmv_combine: topk=%d K=%d needs the scratch buffer", topk, K);
+    rc = exo_gather_qmv(x, w, scales, biases, idx, scratch, T, topk, topk, E, N, K, bits,
+                        group_size, stream);
+    if (rc) return rc;
+    return exo_moe_combine(scratch, scores, residual, out, T, topk, N, stream);
+  }
+  DownCombineParams p;
+  p.x = x;
+  p.w = w;
+  p.s = scales;
+  p.b = biases;
+  p.idx = idx;
+  p.scores = scores;
+  p.residual = residual;
+  p.out = out;
+  p.topk = topk;
+  p.E = E;
+  p.N = N;
+  p.K = K;
+  p.wpr = K * bits / 32;
+  p.lpr_log2 = pl.lpr_log2;
+  p.iters = pl.iters;
+  const int rpwi = 64 >> pl.lpr_log2;
+  const dim3 grid(exo_ceil_div(N, kDownRW * rpwi), T);
+  const size_t lds = (size_t)topk * ((size_t)p.wpr * 16 + (size_t)(p.wpr / 4) * 8);
+  if (bits == 4)
+    moe_down_combine_kernel<4><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+  else
+    moe_down_combine_kernel<8><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+  EXO_CHECK_LAUNCH("exo_gather_qmv_combine");
+  return EXO_OK;
 }

@@ -225,8 +225,8 @@ class ShardModel:
             return
         ops.gather_qmv_swiglu(bf.h, L.gate, L.up, idx, out=bf.act, norm_weight=L.post_norm,
                               eps=c.rms_norm_eps)
-        ops.gather_qmm(bf.act, L.down, idx, out=bf.expert_out)
-        ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
+        ops.gather_qmv_combine(bf.act, L.down, idx, sc, residual=bf.h, out=bf.h,
+                               scratch=bf.expert_out)
 
     def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
              rows: slice | None = None):

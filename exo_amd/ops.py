@@ -299,6 +299,27 @@ def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, 
     return out
 
 
+def gather_qmv_combine(x, qw: QuantizedWeight, idx, scores, residual=None, out=None, scratch=None):
+    """SwitchGLU's down projection for decode-sized inputs fused with the weighted sum over
+    the top-k experts and the residual: x bf16 [T,topk,K], idx int32 [T,topk], scores bf16
+    [T,topk], residual bf16 [T,N] -> bf16 [T,N].  ``scratch`` (bf16 [T,topk,N]) serves the
+    shapes the fused kernel does not take."""
+    lib = native.load()
+    T, topk, K = x.shape
+    E = qw.weight.shape[0]
+    if out is None:
+        out = torch.empty(T, qw.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_gather_qmv_combine(
+            _ptr(x), _ptr(qw.weight), _ptr(qw.scales), _ptr(qw.biases), _ptr(idx), _ptr(scores),
+            _ptr(residual), _ptr(out), _ptr(scratch), T, topk, E, qw.N, K, qw.bits,
+            qw.group_size, _stream(),
+        ),
+        "gather_qmv_combine",
+    )
+    return out
+
+
 def moe_group(idx: torch.Tensor, E: int) -> torch.Tensor:
     """Sort the (token, slot) pairs of idx int32 [T, topk] by expert; the returned workspace
     feeds grouped_qmm for every projection that shares this routing decision."""

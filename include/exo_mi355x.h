@@ -242,6 +242,19 @@ int exo_swiglu(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t 
 int exo_router_topk(const uint16_t* logits, int32_t* idx, uint16_t* scores, int rows, int E,
                     int k, int renorm, exo_stream_t stream);
 
+/* K3 (down projection of SwitchGLU, decode) fused with the block's weighted sum over
+ * the top-k experts and the residual: out[t,:] = bf16(bf16(sum_j bf16(bf16(x[t,j,:] @
+ * dq(w[idx[t,j]])^T) * scores[t,j])) + residual[t,:]), the rounding points of
+ * exo_gather_qmv followed by exo_moe_combine.  x bf16 [T,topk,K], out bf16 [T,N].
+ * Shapes outside the fused kernel (topk > 8, or rows of more than 4 chunks per lane) run
+ * those two calls through `scratch` (bf16 [T,topk,N]); scratch may be NULL otherwise.
+ * (.typings/mlx/core/__init__.pyi:2957-3006; .typings/mlx_lm/models/switch_layers.pyi:59-73) */
+int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, const int32_t* idx, const uint16_t* scores,
+                           const uint16_t* residual, uint16_t* out, uint16_t* scratch, int T,
+                           int topk, int E, int N, int K, int bits, int group_size,
+                           exo_stream_t stream);
+
 /* MoE combine: out[t,:] = bf16( sum_j bf16(y[t,j,:] * scores[t,j]) ) (+ residual[t,:]
  * added in bf16 when non-null).  y bf16 [T,topk,H]. */
 int exo_moe_combine(const uint16_t* y, const uint16_t* scores, const uint16_t* residual,

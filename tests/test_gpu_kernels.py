@@ -370,6 +370,33 @@ def test_router_topk(device, E, k, renorm):
     assert_close(n_f32(sc), wsc, rtol=2.0**-7, what="router scores")
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("E,N,K,T,topk", [(6, 200, 768, 3, 8), (5, 96, 1536, 2, 4), (4, 64, 2048, 1, 2),
+                                          (3, 72, 192, 2, 3), (9, 64, 768, 2, 9)])
+def test_gather_qmv_combine(device, bits, E, N, K, T, topk):
+    """Down projection of SwitchGLU + weighted sum over the experts + residual in one
+    launch: against the oracle, and against the two separate launches it replaces
+    (same rounding points; the dot products are summed in another order).  The last two
+    shapes take the fallback through the scratch buffer (rows that share a wave by
+    threes; more than 8 experts per token)."""
+    trip = rand_quantized(N, K, bits, seed=E + N, E=E)
+    idx = rng(43).integers(0, E, size=(T, topk)).astype(np.int32)
+    x = rand_bf16((T, topk, K), seed=44)
+    sc = affine.bf16_round(np.abs(rand_bf16((T, topk), seed=45)) / 8)
+    r = rand_bf16((T, N), seed=46)
+    qw, xt, it = t_qw(trip, bits, device), t_bf16(x, device), torch.from_numpy(idx).to(device)
+    st, rt = t_bf16(sc, device), t_bf16(r, device)
+    scratch = torch.empty(T, topk, N, dtype=torch.bfloat16, device=device)
+    got = ops.gather_qmv_combine(xt, qw, it, st, residual=rt, scratch=scratch)
+    eo = affine.gather_qmm(x, *trip, idx, 64, bits)
+    acc = affine.bf16_round(affine.bf16_round(eo * sc[..., None]).sum(1, dtype=np.float32))
+    assert_close(n_f32(got), affine.bf16_round(acc + r), what="gather_qmv_combine")
+    sep = ops.moe_combine(ops.gather_qmm(xt, qw, it), st, rt)
+    assert_close(n_f32(got), n_f32(sep), rtol=1e-2, what="fused vs separate")
+    no_res = ops.gather_qmv_combine(xt, qw, it, st, scratch=scratch)
+    assert_close(n_f32(no_res), acc, what="gather_qmv_combine without residual")
+
+
 def test_moe_combine(device):
     T, topk, H = 3, 8, 2048
     y = rand_bf16((T, topk, H), seed=1)
