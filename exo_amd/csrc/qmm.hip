@@ -113,6 +113,26 @@ __device__ __forceinline__ bf16x8_t dequant8(const WRaw<BITS>& r, int t, float s
   return __builtin_bit_cast(bf16x8_t, o);
 }
 
+// One 32-bit register (two bf16) of that operand: piece P = 0..3.  `lo`, `hi` are the two
+// source words prepared by dequant_words().
+template <int BITS>
+__device__ __forceinline__ void dequant_words(const WRaw<BITS>& r, int t, uint32_t& lo, uint32_t& hi) {
+  if (BITS == 4) {
+    const uint32_t v = reinterpret_cast<const uint32_t*>(&r.q[0])[t];
+    lo = v & 0x0f0f0f0fu;         // even codes, one per byte
+    hi = (v >> 4) & 0x0f0f0f0fu;  // odd codes
+  } else {
+    lo = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t];
+    hi = reinterpret_cast<const uint32_t*>(&r.q[0])[2 * t + 1];
+  }
+}
+template <int BITS, int P>
+__device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, float s, float b) {
+  if (BITS == 4) return pack_bf2(fmaf(s, ubyte_f<P>(lo), b), fmaf(s, ubyte_f<P>(hi), b));
+  const uint32_t v = P < 2 ? lo : hi;
+  return pack_bf2(fmaf(s, ubyte_f<(2 * P) & 3>(v), b), fmaf(s, ubyte_f<((2 * P) & 3) + 1>(v), b));
+}
+
 // MI = 32-row MFMA tiles per wave along M: the workgroup tile is (64*MI) x 128.
 // SB4: rows of scales / biases are 8-byte aligned (K a multiple of 256), so the (scale,
 // bias) of four consecutive K steps come in one 8-byte load each instead of four 2-byte
@@ -247,29 +267,53 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
       bi[j] = SB4 ? pick(sb.b[j], e) : bf2f(st.w[j].b);
       if (!w_ok[j]) sc[j] = bi[j] = 0.f;
     }
-    // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step.  The A operands of step t+1
-    // are requested before the products of step t, so their LDS latency hides behind them.
+    // MFMA step t covers k = 32*kq + 8*t .. +8 of the K step.  Software pipeline: the A
+    // operands and the dequantised B operands of step t+1 are produced while the products
+    // of step t run - a 32x32x16 MFMA occupies the matrix core for 8 passes, time for about
+    // seven vector instructions of the same wave.  The order is pinned slot by slot (one
+    // MFMA, one register of the next B operand, one LDS read) with scheduling barriers;
+    // left alone, the compiler clumps the MFMAs behind all the vector work.
+    static_assert(MI == 2 || MI == 4, "eight operand registers are spread over 2*MI slots");
     const char* arow = tiles + buf * TILE_BYTES + (wm + frow) * 128;
     bf16x8_t a[2][MI];
+    uint4 bq[2][2];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
       a[0][i] = *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * 128 + aoff[0]);
 #pragma unroll
+    for (int j = 0; j < 2; ++j) bq[0][j] = __builtin_bit_cast(uint4, dequant8<BITS>(st.w[j], 0, sc[j], bi[j]));
+#pragma unroll
     for (int t = 0; t < 4; ++t) {
-      bf16x8_t bq[2];
+      const int cur = t & 1, nxt = cur ^ 1;
+      uint32_t lo[2], hi[2];
       if (t < 3) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
-          a[(t + 1) & 1][i] =
-              *reinterpret_cast<const bf16x8_t*>(arow + i * 32 * 128 + aoff[t + 1]);
+        for (int j = 0; j < 2; ++j) dequant_words<BITS>(st.w[j], t + 1, lo[j], hi[j]);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) bq[j] = dequant8<BITS>(st.w[j], t, sc[j], bi[j]);
+      for (int m = 0; m < 2 * MI; ++m) {
+        const int i = m >> 1, j = m & 1;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[cur][i], __builtin_bit_cast(bf16x8_t, bq[cur][j]), acc[i][j], 0, 0, 0);
+        if (t < 3) {
+          // 8 registers of the next B operands over the 2*MI slots
+          constexpr int PER = 8 / (2 * MI);
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1][i], bq[j], acc[i][j], 0, 0, 0);
+          for (int u = 0; u < PER; ++u) {
+            const int r8 = m * PER + u, jj = r8 >> 2;
+            uint32_t* dst = reinterpret_cast<uint32_t*>(&bq[nxt][jj]);
+            switch (r8 & 3) {
+              case 0: dst[0] = dequant_piece<BITS, 0>(lo[jj], hi[jj], sc[jj], bi[jj]); break;
+              case 1: dst[1] = dequant_piece<BITS, 1>(lo[jj], hi[jj], sc[jj], bi[jj]); break;
+              case 2: dst[2] = dequant_piece<BITS, 2>(lo[jj], hi[jj], sc[jj], bi[jj]); break;
+              default: dst[3] = dequant_piece<BITS, 3>(lo[jj], hi[jj], sc[jj], bi[jj]); break;
+            }
+          }
+          if (m < MI)
+            a[nxt][m] = *reinterpret_cast<const bf16x8_t*>(arow + m * 32 * 128 + aoff[t + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
