@@ -358,40 +358,15 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
       bool write = !pair_open;
       if (p.ksplit > 1) {
         // partial sums go out at device scope (the merging workgroup may sit on another
-        // XCD); the last of the ksplit workgroups of this row block adds them up in a
-        // fixed order, so the result does not depend on arrival order
+        // XCD) and are added up after the last row block, see the end of the kernel:
+        // nothing here waits for them
 #pragma unroll
         for (int q = 0; q < MR; ++q) {
           const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
           if (m < p.M && row < p.N)
             st_dev(&p.part[(((size_t)blockIdx.y * nmat + mat) * p.M + m) * p.N + row], v[q]);
         }
-        if (!pair_open) {
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-          int last = 0;
-          if (lane == 0) {
-            const int old = __hip_atomic_fetch_add(&p.counters[blk], 1, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-            last = (old == p.ksplit - 1);
-            if (last)
-              __hip_atomic_store(&p.counters[blk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-          write = __builtin_amdgcn_readfirstlane(last) != 0;
-          if (write) {
-#pragma unroll
-            for (int q = 0; q < MR; ++q) {
-              const int m = 8 * (q >> 2) + 4 * Rg + (q & 3);
-              float t = 0.f, tg = 0.f;
-              if (m < p.M && row < p.N)
-                for (int ks = 0; ks < p.ksplit; ++ks) {
-                  t += ld_dev(&p.part[(((size_t)ks * nmat + mat) * p.M + m) * p.N + row]);
-                  if (nmat == 2) tg += ld_dev(&p.part[((size_t)ks * nmat * p.M + m) * p.N + row]);
-                }
-              v[q] = t;
-              vg[q] = tg;
-            }
-          }
-        }
+        write = false;
       } else if (pair_open) {
 #pragma unroll
         for (int q = 0; q < MR; ++q) vg[q] = v[q];
@@ -426,6 +401,46 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
     consume(b1, it % n_super);
     if (it % n_super == n_super - 1) finish_block(blk_of(it), mat_of(it));
     if (++it >= n_items) break;
+  }
+  if (p.ksplit == 1) return;
+
+  // Split K: the ksplit workgroups of one blockIdx.x have walked the same row blocks.  The
+  // last of them to get here adds the float32 partials of all those blocks, in a fixed
+  // order (the result does not depend on arrival order), and writes y.  One counter round
+  // trip per workgroup, after the streaming, instead of one per row block inside it.
+  __shared__ int s_last;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this wave's partials are out
+  __syncthreads();
+  if (tid == 0) {
+    int* cnt = &p.counters[blockIdx.x];
+    const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == p.ksplit - 1);
+    if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  const int per_blk = 32 * p.M;
+  const int total = my_blocks * NG * per_blk;
+  const size_t mstride = (size_t)p.M * p.N;  // one matrix of one K chunk
+  for (int e = tid; e < total; e += kThreads) {
+    const int bq = e / per_blk, rem = e - bq * per_blk;
+    const int m = rem >> 5;
+    const int blk = ((int)blockIdx.x + (bq / NG) * (int)gridDim.x) * NG + bq % NG;
+    const int row = blk * 32 + (rem & 31);
+    if (blk >= NB || row >= p.N) continue;
+    const size_t o = (size_t)m * p.N + row;
+    float t = 0.f, tg = 0.f;
+    for (int ks = 0; ks < p.ksplit; ++ks) {
+      t += ld_dev(&p.part[((size_t)ks * nmat + (nmat - 1)) * mstride + o]);
+      if (nmat == 2) tg += ld_dev(&p.part[(size_t)ks * nmat * mstride + o]);
+    }
+    if (nmat == 2) {  // SwiGLU on the bf16-rounded projections
+      const float g = bf2f(f2bf(tg)), up = bf2f(f2bf(t));
+      t = g / (1.f + __expf(-g)) * up;
+    } else if (p.residual) {
+      t = bf2f(f2bf(t)) + bf2f(p.residual[o]);
+    }
+    p.y[o] = f2bf(t);
   }
 }
 
