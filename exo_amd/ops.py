@@ -189,8 +189,8 @@ def quantized_matmul(
     if norm_weight is not None and M > QMV_MAX_M:
         raise ValueError("fused rms_norm is only available on the GEMV path (M <= 16)")
     # 9..16 rows: the matrix-core GEMV needs its 16-row variant there, which the split-K
-    # GEMM beats for 8-bit weights and for long rows (measured on the Llama-8B shapes)
-    gemm_rows = M > 8 and norm_weight is None and (qw.bits == 8 or K >= 8192)
+    # GEMM matches or beats for 8-bit weights (measured on the Llama-8B shapes)
+    gemm_rows = M > 8 and norm_weight is None and qw.bits == 8
     if 2 <= M <= QMV_MAX_M and not gemm_rows:
         ws = qmv_workspace(qw.N, x.device)
         check(

@@ -136,7 +136,7 @@ def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
         fused = ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
         sep = ops.swiglu(ops.quantized_matmul(x, g, norm_weight=nw, eps=1e-5),
                          ops.quantized_matmul(x, u, norm_weight=nw, eps=1e-5))
-        if nw is None and M > 8 and (bits == 8 or K >= 8192):
+        if nw is None and M > 8 and bits == 8:
             # these single projections take the split-K GEMM (another summation order)
             assert_close(n_f32(fused), n_f32(sep), what="fused pair vs GEMM projections")
         else:
