@@ -51,6 +51,11 @@ struct QmmParams {
   // float32 partial tile; qmm_reduce_kernel adds them
   int ksplit, kc;
   float* part;  // [ksplit][M][N]
+  // pair mode (Llama MLP, prefill): w/s/b is the gate matrix, w2/s2/b2 the up matrix, both
+  // [N, K]; y[M,N] = silu(x gate^T) * (x up^T) with both projections rounded to bf16 first
+  const uint32_t* w2 = nullptr;
+  const bf16_t* s2 = nullptr;
+  const bf16_t* b2 = nullptr;
 };
 
 // byte I of v as float.  Written as the instruction: the compiler otherwise extracts
@@ -138,17 +143,21 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // bias) of four consecutive K steps come in one 8-byte load each instead of four 2-byte
 // ones - a 2-byte load that touches 32 rows costs the memory pipeline as much as a
 // 16-byte one.
-template <int BITS, int MI, bool GROUPED = false, bool SB4 = false>
+// PAIR: the workgroup's 128 weight rows are 64 rows of the gate matrix and the same 64 rows
+// of the up matrix - a wave's two column tiles are (gate, up) of the same 32 output columns,
+// so the SwiGLU happens in the epilogue and neither projection is written to memory.
+template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false>
 __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   constexpr int kThreads = 256;
-  constexpr int BM = 64 * MI, BN = 128;
+  constexpr int BM = 64 * MI, BN = PAIR ? 64 : 128;  // BN: output columns per workgroup
+  constexpr int WN = PAIR ? 32 : 64;                 // output columns per wave
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * BN;
-  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * 64;
+  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * WN;
   const int G = p.K >> 6;
   const int wpr = p.K * BITS / 32;
   int m0 = blockIdx.y * BM, m_end = p.M;
@@ -177,7 +186,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   bool w_ok[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn + j * 32 + frow;
+    const int n = n0 + wn + (PAIR ? 0 : j * 32) + frow;
     w_ok[j] = n < p.N;
     const uint32_t rel = (uint32_t)(min(n, p.N - 1) - n0);  // rows past N re-read the last one
     woff[j] = (rel * (uint32_t)wpr + kq * BITS) * 4;  // bytes; 32 codes = BITS words per half K step
@@ -185,8 +194,18 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   }
   // Loads go through buffer instructions: a workgroup-uniform descriptor, a 32-bit lane
   // offset that never changes, and the K step as the scalar offset.
-  const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x), rw = make_rsrc(wbase), rs = make_rsrc(sbase),
-                               rb = make_rsrc(bbase);
+  // (pair mode: a second set of descriptors for the up matrix, column tile 1)
+  constexpr int ND = PAIR ? 2 : 1;
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x);
+  __amdgpu_buffer_rsrc_t rw[ND], rs[ND], rb[ND];
+  rw[0] = make_rsrc(wbase);
+  rs[0] = make_rsrc(sbase);
+  rb[0] = make_rsrc(bbase);
+  if (PAIR) {
+    rw[ND - 1] = make_rsrc(p.w2 + (size_t)n0 * wpr);
+    rs[ND - 1] = make_rsrc(p.s2 + (size_t)n0 * G);
+    rb[ND - 1] = make_rsrc(p.b2 + (size_t)n0 * G);
+  }
   // activation rows of this thread: rows past the end re-read the last valid row (their
   // products are never written)
   uint32_t xoff[XR];
@@ -222,10 +241,10 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 #pragma unroll
       for (int i = 0; i < BITS / 4; ++i)
         st.w[j].q[i] = __builtin_bit_cast(
-            uint4, __builtin_amdgcn_raw_buffer_load_b128(rw, woff[j] + i * 16, k0 * BITS / 8, 0));
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(rw[PAIR ? j : 0], woff[j] + i * 16, k0 * BITS / 8, 0));
       if (!SB4) {
-        st.w[j].s = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, soff[j], (k0 >> 6) * 2, 0);
-        st.w[j].b = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rb, soff[j], (k0 >> 6) * 2, 0);
+        st.w[j].s = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs[PAIR ? j : 0], soff[j], (k0 >> 6) * 2, 0);
+        st.w[j].b = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rb[PAIR ? j : 0], soff[j], (k0 >> 6) * 2, 0);
       }
     }
   };
@@ -236,8 +255,8 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   auto load_sb = [&](SBlock& sb, int blk) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      sb.s[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs, soff[j], blk * 8, 0));
-      sb.b[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rb, soff[j], blk * 8, 0));
+      sb.s[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs[PAIR ? j : 0], soff[j], blk * 8, 0));
+      sb.b[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rb[PAIR ? j : 0], soff[j], blk * 8, 0));
     }
   };
   auto pick = [&](const uint2& v, int e) {  // element e (uniform) of four bf16
@@ -355,7 +374,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     buf ^= 1;
   }
 
-  if (!GROUPED && p.ksplit > 1) {
+  if (!GROUPED && !PAIR && p.ksplit > 1) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel)
     float* mine = p.part + (size_t)blockIdx.z * part_stride(p.M, p.N);
@@ -381,6 +400,40 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   __syncthreads();  // every wave has finished reading the last activation tile
   constexpr int TS = 64 + 8;  // row stride of the staging tile (bf16)
   bf16_t* stage = &xs[0][0] + (size_t)wave * (32 * MI) * TS;
+  if (PAIR) {
+    // SwiGLU of the bf16-rounded projections (the rounding points of two GEMMs followed by
+    // the elementwise kernel), then rows of 32 columns out
+    bf16_t* sp = stage + (kq * 4) * TS + frow;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float g = bf2f(f2bf(acc[i][0][r])), u = bf2f(f2bf(acc[i][1][r]));
+        sp[(i * 32 + (r >> 2) * 8 + (r & 3)) * TS] = f2bf(g / (1.f + __expf(-g)) * u);
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    const bool vec_ok = (p.N & 7) == 0;
+    const int c8 = (lane & 3) * 8;
+    for (int it = 0; it < 2 * MI; ++it) {
+      const int row = it * 16 + (lane >> 2);
+      const int m = m0 + wm + row, n = n0 + wn + c8;
+      if (m >= m_end || n >= p.N) continue;
+      const size_t o = (size_t)m * p.N + n;
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + row * TS + c8);
+      if (vec_ok) {
+        *reinterpret_cast<uint4*>(p.y + o) = v;
+      } else {
+        const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          if (n + c >= p.N) break;
+          p.y[o + c] = f2bf((c & 1) ? bf_hi(w4[c >> 1]) : bf_lo(w4[c >> 1]));
+        }
+      }
+    }
+    return;
+  }
   {
     bf16_t* sp = stage + (kq * 4) * TS + frow;
 #pragma unroll
@@ -631,6 +684,58 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   else
     launch_grouped<8>(p, grid, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_gather_qmm");
+  return EXO_OK;
+}
+
+template <int BITS>
+void launch_pair(const QmmParams& p, hipStream_t st) {
+  const dim3 g2(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 128)), g4(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 256));
+  const bool sb4 = p.K % 256 == 0 &&
+                   (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
+  const bool small_grid = (int64_t)g4.x * g4.y < 128;
+  if (p.M <= 128 || small_grid) {
+    if (sb4)
+      qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 2, false, false, true><<<g2, 256, 0, st>>>(p);
+  } else {
+    if (sb4)
+      qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 4, false, false, true><<<g4, 256, 0, st>>>(p);
+  }
+}
+
+extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
+                              const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
+                              const uint16_t* b_up, uint16_t* y, int M, int N, int K, int bits,
+                              int group_size, exo_stream_t stream) {
+  EXO_REQUIRE(bits == 4 || bits == 8, "exo_qmm_swiglu: bits must be 4 or 8, got %d", bits);
+  EXO_REQUIRE(group_size == 64, "exo_qmm_swiglu: group_size must be 64, got %d", group_size);
+  EXO_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 64 == 0, "exo_qmm_swiglu: bad shape M=%d N=%d K=%d",
+              M, N, K);
+  EXO_REQUIRE(x && w_gate && s_gate && b_gate && w_up && s_up && b_up && y,
+              "exo_qmm_swiglu: null pointer");
+  if (M == 0) return EXO_OK;
+  EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm_swiglu: M=%d too large", M);
+  EXO_REQUIRE((int64_t)M * K < (1ll << 31),
+              "exo_qmm_swiglu: M*K=%lld exceeds 32-bit byte offsets", (long long)M * K);
+  QmmParams p{x, w_gate, s_gate, b_gate, nullptr, y, M, N, K};
+  p.sorted = nullptr;
+  p.tiles = nullptr;
+  p.x_div = 1;
+  p.w_stride = p.s_stride = 0;
+  p.ksplit = 1;
+  p.kc = K;
+  p.part = nullptr;
+  p.w2 = w_up;
+  p.s2 = s_up;
+  p.b2 = b_up;
+  if (bits == 4)
+    launch_pair<4>(p, (hipStream_t)stream);
+  else
+    launch_pair<8>(p, (hipStream_t)stream);
+  EXO_CHECK_LAUNCH("exo_qmm_swiglu");
   return EXO_OK;
 }
 

@@ -195,7 +195,9 @@ class ShardModel:
             if gemv:  # post-attention norm and SwiGLU fused into the gate/up GEMV pair
                 ops.qmv_swiglu(bf.h, L.gate, L.up, out=bf.act, norm_weight=L.post_norm,
                                eps=c.rms_norm_eps)
-            else:
+            elif R > 128:  # one GEMM launch for both projections, SwiGLU in its epilogue
+                ops.qmm_swiglu(bf.n, L.gate, L.up, out=bf.act)
+            else:  # short chunks: the split-K GEMM per projection is faster
                 if bf.gate is None:
                     bf.gate = torch.empty_like(bf.act)
                     bf.up = torch.empty_like(bf.act)

@@ -233,6 +233,25 @@ def quantized_matmul(
     return out
 
 
+def qmm_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) on the matrix cores, one launch (any M)."""
+    lib = native.load()
+    M, K = x.shape
+    if K != gate.K or gate.K != up.K or gate.N != up.N or gate.bits != up.bits:
+        raise ValueError("qmm_swiglu: gate and up must have the same shape and bits as x's K")
+    if out is None:
+        out = torch.empty(M, gate.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_qmm_swiglu(
+            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+            _ptr(up.scales), _ptr(up.biases), _ptr(out), M, gate.N, K, gate.bits,
+            gate.group_size, _stream(),
+        ),
+        "qmm_swiglu",
+    )
+    return out
+
+
 def qmm(x, qw: QuantizedWeight, residual=None, out=None) -> torch.Tensor:
     """Force the matrix-core path (any M)."""
     lib = native.load()

@@ -118,6 +118,16 @@ int exo_qmm_ws(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
                int64_t workspace_bytes, int M, int N, int K, int bits, int group_size,
                exo_stream_t stream);
 
+/* K2 + K8 for a (gate, up) pair, any M (the prefill form of exo_qmv_swiglu): y[M,N] =
+ * silu(x @ dq(w_gate)^T) * (x @ dq(w_up)^T), both projections rounded to bf16 before the
+ * SwiGLU - the bits of two exo_qmm calls followed by exo_swiglu, without writing either
+ * projection.  Both matrices [N,K].  (mlx_lm llama MLP `down(silu(gate(x)) * up(x))`;
+ * `swiglu` .typings/mlx_lm/models/switch_layers.pyi:52-57) */
+int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
+                   const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
+                   const uint16_t* b_up, uint16_t* y, int M, int N, int K, int bits,
+                   int group_size, exo_stream_t stream);
+
 /* K3 for prefill-sized T: the same operator as exo_gather_qmv on the matrix cores.  The
  * (token, slot) pairs are first sorted by expert (exo_moe_group, once per routing
  * decision; its workspace of exo_moe_group_workspace(T, topk, E) bytes then serves every

@@ -11,7 +11,7 @@ import torch
 from oracle import affine
 from oracle import ops as O
 from tests.util import (
-    assert_close, n_bits, n_f32, rand_bf16, rand_quantized, rng, t_bf16, t_qw, t_u32,
+    assert_close, assert_close_stat, n_bits, n_f32, rand_bf16, rand_quantized, rng, t_bf16, t_qw, t_u32,
 )
 
 pytestmark = pytest.mark.gpu
@@ -144,6 +144,27 @@ def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
     # the shared workspace is left clean for a launch of another shape
     y = ops.quantized_matmul(x[:2], g)
     assert torch.equal(y.view(torch.int16), ops.quantized_matmul(x[:2], g).view(torch.int16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(300, 256, 512), (129, 100, 192), (513, 192, 1024), (40, 64, 256), (2046, 1000, 320)])
+def test_qmm_swiglu_pair(device, bits, M, N, K):
+    """Gate and up projections with the SwiGLU in the GEMM's epilogue: the bits of the two
+    GEMMs followed by the elementwise kernel (same products, same rounding points), and the
+    oracle within tolerance.  Ragged M and N, N not a multiple of 8, K with and without the
+    four-step scale blocks."""
+    g = rand_quantized(N, K, bits, seed=N + 11)
+    u = rand_quantized(N, K, bits, seed=N + 12)
+    x = rand_bf16((M, K), seed=M + K)
+    gq, uq, xt = t_qw(g, bits, device), t_qw(u, bits, device), t_bf16(x, device)
+    got = ops.qmm_swiglu(xt, gq, uq)
+    sep = ops.swiglu(ops.qmm(xt, gq), ops.qmm(xt, uq))
+    assert torch.equal(got.view(torch.int16), sep.view(torch.int16))
+    # two roundings in a row (projection, then SwiGLU): a flipped bf16 rounding of a
+    # projection near zero can leave a handful of the elements outside the elementwise
+    # bound, so a fraction of 1e-5 is allowed
+    want = O.swiglu(affine.qmm(x, *g, 64, bits), affine.qmm(x, *u, 64, bits))
+    assert_close_stat(n_f32(got), want, max_outlier_frac=1e-5, what="qmm_swiglu")
 
 
 @pytest.mark.parametrize("bits", [4, 8])
