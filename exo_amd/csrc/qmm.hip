@@ -202,9 +202,9 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   rs[0] = make_rsrc(sbase);
   rb[0] = make_rsrc(bbase);
   if (PAIR) {
-    rw[ND - 1] = make_rsrc(p.w2 + (size_t)n0 * wpr);
-    rs[ND - 1] = make_rsrc(p.s2 + (size_t)n0 * G);
-    rb[ND - 1] = make_rsrc(p.b2 + (size_t)n0 * G);
+    rw[ND - 1] = make_rsrc(p.w2 + w_off + (size_t)n0 * wpr);
+    rs[ND - 1] = make_rsrc(p.s2 + s_off + (size_t)n0 * G);
+    rb[ND - 1] = make_rsrc(p.b2 + s_off + (size_t)n0 * G);
   }
   // activation rows of this thread: rows past the end re-read the last valid row (their
   // products are never written)
@@ -419,7 +419,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
       const int row = it * 16 + (lane >> 2);
       const int m = m0 + wm + row, n = n0 + wn + c8;
       if (m >= m_end || n >= p.N) continue;
-      const size_t o = (size_t)m * p.N + n;
+      const size_t o = (size_t)(GROUPED ? row_pair[m] : m) * p.N + n;
       const uint4 v = *reinterpret_cast<const uint4*>(stage + row * TS + c8);
       if (vec_ok) {
         *reinterpret_cast<uint4*>(p.y + o) = v;
@@ -569,10 +569,18 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
 
 template <int BITS>
 void launch_grouped(const QmmParams& p, dim3 grid, hipStream_t st) {
-  if (p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0)
+  const bool sb4 = p.K % 256 == 0 &&
+                   (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
+  if (p.w2) {  // (gate, up) pair with the SwiGLU in the epilogue
+    if (sb4)
+      qmm_kernel<BITS, 2, true, true, true><<<grid, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 2, true, false, true><<<grid, 256, 0, st>>>(p);
+  } else if (sb4) {
     qmm_kernel<BITS, 2, true, true><<<grid, 256, 0, st>>>(p);
-  else
+  } else {
     qmm_kernel<BITS, 2, true, false><<<grid, 256, 0, st>>>(p);
+  }
 }
 
 constexpr int kGroupBM = 128;  // rows per tile of the grouped GEMM
@@ -651,10 +659,11 @@ extern "C" int exo_moe_group(const int32_t* idx, int T, int topk, int E, void* w
   return EXO_OK;
 }
 
-extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
-                              const uint16_t* biases, const void* workspace, uint16_t* y, int T,
-                              int topk, int x_rows, int E, int N, int K, int bits,
-                              int group_size, exo_stream_t stream) {
+static int gather_qmm_impl(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, const uint32_t* w2, const uint16_t* s2,
+                           const uint16_t* b2, const void* workspace, uint16_t* y, int T, int topk,
+                           int x_rows, int E, int N, int K, int bits, int group_size,
+                           exo_stream_t stream) {
   EXO_REQUIRE(bits == 4 || bits == 8, "exo_gather_qmm: bits must be 4 or 8, got %d", bits);
   EXO_REQUIRE(group_size == 64, "exo_gather_qmm: group_size must be 64, got %d", group_size);
   EXO_REQUIRE(N > 0 && K > 0 && K % 64 == 0, "exo_gather_qmm: bad shape N=%d K=%d", N, K);
@@ -678,13 +687,35 @@ extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16
   p.ksplit = 1;
   p.kc = K;
   p.part = nullptr;
-  const dim3 grid(exo_ceil_div(N, 128), max_tiles);
+  p.w2 = w2;
+  p.s2 = s2;
+  p.b2 = b2;
+  const dim3 grid(exo_ceil_div(N, w2 ? 64 : 128), max_tiles);
   if (bits == 4)
     launch_grouped<4>(p, grid, (hipStream_t)stream);
   else
     launch_grouped<8>(p, grid, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_gather_qmm");
   return EXO_OK;
+}
+
+extern "C" int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const void* workspace, uint16_t* y, int T,
+                              int topk, int x_rows, int E, int N, int K, int bits,
+                              int group_size, exo_stream_t stream) {
+  return gather_qmm_impl(x, w, scales, biases, nullptr, nullptr, nullptr, workspace, y, T, topk,
+                         x_rows, E, N, K, bits, group_size, stream);
+}
+
+extern "C" int exo_gather_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate,
+                                     const uint16_t* s_gate, const uint16_t* b_gate,
+                                     const uint32_t* w_up, const uint16_t* s_up,
+                                     const uint16_t* b_up, const void* workspace, uint16_t* y,
+                                     int T, int topk, int x_rows, int E, int N, int K, int bits,
+                                     int group_size, exo_stream_t stream) {
+  EXO_REQUIRE(w_up && s_up && b_up, "exo_gather_qmm_swiglu: null pointer");
+  return gather_qmm_impl(x, w_gate, s_gate, b_gate, w_up, s_up, b_up, workspace, y, T, topk,
+                         x_rows, E, N, K, bits, group_size, stream);
 }
 
 template <int BITS>

@@ -213,15 +213,9 @@ class ShardModel:
             ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
         idx, sc = ops.router_topk(bf.router_logits, c.num_experts_per_tok, c.norm_topk_prob)
         k = c.num_experts_per_tok
-        if not gemv:  # prefill: rows sorted by expert, one MFMA GEMM per projection
-            if bf.gate is None:
-                bf.gate = torch.empty_like(bf.act)
-                bf.up = torch.empty_like(bf.act)
+        if not gemv:  # prefill: rows sorted by expert; gate, up and SwiGLU in one grouped GEMM
             ws = ops.moe_group(idx, c.num_experts)
-            x3 = bf.n.view(R, 1, -1)
-            ops.grouped_qmm(x3, L.gate, ws, k, out=bf.gate)
-            ops.grouped_qmm(x3, L.up, ws, k, out=bf.up)
-            ops.swiglu(bf.gate, bf.up, out=bf.act)
+            ops.grouped_qmm_swiglu(bf.n.view(R, 1, -1), L.gate, L.up, ws, k, out=bf.act)
             ops.grouped_qmm(bf.act, L.down, ws, k, out=bf.expert_out)
             ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
             return

@@ -34,6 +34,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_moe_group_workspace": (_i64, [_i, _i, _i]),
     "exo_moe_group": (_i, [_vp, _i, _i, _i, _vp, _i64, _vp]),
     "exo_gather_qmm": (_i, [_vp] * 6 + [_i] * 8 + [_vp]),
+    "exo_gather_qmm_swiglu": (_i, [_vp] * 9 + [_i] * 8 + [_vp]),
     "exo_qmm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "exo_qmm_workspace": (_i64, [_i, _i]),
     "exo_qmm_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),

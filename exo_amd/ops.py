@@ -371,6 +371,28 @@ def grouped_qmm(x: torch.Tensor, qw: QuantizedWeight, group_ws: torch.Tensor, to
     return out
 
 
+def grouped_qmm_swiglu(x: torch.Tensor, gate: QuantizedWeight, up: QuantizedWeight,
+                       group_ws: torch.Tensor, topk: int, out=None):
+    """SwitchGLU's gate/up + swiglu for prefill-sized inputs, one launch: x bf16 [T, R, K]
+    (R == 1 or topk), routing prepared by moe_group -> bf16 [T, topk, N]."""
+    lib = native.load()
+    T, R, K = x.shape
+    E = gate.weight.shape[0]
+    if K != gate.K or gate.K != up.K or gate.N != up.N or gate.bits != up.bits:
+        raise ValueError("grouped_qmm_swiglu: gate and up must have the same shape and bits as x's K")
+    if out is None:
+        out = torch.empty(T, topk, gate.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_gather_qmm_swiglu(
+            _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+            _ptr(up.scales), _ptr(up.biases), _ptr(group_ws), _ptr(out), T, topk, R, E, gate.N, K,
+            gate.bits, gate.group_size, _stream(),
+        ),
+        "grouped_qmm_swiglu",
+    )
+    return out
+
+
 def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None,
                       norm_weight=None, eps: float = 0.0):
     """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N];

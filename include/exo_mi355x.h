@@ -142,6 +142,16 @@ int exo_gather_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
                    const uint16_t* biases, const void* workspace, uint16_t* y, int T, int topk,
                    int x_rows, int E, int N, int K, int bits, int group_size,
                    exo_stream_t stream);
+/* SwitchGLU's gate and up projections with their swiglu for prefill-sized T, one launch:
+ * y[t,j,:] = silu(x @ dq(w_gate[e])^T) * (x @ dq(w_up[e])^T), e = the expert of pair (t,j),
+ * both projections rounded to bf16 first - the bits of two exo_gather_qmm calls followed by
+ * exo_swiglu.  Same workspace and shapes as exo_gather_qmm; both matrices [E,N,K].
+ * (.typings/mlx_lm/models/switch_layers.pyi:52-73) */
+int exo_gather_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
+                          const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
+                          const uint16_t* b_up, const void* workspace, uint16_t* y, int T,
+                          int topk, int x_rows, int E, int N, int K, int bits, int group_size,
+                          exo_stream_t stream);
 
 /* K3: mx.gather_qmm(x, w, scales, biases, rhs_indices=idx, transpose=True) as
  * QuantizedSwitchLinear calls it: w uint32 [E,N,K*bits/32]; idx int32 [T,topk];

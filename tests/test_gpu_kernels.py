@@ -251,6 +251,25 @@ def test_grouped_qmm(device, bits, x_rows, E, N, K, T, topk):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("E,N,K,T,topk", [(6, 96, 768, 40, 4), (128, 200, 256, 300, 8), (3, 60, 64, 1, 2)])
+def test_grouped_qmm_swiglu(device, bits, E, N, K, T, topk):
+    """SwitchGLU's gate and up projections with the SwiGLU in the grouped GEMM's epilogue:
+    the bits of the two grouped GEMMs followed by the elementwise kernel (ragged tiles,
+    N not a multiple of 64 or 8, K with and without the four-step scale blocks)."""
+    g = rand_quantized(N, K, bits, seed=60 + E, E=E)
+    u = rand_quantized(N, K, bits, seed=61 + E, E=E)
+    idx = rng(62 + T).integers(0, E, size=(T, topk)).astype(np.int32)
+    if E == 128:
+        idx[: T // 2, 0] = 5
+    x = t_bf16(rand_bf16((T, 1, K), seed=63), device)
+    gq, uq = t_qw(g, bits, device), t_qw(u, bits, device)
+    ws = ops.moe_group(torch.from_numpy(idx).to(device), E)
+    got = ops.grouped_qmm_swiglu(x, gq, uq, ws, topk)
+    sep = ops.swiglu(ops.grouped_qmm(x, gq, ws, topk), ops.grouped_qmm(x, uq, ws, topk))
+    assert torch.equal(got.view(torch.int16), sep.view(torch.int16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 def test_gather_qmv_swiglu(device, bits):
     E, N, K, T, topk = 5, 64, 2048, 2, 3
     g = rand_quantized(N, K, bits, seed=50, E=E)
