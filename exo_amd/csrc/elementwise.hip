@@ -77,56 +77,59 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
 }
 
 // ------------------------------------------------------ RoPE + KV append (+ head norm)
-// One wave per (token, head); lane i < D/2 owns the pair (i, i + D/2).
-__global__ __launch_bounds__(64) void rope_kv_kernel(
+// One workgroup per token; its four waves take the heads in turn, lane i < D/2 owns the
+// pair (i, i + D/2) of every head - so the angle's sine and cosine (a precise sincosf: the
+// angle reaches thousands of radians) are computed once per token and lane, not per head.
+__global__ __launch_bounds__(256) void rope_kv_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kc,
     bf16_t* __restrict__ vc, const int32_t* __restrict__ pos, const float* __restrict__ inv_freq,
     const bf16_t* __restrict__ qn, const bf16_t* __restrict__ kn, float eps, int T, int Hq,
     int Hkv, int D, int S_max) {
   const int tok = blockIdx.x;  // b*T + t
-  const int head = blockIdx.y; // [0,Hq) q, [Hq,Hq+Hkv) k, then v
   const int b = tok / T, t = tok - b * T;
-  const int i = threadIdx.x, half = D >> 1;
+  const int i = threadIdx.x & 63, wave = threadIdx.x >> 6, half = D >> 1;
   const bool active = i < half;
   const int p = pos[b] + t;
-  const bf16_t* src = qkv + (size_t)tok * (Hq + 2 * Hkv) * D + (size_t)head * D;
-  float x1 = 0.f, x2 = 0.f;
-  if (active) {
-    x1 = bf2f(src[i]);
-    x2 = bf2f(src[i + half]);
-  }
-  if (head >= Hq + Hkv) {  // v: copy into the cache
-    if (active && p < S_max) {
-      bf16_t* dst = vc + (((size_t)b * Hkv + (head - Hq - Hkv)) * S_max + p) * D;
-      dst[i] = src[i];
-      dst[i + half] = src[i + half];
+  float sn = 0.f, cs = 1.f;
+  if (active) sincosf((float)p * inv_freq[i], &sn, &cs);
+  // heads [0,Hq) are q, [Hq,Hq+Hkv) k, then v
+  for (int head = wave; head < Hq + 2 * Hkv; head += 4) {
+    const bf16_t* src = qkv + (size_t)tok * (Hq + 2 * Hkv) * D + (size_t)head * D;
+    if (head >= Hq + Hkv) {  // v: copy into the cache
+      if (active && p < S_max) {
+        bf16_t* dst = vc + (((size_t)b * Hkv + (head - Hq - Hkv)) * S_max + p) * D;
+        dst[i] = src[i];
+        dst[i + half] = src[i + half];
+      }
+      continue;
     }
-    return;
-  }
-  const bool is_q = head < Hq;
-  const bf16_t* nw = is_q ? qn : kn;
-  if (nw) {  // per-head RMSNorm, rounded to bf16 like a separate rms_norm call
-    const float ss = wave_sum(x1 * x1 + x2 * x2);
-    const float inv = rsqrtf(ss / (float)D + eps);
+    float x1 = 0.f, x2 = 0.f;
     if (active) {
-      x1 = bf2f(f2bf(x1 * inv * bf2f(nw[i])));
-      x2 = bf2f(f2bf(x2 * inv * bf2f(nw[i + half])));
+      x1 = bf2f(src[i]);
+      x2 = bf2f(src[i + half]);
     }
-  }
-  if (!active) return;
-  const float ang = (float)p * inv_freq[i];
-  float sn, cs;
-  sincosf(ang, &sn, &cs);
-  const bf16_t o1 = f2bf(x1 * cs - x2 * sn);
-  const bf16_t o2 = f2bf(x2 * cs + x1 * sn);
-  if (is_q) {
-    bf16_t* dst = q_out + (size_t)tok * Hq * D + (size_t)head * D;
-    dst[i] = o1;
-    dst[i + half] = o2;
-  } else if (p < S_max) {
-    bf16_t* dst = kc + (((size_t)b * Hkv + (head - Hq)) * S_max + p) * D;
-    dst[i] = o1;
-    dst[i + half] = o2;
+    const bool is_q = head < Hq;
+    const bf16_t* nw = is_q ? qn : kn;
+    if (nw) {  // per-head RMSNorm, rounded to bf16 like a separate rms_norm call
+      const float ss = wave_sum(x1 * x1 + x2 * x2);
+      const float inv = rsqrtf(ss / (float)D + eps);
+      if (active) {
+        x1 = bf2f(f2bf(x1 * inv * bf2f(nw[i])));
+        x2 = bf2f(f2bf(x2 * inv * bf2f(nw[i + half])));
+      }
+    }
+    if (!active) continue;
+    const bf16_t o1 = f2bf(x1 * cs - x2 * sn);
+    const bf16_t o2 = f2bf(x2 * cs + x1 * sn);
+    if (is_q) {
+      bf16_t* dst = q_out + (size_t)tok * Hq * D + (size_t)head * D;
+      dst[i] = o1;
+      dst[i + half] = o2;
+    } else if (p < S_max) {
+      bf16_t* dst = kc + (((size_t)b * Hkv + (head - Hq)) * S_max + p) * D;
+      dst[i] = o1;
+      dst[i + half] = o2;
+    }
   }
 }
 
@@ -353,8 +356,7 @@ extern "C" int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t
   EXO_REQUIRE(B > 0 && T > 0 && Hq > 0 && Hkv > 0 && S_max > 0,
               "exo_rope_kv_append: non-positive size");
   EXO_REQUIRE(D == 64 || D == 128, "exo_rope_kv_append: head_dim %d not supported (64, 128)", D);
-  EXO_REQUIRE(Hq + 2 * Hkv <= 65535, "exo_rope_kv_append: too many heads");
-  rope_kv_kernel<<<dim3(B * T, Hq + 2 * Hkv), 64, 0, (hipStream_t)stream>>>(
+  rope_kv_kernel<<<dim3(B * T), 256, 0, (hipStream_t)stream>>>(
       qkv, q_out, k_cache, v_cache, pos, inv_freq, q_norm_w, k_norm_w, eps, T, Hq, Hkv, D,
       S_max);
   EXO_CHECK_LAUNCH("exo_rope_kv_append");
