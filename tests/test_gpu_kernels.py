@@ -437,8 +437,10 @@ def test_gather_qmv_combine(device, bits, E, N, K, T, topk):
     assert_close(n_f32(no_res), acc, what="gather_qmv_combine without residual")
 
 
-def test_moe_combine(device):
-    T, topk, H = 3, 8, 2048
+@pytest.mark.parametrize("T,topk,H", [(3, 8, 2048), (5, 6, 4096), (2, 3, 100), (4, 9, 264)])
+def test_moe_combine(device, T, topk, H):
+    """Rows of 8-element multiples take the 16-byte kernel (slots in groups of four, the
+    last group partial), the others the scalar one."""
     y = rand_bf16((T, topk, H), seed=1)
     s = affine.bf16_round(np.abs(rand_bf16((T, topk), seed=2)) / 8)
     r = rand_bf16((T, H), seed=3)
