@@ -523,13 +523,18 @@ __global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict
   }
 }
 
-// K split of a launch: only for up to 128 rows (one row tile) when the column tiles alone
-// cover less than the chip; chunks of whole blocks of four K steps, at least two blocks
+// launches of fewer than this many 128 x 128 output tiles may split K
+constexpr int kQmmSplitTiles = 128;
+
+// K split of a launch: when its 128 x 128 output tiles cover less than half the chip (a
+// short input, or a narrow matrix such as a MoE router under a long prompt); chunks of whole
+// blocks of four K steps, at least two blocks
 void plan_split(int M, int N, int K, bool have_ws, int* ksplit, int* kc) {
   *ksplit = 1;
   *kc = K;
-  if (!have_ws || M > 128 || K % 256 != 0) return;
-  const int tiles = exo_ceil_div(N, 128);
+  if (!have_ws || K % 256 != 0) return;
+  const int tiles = exo_ceil_div(N, 128) * exo_ceil_div(M, 128);
+  if (tiles >= kQmmSplitTiles) return;
   int ks = 1;
   while (ks < kQmmMaxSplit && tiles * ks < 256 && K / (ks * 2) >= 512) ks *= 2;
   if (ks == 1) return;
@@ -771,7 +776,8 @@ extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const u
 }
 
 extern "C" int64_t exo_qmm_workspace(int M, int N) {
-  if (M <= 0 || N <= 0 || M > 128) return 0;
+  if (M <= 0 || N <= 0) return 0;
+  if ((int64_t)exo_ceil_div(N, 128) * exo_ceil_div(M, 128) >= kQmmSplitTiles) return 0;
   return (int64_t)kQmmMaxSplit * (int64_t)part_stride(M, N) * 4;
 }
 

@@ -152,8 +152,8 @@ _QMM_WS: dict[int, list[torch.Tensor]] = {}
 
 
 def qmm_workspace(M: int, N: int, device) -> torch.Tensor | None:
-    """Split-K workspace of the GEMM for inputs of up to 128 rows (None above), one per
-    device, grown on demand; a replaced buffer stays alive (a captured graph may still
+    """Split-K workspace of the GEMM for launches of few output tiles (None for the others),
+    one per device, grown on demand; a replaced buffer stays alive (a captured graph may still
     point at it)."""
     need = native.load().exo_qmm_workspace(M, N)
     if need == 0:

@@ -106,10 +106,11 @@ int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_weight, float
 int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
             const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
             int K, int bits, int group_size, exo_stream_t stream);
-/* exo_qmm with a workspace for short inputs (M <= 128, e.g. a short prompt): one row
- * tile has too few column tiles to fill the chip, so K is split over up to 8 workgroups
- * per tile, the float32 partial tiles go to `workspace` and a second small launch adds
- * them in a fixed order.  exo_qmm_workspace(M, N) bytes (0: this M never splits),
+/* exo_qmm with a workspace for launches of few output tiles (fewer than 128 tiles of
+ * 128 x 128: a short prompt, or a narrow matrix such as a MoE router under a long one): the
+ * tiles alone do not fill the chip, so K is split over up to 8 workgroups per tile, the
+ * float32 partial tiles go to `workspace` and a second small launch adds them in a fixed
+ * order.  exo_qmm_workspace(M, N) bytes (0: this shape never splits),
  * 256-byte aligned, no initialisation needed.  Launches that share a workspace must be
  * ordered on one stream.  workspace == NULL behaves like exo_qmm. */
 int64_t exo_qmm_workspace(int M, int N);

@@ -179,10 +179,11 @@ def test_qmm_mfma(device, bits, M, N, K):
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024),
-                                   (12, 256, 8192), (9, 96, 1024)])
+                                   (12, 256, 8192), (9, 96, 1024), (1023, 128, 2048), (300, 200, 4096)])
 def test_qmm_split_k(device, bits, M, N, K):
-    """Up to 128 rows and few column tiles: K is split over workgroups and the float32
-    partial tiles are merged by the last arrival.  Against the oracle, against the
+    """Few output tiles (a short input, or a narrow matrix under a long one): K is split
+    over workgroups and the float32 partial tiles are added by a second launch.  Against
+    the oracle, against the
     unsplit kernel (same products, another summation order: a few bf16 ulps at most),
     with the residual, and twice in a row (the counters return to zero)."""
     trip = rand_quantized(N, K, bits, seed=M + N)
