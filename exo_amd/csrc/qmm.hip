@@ -550,9 +550,10 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
   // taller inputs: 256-row tiles halve the dequantisation work and the LDS reads per output
   const dim3 g2(exo_ceil_div(N, 128), exo_ceil_div(M, 128), p.ksplit), g4(exo_ceil_div(N, 128), exo_ceil_div(M, 256));
   const bool sb4 = p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0;
-  // a grid of fewer than 128 of the tall tiles leaves most CUs idle: twice as many
-  // 128-row tiles are faster there (1024x4096 at 2046 rows: 89 -> 70 us), not beyond
-  const bool small_grid = (int64_t)g4.x * g4.y < 128;
+  // a grid of up to 128 of the tall tiles leaves at least half of the CUs idle: twice as
+  // many 128-row tiles are faster there (1024x4096 at 2046 rows: 89 -> 70 us; 4096x4096 at
+  // 1023 rows, exactly 128 tall tiles: 93 -> 77 us), not beyond (192 tall tiles: 88 vs 97 us)
+  const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (M <= 128 || small_grid) {
     if (sb4)
       qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
@@ -728,7 +729,7 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
   const dim3 g2(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 128)), g4(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 256));
   const bool sb4 = p.K % 256 == 0 &&
                    (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
-  const bool small_grid = (int64_t)g4.x * g4.y < 128;
+  const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (p.M <= 128 || small_grid) {
     if (sb4)
       qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
