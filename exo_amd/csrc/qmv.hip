@@ -911,7 +911,7 @@ int launch_ksplit(const QmvParams& p, hipStream_t st) {
 //   out[t,n] = bf16( bf16( sum_j bf16( bf16(W[e_j][n,:] . x[t,j,:]) * score[t,j] ) ) + res[t,n] )
 // - the same rounding points as exo_gather_qmv followed by exo_moe_combine.
 // blockIdx.y = token; a workgroup has one wave per expert slot.  Wave j stages ITS
-// activation row x[t,j,:], multiplies kDownRW sets of 64/LPR rows of expert e_j (all its
+// activation row x[t,j,:], multiplies kDownRW (1 or 2) sets of 64/LPR rows of expert e_j (all its
 // loads in flight from the start) and leaves bf16(bf16(dot) * score_j) in LDS; the first
 // wave adds the k contributions in slot order.  The launch is latency-bound, hence the
 // many short waves.
@@ -929,9 +929,8 @@ struct DownCombineParams {
 
 constexpr int kDownMaxIters = 4;  // 16-byte chunks per lane and expert row
 constexpr int kDownMaxTopk = 8;
-constexpr int kDownRW = 2;        // row sets per wave
 
-template <int BITS>
+template <int BITS, int kDownRW>
 __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
     const DownCombineParams p) {
   extern __shared__ uint4 smem[];
@@ -1031,14 +1030,16 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
   }
   __syncthreads();
 
-  if (slot == 0 && lane < kDownRW * rpwi) {
-    const int row = row0 + lane;  // lane = i * rpwi + sub
-    if (row < p.N) {
-      float total = 0.f;
-      for (int j = 0; j < p.topk; ++j) total += contrib[j][lane];
-      float o = bf2f(f2bf(total));
-      if (p.residual) o += bf2f(p.residual[(size_t)t * p.N + row]);
-      p.out[(size_t)t * p.N + row] = f2bf(o);
+  if (slot == 0) {
+    for (int r = lane; r < kDownRW * rpwi; r += 64) {  // r = i * rpwi + sub
+      const int row = row0 + r;
+      if (row < p.N) {
+        float total = 0.f;
+        for (int j = 0; j < p.topk; ++j) total += contrib[j][r];
+        float o = bf2f(f2bf(total));
+        if (p.residual) o += bf2f(p.residual[(size_t)t * p.N + row]);
+        p.out[(size_t)t * p.N + row] = f2bf(o);
+      }
     }
   }
 }
@@ -1457,12 +1458,24 @@ extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, cons
   p.lpr_log2 = pl.lpr_log2;
   p.iters = pl.iters;
   const int rpwi = 64 >> pl.lpr_log2;
-  const dim3 grid(exo_ceil_div(N, kDownRW * rpwi), T);
+  // two row sets per wave only while that leaves 512 workgroups per token: the launch is
+  // latency-bound and wants a wide grid (Qwen3-30B, 2048 outputs in sets of 8: one set,
+  // 256 workgroups, 482 -> 509 tok/s; Qwen3-235B, 4096 outputs in sets of 2: two sets, 1024
+  // workgroups - one set per wave loses 5 % there, four lose 6 %)
+  const int rw = exo_ceil_div(N, 2 * rpwi) >= 512 ? 2 : 1;
+  const dim3 grid(exo_ceil_div(N, rw * rpwi), T);
   const size_t lds = (size_t)topk * ((size_t)p.wpr * 16 + (size_t)(p.wpr / 4) * 8);
-  if (bits == 4)
-    moe_down_combine_kernel<4><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
-  else
-    moe_down_combine_kernel<8><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+  if (bits == 4) {
+    if (rw == 2)
+      moe_down_combine_kernel<4, 2><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+    else
+      moe_down_combine_kernel<4, 1><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+  } else {
+    if (rw == 2)
+      moe_down_combine_kernel<8, 2><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+    else
+      moe_down_combine_kernel<8, 1><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+  }
   EXO_CHECK_LAUNCH("exo_gather_qmv_combine");
   return EXO_OK;
 }
