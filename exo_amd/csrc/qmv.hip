@@ -1092,7 +1092,10 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   // at least one full batch of rows per wave
   int per_cu = pl.lds <= 36 * 1024 ? 4 : (pl.lds <= 72 * 1024 ? 2 : 1);
   int grid = 256 * per_cu;
-  const int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
+  // (gather mode, several (token, slot) pairs: half of that - the launch is latency-bound
+  // and twice as many workgroups finish sooner; a quarter was slower again)
+  int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
+  if (pairs > 1 && min_rows > 1) min_rows /= 2;
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
   if (grid < 1) grid = 1;
