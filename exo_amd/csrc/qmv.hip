@@ -1096,6 +1096,10 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   // and twice as many workgroups finish sooner; a quarter was slower again)
   int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
   if (pairs > 1 && min_rows > 1) min_rows /= 2;
+  // short matrices: fewer rows per wave while that grid would stay under 160 workgroups
+  // (2048x2048: 64 -> 256 workgroups, 4.0 -> 2.9 us; 2048x4096: 3.5 -> 3.2 us; 160 and more
+  // workgroups were faster as they are: 5120x2048, 4096x4096, 6144x4096)
+  while (min_rows > 1 && p.N / (min_rows * kWaves) < 160) min_rows /= 2;
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
   if (grid < 1) grid = 1;
