@@ -306,16 +306,41 @@ __global__ __launch_bounds__(256) void argmax_stage1(const bf16_t* __restrict__ 
   __shared__ float smax[4], ssum[4];
   __shared__ int sidx[4];
   const int row = blockIdx.y;
-  const int per = (V + kArgBlocks - 1) / kArgBlocks;
-  const int lo = blockIdx.x * per, hi = min(lo + per, V);
   const bf16_t* src = logits + (size_t)row * V;
+  // rows of 16-byte multiples (every vocabulary here): the block's share is whole 8-element
+  // chunks, up to two per thread, which stay in registers for the second pass
+  const bool vec = (V & 7) == 0 && (V >> 3) <= kArgBlocks * 512 && ((uintptr_t)logits & 15) == 0;
+  const int per = vec ? (((V >> 3) + kArgBlocks - 1) / kArgBlocks) << 3 : (V + kArgBlocks - 1) / kArgBlocks;
+  const int lo = min((int)blockIdx.x * per, V), hi = min(lo + per, V);
   float mx = -INFINITY;
   int mi = 0x7fffffff;
-  for (int i = lo + threadIdx.x; i < hi; i += 256) {
-    const float x = bf2f(src[i]);
-    if (x > mx) {
-      mx = x;
-      mi = i;
+  float xv[16];
+  if (vec) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int i0 = lo + (threadIdx.x + 256 * u) * 8;
+      uint4 v = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // -inf
+      if (i0 < hi) v = *reinterpret_cast<const uint4*>(src + i0);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        xv[8 * u + 2 * k] = bf_lo(w[k]);
+        xv[8 * u + 2 * k + 1] = bf_hi(w[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (xv[8 * u + k] > mx) {
+          mx = xv[8 * u + k];
+          mi = i0 + k;
+        }
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+      const float x = bf2f(src[i]);
+      if (x > mx) {
+        mx = x;
+        mi = i;
+      }
     }
   }
 #pragma unroll
@@ -342,8 +367,14 @@ __global__ __launch_bounds__(256) void argmax_stage1(const bf16_t* __restrict__ 
       bi = sidx[w];
     }
   float se = 0.f;
-  if (bm > -INFINITY)
-    for (int i = lo + threadIdx.x; i < hi; i += 256) se += expf(bf2f(src[i]) - bm);
+  if (bm > -INFINITY) {
+    if (vec) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) se += expf(xv[k] - bm);  // padding is -inf: exp = 0
+    } else {
+      for (int i = lo + threadIdx.x; i < hi; i += 256) se += expf(bf2f(src[i]) - bm);
+    }
+  }
   se = wave_sum(se);
   if (lane == 0) ssum[wave] = se;
   __syncthreads();
