@@ -403,6 +403,324 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   }
 }
 
+typedef short short4_t __attribute__((ext_vector_type(4)));
+// ds_read_b64_tr_b16: four consecutive rows of one column out of a row-major bf16 tile
+__device__ __forceinline__ uint2 lds_read_tr16(const bf16_t* p) {
+  const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4_t __attribute__((address_space(3)))*)p);
+  return __builtin_bit_cast(uint2, v);
+}
+
+// ---------------------------------------------------------------- matrix-core decode
+// Fused decode attention (RoPE, head norm, cache append, attention) for D = 128 with the
+// two products on v_mfma_f32_32x32x16_bf16.  The scalar kernel above spends ~10 vector
+// instructions per (query head, key) and lane group; with several sequences in the step
+// that - not the K/V bytes - bounds it.  Here one wave multiplies a tile
+// of 32 keys by ALL G query heads of the kv head at once (they are columns of the B operand,
+// the unused ones zero):
+//   S^T[key][head] = K . Q^T     A = K rows from the wave's LDS tile, B = Q^T from registers
+//   O^T[d][head]  += V^T . P^T   A = V^T: 8 keys of one d per lane, out of the row-major V
+//                                tile with two transposing LDS reads; B = the S^T registers
+// as in the prefill kernel (same permuted key order, same per-lane softmax state).
+// Work split: grid (splits, Hkv, B); a workgroup's four waves take a quarter of the split's
+// keys each, in tiles of 32 that go global -> registers -> the wave's own LDS region (no
+// block barrier in the loop).  The new token's key and value come from registers / LDS and
+// are added by wave 0 of the split that owns position len-1.  The partial results leave in
+// the layout of the scalar kernel, so the merge of waves and splits is the same code.
+template <int G>
+__global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const SdpaParams p) {
+  constexpr int D = 128;
+  constexpr int TK = 32;          // keys per tile
+  constexpr int KS = D + 8;       // LDS row stride (bf16)
+  constexpr int STEPS = D / 16, DT = D / 32;
+  constexpr int VS = D + 16;      // V rows: 32 bytes past a multiple of the 256-byte bank span
+  constexpr int TILE = TK * KS;   // bf16 elements of a K tile
+  constexpr int WAVE_TILES = TK * KS + TK * VS;  // K tile + V tile of one wave
+  constexpr int TILE_BYTES = kWaves * WAVE_TILES * 2;
+  constexpr int RED_BYTES = kWaves * G * (D + 2) * 4;
+  constexpr int SMEM = TILE_BYTES > RED_BYTES ? TILE_BYTES : RED_BYTES;
+  __shared__ __attribute__((aligned(16))) char smem[SMEM];
+  __shared__ __attribute__((aligned(16))) bf16_t q_lds[G * D];
+  __shared__ __attribute__((aligned(16))) bf16_t kv_new[2 * D];
+  __shared__ int s_last;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, kq = lane >> 5;
+  const int b = blockIdx.z, kvh = blockIdx.y;
+  const int h0 = kvh * G;
+  const int len = min(p.pos[b] + 1, p.S_max);
+  // the cache holds keys [0, len-1); key len-1 comes from the qkv row
+  int chunk = (len + p.splits - 1) / p.splits;
+  chunk = (chunk + TK * kWaves - 1) / (TK * kWaves) * (TK * kWaves);
+  const bool own_new = (len - 1) / chunk == (int)blockIdx.x;
+  const int k_begin = min(min((int)blockIdx.x * chunk, len), len - 1);
+  const int k_end = min(min((int)blockIdx.x * chunk + chunk, len), len - 1);
+  const int per_wave = ((k_end - k_begin + kWaves - 1) / kWaves + TK - 1) / TK * TK;
+  const int w_begin = min(k_begin + wave * per_wave, k_end);
+  const int w_end = min(w_begin + per_wave, k_end);
+
+  const size_t head_base = ((size_t)b * p.Hkv + kvh) * p.S_max * D;
+  const bf16_t* kb = p.kc + head_base;
+  const bf16_t* vb = p.vc + head_base;
+  // tile loads: 16-byte chunk vi = lane + 64*i of the tile is (key vi/16, chunk vi%16)
+  // (always executed, with clamped keys, so that the tile registers are plain values: a
+  // conditional refill made the compiler keep them in scratch memory and wait for every
+  // load right after issuing it)
+  // (eight named registers each, not arrays: those stayed in scratch memory here)
+  uint4 k0r, k1r, k2r, k3r, k4r, k5r, k6r, k7r, v0r, v1r, v2r, v3r, v4r, v5r, v6r, v7r;
+#define EXO_LOAD1(I, K0)                                                                \
+  {                                                                                     \
+    const int vi = lane + 64 * I;                                                       \
+    const int key = max(min((K0) + (vi >> 4), w_end - 1), 0); /* past the range: masked */ \
+    k##I##r = *reinterpret_cast<const uint4*>(kb + (size_t)key * D + (vi & 15) * 8);    \
+    v##I##r = *reinterpret_cast<const uint4*>(vb + (size_t)key * D + (vi & 15) * 8);    \
+  }
+#define EXO_LOAD_TILE(K0) \
+  EXO_LOAD1(0, K0) EXO_LOAD1(1, K0) EXO_LOAD1(2, K0) EXO_LOAD1(3, K0) EXO_LOAD1(4, K0) EXO_LOAD1(5, K0) EXO_LOAD1(6, K0) EXO_LOAD1(7, K0)
+#define EXO_STORE1(I)                                                                  \
+  {                                                                                    \
+    const int vi = lane + 64 * I;                                                      \
+    *reinterpret_cast<uint4*>(&k_t[(vi >> 4) * KS + (vi & 15) * 8]) = k##I##r;         \
+    *reinterpret_cast<uint4*>(&v_t[(vi >> 4) * VS + (vi & 15) * 8]) = v##I##r;         \
+  }
+  EXO_LOAD_TILE(w_begin)  // in flight during the q work
+
+  // ---- q of the G heads (RoPE, optional head norm) -> LDS; the new token's k and v
+  {
+    const int sub = lane >> 4, sl = lane & 15;
+    float cs[8], sn[8];
+    if (p.rope_tab) {
+      const float4* tp = reinterpret_cast<const float4*>(
+          p.rope_tab + (size_t)(len - 1) * (D / 2) + (sl * 8) % (D / 2));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float4 v = tp[e];
+        cs[2 * e] = v.x;
+        sn[2 * e] = v.y;
+        cs[2 * e + 1] = v.z;
+        sn[2 * e + 1] = v.w;
+      }
+    } else {
+      const float fpos = (float)(len - 1);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sincosf(fpos * p.inv_freq[(sl * 8 + e) % (D / 2)], &sn[e], &cs[e]);
+    }
+    const bf16_t* row = p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
+    for (int g = wave * 4 + sub; g < G; g += 4 * kWaves)  // a 16-lane group per head
+      *reinterpret_cast<uint4*>(&q_lds[g * D + sl * 8]) =
+          head_slice<D, true>(row + (size_t)(h0 + g) * D, sl, p.qn, p.eps, cs, sn);
+    if (own_new && wave == kWaves - 1 && sub < 2) {
+      const uint4 t = sub == 0 ? head_slice<D, true>(row + (size_t)(p.Hq + kvh) * D, sl, p.kn, p.eps, cs, sn)
+                               : head_slice<D, false>(row + (size_t)(p.Hq + p.Hkv + kvh) * D, sl, nullptr, 0.f, cs, sn);
+      *reinterpret_cast<uint4*>(&kv_new[sub * D + sl * 8]) = t;
+      // appended to the cache for the following steps
+      bf16_t* dst = const_cast<bf16_t*>(sub == 0 ? p.kc : p.vc) + head_base + (size_t)(len - 1) * D + sl * 8;
+      *reinterpret_cast<uint4*>(dst) = t;
+    }
+  }
+  __syncthreads();
+
+  // Q^T operand: lane (head n, half kq) takes d = 16*st + 8*kq .. +8 of its head for step
+  // st - re-read from LDS for every tile (32 registers fewer to carry through the loop;
+  // lanes beyond the G heads read head 0 and their columns are never stored)
+  const bf16_t* qrow_lds = &q_lds[(n < G ? n : 0) * D + kq * 8];
+
+  bf16_t* k_t = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * WAVE_TILES;
+  bf16_t* v_t = k_t + TILE;
+  // A-operand row r of the 32-key tile holds this key, so that D registers 8s..8s+7 of
+  // lane half kq are keys 16s + 8kq .. +8
+  const int jr = n >> 3;
+  const int key_of_row = 16 * (jr >> 1) + 8 * ((n >> 2) & 1) + 4 * (jr & 1) + (n & 3);
+  const float scale_log2e = p.scale * 1.4426950408889634f;
+
+  floatx16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;  // log2 domain
+
+  for (int k0 = w_begin; k0 < w_end; k0 += TK) {
+    EXO_STORE1(0) EXO_STORE1(1) EXO_STORE1(2) EXO_STORE1(3) EXO_STORE1(4) EXO_STORE1(5) EXO_STORE1(6) EXO_STORE1(7)
+    // the tile is private to the wave: its writes are complete before its reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    EXO_LOAD_TILE(k0 + TK)
+
+    floatx16 sc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sc[e] = 0.f;
+    {
+      const bf16_t* kr = &k_t[key_of_row * KS + kq * 8];
+#pragma unroll
+      for (int st = 0; st < STEPS; ++st) {
+        const uint4 a = *reinterpret_cast<const uint4*>(kr + st * 16);
+        const uint4 qv = *reinterpret_cast<const uint4*>(qrow_lds + st * 16);
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                     __builtin_bit_cast(bf16x8_t, qv), sc, 0, 0, 0);
+      }
+    }
+    const int vis = w_end - k0;  // keys [0, vis) of the tile are real
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int key = 16 * (e >> 3) + 8 * kq + (e & 7);
+      const float x = key < vis ? sc[e] * scale_log2e : -INFINITY;
+      sc[e] = x;
+      mx = fmaxf(mx, x);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);  // finite: key 0 of the tile is real
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float sum = 0.f;
+    uint4 pb[2];
+    {
+      float pr[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        pr[e] = __builtin_amdgcn_exp2f(sc[e] - m_new);
+        sum += pr[e];
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        pb[st].x = pack_bf2(pr[8 * st + 0], pr[8 * st + 1]);
+        pb[st].y = pack_bf2(pr[8 * st + 2], pr[8 * st + 3]);
+        pb[st].z = pack_bf2(pr[8 * st + 4], pr[8 * st + 5]);
+        pb[st].w = pack_bf2(pr[8 * st + 6], pr[8 * st + 7]);
+      }
+    }
+    sum += __shfl_xor(sum, 32, 64);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      // V^T operand: lane (d = 32*dt + n, half kq) takes keys 16*st + 8*kq .. +8 of that d,
+      // four at a time with the transposing LDS read: a block of 16 lanes whose lane r
+      // points at V[key0 + r/4][d0 + 4*(r%4) ..+4] gets V[key0 .. key0+4][d0 + i] in lane i
+      const bf16_t* vr = &v_t[(kq * 8 + ((lane & 15) >> 2)) * VS + dt * 32 + ((lane >> 4) & 1) * 16 +
+                              (lane & 3) * 4];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const uint2 lo = lds_read_tr16(vr + (st * 16) * VS);
+        const uint2 hi = lds_read_tr16(vr + (st * 16 + 4) * VS);
+        const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                        __builtin_bit_cast(bf16x8_t, pb[st]),
+                                                        o[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (own_new && wave == 0) {
+    // the new token: one more key for every head, from LDS; this lane's half of the dot
+    float part = 0.f;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const uint4 kn4 = *reinterpret_cast<const uint4*>(&kv_new[st * 16 + kq * 8]);
+      const uint4 qv = *reinterpret_cast<const uint4*>(qrow_lds + st * 16);
+      part = dot2_bf16(qv.x, kn4.x, part);
+      part = dot2_bf16(qv.y, kn4.y, part);
+      part = dot2_bf16(qv.z, kn4.z, part);
+      part = dot2_bf16(qv.w, kn4.w, part);
+    }
+    const float sv = (part + __shfl_xor(part, 32, 64)) * scale_log2e;
+    const float m_new = fmaxf(m_run, sv);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    const float pn = __builtin_amdgcn_exp2f(sv - m_new);
+    l_run = l_run * alpha + pn;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int d = dt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+        o[dt][r] = o[dt][r] * alpha + pn * bf2f(kv_new[D + d]);
+      }
+  }
+
+#undef EXO_LOAD_TILE
+#undef EXO_LOAD1
+#undef EXO_STORE1
+  // ---- partial results of the waves, in the scalar kernel's layout: red[wave][head][d],
+  // then (max, sum) in natural-log units
+  __syncthreads();  // every wave is done with its tiles: the memory changes hands
+  float (*red)[G][D + 2] = reinterpret_cast<float (*)[G][D + 2]>(smem);
+  if (n < G) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        red[wave][n][dt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3)] = o[dt][r];
+    if (kq == 0) {
+      red[wave][n][D] = m_run * 0.6931471805599453f;
+      red[wave][n][D + 1] = l_run;
+    }
+  }
+  __syncthreads();
+
+  const size_t qrow = (size_t)b * p.Hq * D;
+  for (int idx = threadIdx.x; idx < G * D; idx += kThreads) {
+    const int g = idx / D, e = idx % D;
+    float mw = red[0][g][D];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mw = fmaxf(mw, red[w][g][D]);
+    float acc = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float mm = red[w][g][D];
+      const float scw = (mm == -INFINITY) ? 0.f : __expf(mm - mw);
+      acc += red[w][g][e] * scw;
+      lsum += red[w][g][D + 1] * scw;
+    }
+    float* dst = p.ws + ((size_t)(b * p.Hq + h0 + g) * p.splits + blockIdx.x) * (D + 2);
+    st_dev(dst + e, acc);
+    if (e == 0) {
+      st_dev(dst + D, mw);
+      st_dev(dst + D + 1, lsum);
+    }
+  }
+  // the last workgroup of this (sequence, kv head) merges the splits (see sdpa_kernel)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* cnt = &p.counters[b * p.Hkv + blockIdx.y];
+    const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (old == p.splits - 1);
+    if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  for (int idx = threadIdx.x; idx < G * D; idx += kThreads) {
+    const int g = idx / D, e = idx % D;
+    const int h = h0 + g;
+    const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
+    constexpr int MS = kMaxSplits;
+    float pm[MS], pl[MS], po[MS];
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp) {
+      const int spc = min(sp, p.splits - 1);
+      pm[sp] = ld_dev(src + (size_t)spc * (D + 2) + D);
+      pl[sp] = ld_dev(src + (size_t)spc * (D + 2) + D + 1);
+      po[sp] = ld_dev(src + (size_t)spc * (D + 2) + e);
+    }
+    float mw = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp)
+      if (sp < p.splits) mw = fmaxf(mw, pm[sp]);
+    float acc = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp) {
+      const float scw = (sp >= p.splits || pm[sp] == -INFINITY) ? 0.f : __expf(pm[sp] - mw);
+      acc += po[sp] * scw;
+      lsum += pl[sp] * scw;
+    }
+    p.out[qrow + (size_t)h * D + e] = f2bf(acc / lsum);
+  }
+}
+
 // Decode work split.  The G = Hq/Hkv query heads of a kv head are spread over `hgroups`
 // workgroups (each re-reads the K/V range from L2, but the per-key arithmetic, the register
 // footprint and the in-wave merge of a workgroup shrink with its head count): as many as
@@ -524,6 +842,28 @@ extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t*
                reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
                Hkv, S_max, pick_splits(B, Hq, Hkv, S_max), qkv, inv_freq,
                reinterpret_cast<const float2*>(rope_table), q_norm_w, k_norm_w, eps};
+  // 128 or more query heads per step (4+ sequences of 32 heads): the scalar kernel is bound
+  // by its vector instructions there and the matrix-core kernel is ahead (measured at 2050
+  // keys, 32 query / 8 kv heads: 4 sequences 16.9 -> 15.7 us, 8 sequences 24.4 -> 21.0 us; 2
+  // sequences level; one sequence with 8 or 16 heads per kv head 8.4 -> 11.8 and 10.5 -> 16.7
+  // us, so those stay with the scalar kernel)
+  const int G = Hq / Hkv;
+  if (D == 128 && (G == 4 || G == 8 || G == 16) && B * Hq >= 128) {
+    int sp = 256 / (B * Hkv);
+    sp = sp > kMaxSplits ? kMaxSplits : (sp < 1 ? 1 : sp);
+    if (sp > S_max / 128) sp = S_max / 128 > 0 ? S_max / 128 : 1;
+    p.splits = sp;
+    p.hgroups = 1;
+    const dim3 grid(p.splits, Hkv, B);
+    if (G == 4)
+      sdpa_decode_mfma_kernel<4><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+    else if (G == 8)
+      sdpa_decode_mfma_kernel<8><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+    else
+      sdpa_decode_mfma_kernel<16><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
+    EXO_CHECK_LAUNCH("exo_attn_decode");
+    return EXO_OK;
+  }
   rc = (D == 64) ? launch_sdpa<64, 2>(p, (hipStream_t)stream)
                  : launch_sdpa<128, 2>(p, (hipStream_t)stream);
   if (rc) return rc;

@@ -482,9 +482,10 @@ def test_norm_qmv_fused(device, bits, N, K, M):
     assert_close(got, O.swiglu(affine.qmm(xn, *trip, 64, bits), affine.qmm(xn, *g, 64, bits)), what="norm+qmv_swiglu")
 
 
-@pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 64, 4), (128, 4, 4)])
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 64, 4), (128, 4, 4), (128, 32, 4),
+                                      (128, 16, 4)])
 @pytest.mark.parametrize("qk_norm", [False, True])
-@pytest.mark.parametrize("lens", [[1, 2], [100, 37], [513, 1000]])
+@pytest.mark.parametrize("lens", [[1, 2], [100, 37], [513, 1000], [129, 33, 1024, 257]])
 @pytest.mark.parametrize("table", [False, True])
 def test_attn_decode_fused(device, D, Hq, Hkv, qk_norm, lens, table):
     """rope + head norm + cache append + attention in one launch == the three oracle ops."""
