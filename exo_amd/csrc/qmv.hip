@@ -1229,6 +1229,12 @@ int check_common(const char* name, int M, int N, int K, int bits, int group_size
   return EXO_OK;
 }
 
+// Exactly two rows over a short reduction run faster on the dot2 kernel with a two-row
+// activation tile (1.3-1.4 x the one-row time) than on the matrix-core GEMV (about 2 x);
+// from three rows on, and for long rows whose activations no longer stay in registers,
+// the matrix cores win.
+inline bool two_rows_on_dot2(int M, int K) { return M == 2 && K <= 8192; }
+
 }  // namespace
 
 extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
@@ -1248,7 +1254,7 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
   if (M == 0) return EXO_OK;
   // two or more rows: the matrix-core GEMV streams W once per tile of up to 16 rows
   // (with a workspace; without one a tile is as many rows as the LDS holds whole)
-  int cap = M >= 2 ? exo_qmv_mfma_max_rows(K, bits) : 0;
+  int cap = (M >= 2 && !two_rows_on_dot2(M, K)) ? exo_qmv_mfma_max_rows(K, bits) : 0;
   if (cap > 0 && workspace) cap = 16;
   if (cap >= 2) {
     int m0 = 0;
@@ -1335,7 +1341,7 @@ extern "C" int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_we
               (long long)workspace_bytes, (long long)exo_qmv_workspace(2 * N));
   if (M == 0) return EXO_OK;
   // two or more rows: both projections in one matrix-core launch per tile of up to 16 rows
-  if (workspace && M >= 2 && exo_qmv_mfma_max_rows(K, bits) > 0) {
+  if (workspace && M >= 2 && !two_rows_on_dot2(M, K) && exo_qmv_mfma_max_rows(K, bits) > 0) {
     int m0 = 0;
     while (M - m0 >= 2) {
       const int mt = (M - m0 < 16) ? (M - m0) : 16;

@@ -79,7 +79,8 @@ int exo_norm_qmv(const uint16_t* x, const uint16_t* norm_weight, float eps, cons
  * bytes, 256-byte aligned; its first 64 KiB are arrival counters, which the caller zeroes
  * once (every launch leaves them zero; one workspace serves launches of any N up to the N
  * it was sized for).  Launches that share a workspace must be ordered
- * on one stream.  workspace == NULL behaves like exo_norm_qmv.  M == 1 never touches it. */
+ * on one stream.  workspace == NULL behaves like exo_norm_qmv.  M == 1 never touches it,
+ * nor does M == 2 with K <= 8192 (two rows ride the single-row kernel's two-row tile). */
 int64_t exo_qmv_workspace(int N);
 int exo_norm_qmv_ws(const uint16_t* x, const uint16_t* norm_weight, float eps,
                     const uint32_t* w, const uint16_t* scales, const uint16_t* biases,

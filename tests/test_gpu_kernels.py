@@ -110,7 +110,7 @@ def test_qmv_residual(device, bits):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("M", [1, 4, 9, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 9, 16])
 def test_qmv_swiglu(device, bits, M):
     N, K = 320, 2048
     g = rand_quantized(N, K, bits, seed=31)
@@ -468,7 +468,8 @@ def test_argmax_logsumexp(device, V):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("N,K,M", [(256, 4096, 1), (128, 14336, 2), (96, 768, 1), (64, 2048, 4), (72, 192, 3)])
+@pytest.mark.parametrize("N,K,M", [(256, 4096, 1), (128, 14336, 2), (96, 768, 1), (64, 2048, 4), (72, 192, 3),
+                                   (200, 4096, 2), (64, 8192, 2)])
 def test_norm_qmv_fused(device, bits, N, K, M):
     trip = rand_quantized(N, K, bits, seed=N + K)
     x = rand_bf16((M, K), seed=K + M, scale=3.0)
