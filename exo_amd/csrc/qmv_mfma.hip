@@ -574,7 +574,7 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   }
   // many row blocks: teams of 4 waves share the staged x (2 teams for up to 8 rows, 3 for
   // up to 16)
-  const int NG = (KW == 4 && NB >= 1024) ? (MR == 8 ? 3 : (M > 4 ? 2 : 1)) : 1;
+  const int NG = (KW == 4 && NB >= 1024) ? (MR == 8 ? 3 : 2) : 1;
   const int NBq = (NB + NG - 1) / NG;
   // LDS the activations of a chunk may take: two workgroups per CU while a workgroup is
   // 4 or 8 waves, one beyond
