@@ -846,9 +846,12 @@ extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t*
   // by its vector instructions there and the matrix-core kernel is ahead (measured at 2050
   // keys, 32 query / 8 kv heads: 4 sequences 16.9 -> 15.7 us, 8 sequences 24.4 -> 21.0 us; 2
   // sequences level; one sequence with 8 or 16 heads per kv head 8.4 -> 11.8 and 10.5 -> 16.7
-  // us, so those stay with the scalar kernel)
+  // us, two sequences of 64 query / 4 kv heads 13.7 -> 17.6 us, so those stay with the
+  // scalar kernel: it also takes 16 or more (sequence, kv head) pairs to fill the chip with
+  // the matrix-core kernel's workgroups; 32 / 4 heads: 4 sequences level, 8 sequences
+  // 22.7 -> 18.4 us; 64 / 4 heads: 4 sequences 21.1 -> 19.2, 8 sequences 34.2 -> 23.5 us)
   const int G = Hq / Hkv;
-  if (D == 128 && (G == 4 || G == 8 || G == 16) && B * Hq >= 128) {
+  if (D == 128 && (G == 4 || G == 8 || G == 16) && B * Hq >= 128 && B * Hkv >= 16) {
     int sp = 256 / (B * Hkv);
     sp = sp > kMaxSplits ? kMaxSplits : (sp < 1 ? 1 : sp);
     if (sp > S_max / 128) sp = S_max / 128 > 0 ? S_max / 128 : 1;
