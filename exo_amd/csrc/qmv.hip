@@ -1091,18 +1091,46 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   // waves get contiguous, balanced row ranges; 4 workgroups per CU (LDS permitting) and
   // at least one full batch of rows per wave
   int per_cu = pl.lds <= 36 * 1024 ? 4 : (pl.lds <= 72 * 1024 ? 2 : 1);
+  // up to 8 per CU for the (gate, up) pair, so that a 14336-row pair runs as 1792
+  // workgroups of exactly two rows per wave (15.8 -> 15.1 us), and for one-unit rows
+  // (128256x2048: 35.4 -> 33.4 us)
+  // (the rules marked 'single' were measured with one activation row and one launch per
+  // matrix; the two-row tile was slower with them)
+  const bool single = MT == 1 && pairs == 1;
+  if (single && per_cu == 4 && (NMAT == 2 || ITERS == 1)) per_cu = 8;
   int grid = 256 * per_cu;
   // (gather mode, several (token, slot) pairs: half of that - the launch is latency-bound
   // and twice as many workgroups finish sooner; a quarter was slower again)
   int min_rows = (8 + ITERS * NMAT - 1) / (ITERS * NMAT);
+  // (8 units per row: two rows per wave, 4096x8192 8-bit 11.9 -> 10.8 us)
+  if (single && ITERS * NMAT == 8) min_rows = 2;
   if (pairs > 1 && min_rows > 1) min_rows /= 2;
   // short matrices: fewer rows per wave while that grid would stay under 160 workgroups
-  // (2048x2048: 64 -> 256 workgroups, 4.0 -> 2.9 us; 2048x4096: 3.5 -> 3.2 us; 160 and more
-  // workgroups were faster as they are: 5120x2048, 4096x4096, 6144x4096)
+  // (2048x2048: 64 -> 256 workgroups, 4.0 -> 2.9 us; 2048x4096: 3.5 -> 3.2 us)
   while (min_rows > 1 && p.N / (min_rows * kWaves) < 160) min_rows /= 2;
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
+  if (single) {
+    // The same number of workgroups on each of the 256 CUs: a grid between two multiples
+    // of 256 leaves some CUs with one workgroup more than the others for the whole launch
+    // (6144x4096 with fused norm: 384 workgroups 7.5 us, 320: 8.2, 512: 6.9, 256: 6.2;
+    // 5120x2048: 160 workgroups 4.4 us, 256: 3.8).
+    if (grid >= 160 && grid < 256 && p.N >= 256 * kWaves) grid = 256;
+    if (grid > 256) {
+      grid -= grid % 256;
+      // ... and, where one exists in the upper half, a multiple that gives every wave the
+      // same number of rows (9216x4096 8-bit: 1024 workgroups 12.4 us, 768: 11.7)
+      for (int g = grid; g >= 256 && 2 * g > grid; g -= 256)
+        if (p.N % (g * kWaves) == 0) {
+          grid = g;
+          break;
+        }
+    }
+  }
   if (grid < 1) grid = 1;
+#ifdef EXO_TUNE_ENV
+  if (const char* e = getenv("EXO_QMV_GRID")) { int g = atoi(e); if (g > 0) grid = g; }
+#endif
   kern<<<dim3(grid, pairs), dim3(kThreads), kRowsXR<MT, ITERS, NMAT> ? 0 : pl.lds, st>>>(p);
   return EXO_OK;
 }
