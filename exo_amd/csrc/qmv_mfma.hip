@@ -564,14 +564,20 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   const int sps = 4;
   const int ssg = sps / (bits == 4 ? 1 : 2);
   const int n_steps = p.G / ssg;  // super-steps along K
-  // waves per row block: as many as keep the whole grid at about 4096 waves with at
-  // least two super-steps each (16 needs the 128-register kernels: M <= 8 only)
+  // waves per row block: as many as keep the grid at about 4096 waves per matrix with at
+  // least one super-step each, 16 only where two remain (16 needs the 128-register kernels:
+  // M <= 8 only).  Measured at 8 rows, K = 4096: 6144 rows 16 waves 12.5 us, 8 waves 12.0;
+  // the 14336-row (gate, up) pair 4 waves 26.5 us, 8 waves 24.6.
   int KW = 4;
   if (MR == 4) {
-    while (KW < 16 && NB * nmat * KW * 2 <= 4096 && n_steps >= KW * 2) KW *= 2;
+    while (KW < 16 && NB * KW * 2 <= 4096 && n_steps >= KW * 2 && (KW < 8 || n_steps >= KW * 4))
+      KW *= 2;
   } else if (NB <= 128 && n_steps <= 16) {
     KW = 8;  // more registers per wave: 8 waves, and only where both N and K are short
   }
+#ifdef EXO_TUNE_ENV
+  if (const char* e = getenv("EXO_MFMA_KW")) { int v = atoi(e); if (v > 0) KW = v; }
+#endif
   // many row blocks: teams of 4 waves share the staged x (2 teams for up to 8 rows, 3 for
   // up to 16)
   const int NG = (KW == 4 && NB >= 1024) ? (MR == 8 ? 3 : 2) : 1;
@@ -582,13 +588,17 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   int ksplit = 1;
   if (workspace && (size_t)NB * 4 > kCounterBytes) workspace = nullptr;  // N beyond 524288
   if (workspace) {
-    // split K until a chunk of x fits the LDS, and further while the grid is narrower
-    // than the chip; a chunk is at least one super-step per wave
+    // split K until a chunk of x fits the LDS, and further while the grid stays within one
+    // workgroup per CU (4096 rows at 8 waves: 128 workgroups 9.8 us, 256: 8.9; 6144 rows:
+    // 192 workgroups 12.0 us, 384: 14.5); a chunk is at least one super-step per wave
     while (ksplit < kMaxSplit && (p.G + ksplit - 1) / ksplit > KW * ssg &&
            (lds_bytes(M, (p.G + ksplit - 1) / ksplit, bits, MR, KW, NG) > lds_cap ||
-            NBq * ksplit < 256))
+            NBq * (ksplit + 1) <= 256))
       ++ksplit;
   }
+#ifdef EXO_TUNE_ENV
+  if (const char* e = getenv("EXO_MFMA_KS")) { int v = atoi(e); if (v > 0 && workspace) ksplit = v; }
+#endif
   int gc = (p.G + ksplit - 1) / ksplit;
   gc = (gc + ssg - 1) / ssg * ssg;  // chunks in whole super-steps
   if (gc > p.G) gc = p.G;
