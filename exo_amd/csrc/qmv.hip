@@ -1128,9 +1128,6 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
     }
   }
   if (grid < 1) grid = 1;
-#ifdef EXO_TUNE_ENV
-  if (const char* e = getenv("EXO_QMV_GRID")) { int g = atoi(e); if (g > 0) grid = g; }
-#endif
   kern<<<dim3(grid, pairs), dim3(kThreads), kRowsXR<MT, ITERS, NMAT> ? 0 : pl.lds, st>>>(p);
   return EXO_OK;
 }

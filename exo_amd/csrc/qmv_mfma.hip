@@ -575,9 +575,6 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
   } else if (NB <= 128 && n_steps <= 16) {
     KW = 8;  // more registers per wave: 8 waves, and only where both N and K are short
   }
-#ifdef EXO_TUNE_ENV
-  if (const char* e = getenv("EXO_MFMA_KW")) { int v = atoi(e); if (v > 0) KW = v; }
-#endif
   // many row blocks: teams of 4 waves share the staged x (2 teams for up to 8 rows, 3 for
   // up to 16)
   const int NG = (KW == 4 && NB >= 1024) ? (MR == 8 ? 3 : 2) : 1;
@@ -596,9 +593,6 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
             NBq * (ksplit + 1) <= 256))
       ++ksplit;
   }
-#ifdef EXO_TUNE_ENV
-  if (const char* e = getenv("EXO_MFMA_KS")) { int v = atoi(e); if (v > 0 && workspace) ksplit = v; }
-#endif
   int gc = (p.G + ksplit - 1) / ksplit;
   gc = (gc + ssg - 1) / ssg * ssg;  // chunks in whole super-steps
   if (gc > p.G) gc = p.G;
