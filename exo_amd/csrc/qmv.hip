@@ -1110,6 +1110,16 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   while (min_rows > 1 && p.N / (min_rows * kWaves) < 160) min_rows /= 2;
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
+  if (pairs > 1) {
+    // gather mode (one launch covers `pairs` (token, slot) products, blockIdx.y each): every
+    // workgroup stages and normalises its token's activations first, so two rows per wave
+    // at least, and about 1536 workgroups in all.  Measured, workgroups per pair: 768x2048
+    // 4-bit (gate, up), 8 pairs: 192 7.3 us, 96 6.3, 64 6.4, 48 6.7; 32 pairs: 192 19.1 us,
+    // 96 14.4, 48 12.9, 32 13.4; 1536x4096 8-bit, 8 pairs: 384 25.0 us, 192 22.2, 128 22.9.
+    const int two_rows = (p.N + 2 * kWaves - 1) / (2 * kWaves);
+    const int share = 1536 / pairs < 1 ? 1 : 1536 / pairs;
+    grid = two_rows < share ? two_rows : share;
+  }
   if (single) {
     // The same number of workgroups on each of the 256 CUs: a grid between two multiples
     // of 256 leaves some CUs with one workgroup more than the others for the whole launch
