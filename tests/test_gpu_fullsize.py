@@ -46,6 +46,38 @@ def _rows_np(qw, rows):
     return (qw.weight[r].cpu().numpy().view(np.uint32), n_bits(qw.scales[r]), n_bits(qw.biases[r]))
 
 
+# projections of the other configurations whose workgroup count is rounded to whole
+# multiples of the CU count or to an even number of rows per wave: 5 and 3 rows per wave,
+# a split of 9216 rows over 768 workgroups, one-unit rows of a 151936-row head
+LAUNCH_SHAPES = [(5120, 2048, 4), (3072, 2048, 4), (6144, 4096, 4), (9216, 4096, 8),
+                 (4096, 8192, 8), (6144, 4096, 8), (151936, 2048, 4)]
+
+
+@pytest.mark.parametrize("N,K,bits", LAUNCH_SHAPES)
+def test_qmv_launch_shapes(device, N, K, bits):
+    """Single-row and 8-row GEMV with the fused RMSNorm and with the fused residual, every
+    output against dequantize + float32 matmul, a row sample against the oracle."""
+    qw = _packed(N, K, bits, seed=N + K + bits, device=device)
+    rows = np.unique(np.concatenate([[0, 1, N - 2, N - 1], np.random.default_rng(N).integers(0, N, 124)]))
+    sub = _rows_np(qw, rows)
+    rt = torch.as_tensor(rows, device=device)
+    wd = ops.dequantize(qw).float()
+    nw = affine.bf16_round(rand_bf16((K,), seed=7) * 0.1 + 1.0)
+    nwt = t_bf16(nw, device)
+    for M in (1, 8):
+        x = rand_bf16((M, K), seed=M + N)
+        xt = t_bf16(x, device)
+        res = rand_bf16((M, N), seed=M + K)
+        y = ops.quantized_matmul(xt, qw, residual=t_bf16(res, device))
+        want = affine.bf16_round(affine.qmm(x, *sub, 64, bits)) + res[:, rows]
+        assert_close(n_f32(y[:, rt]), affine.bf16_round(want), what=f"residual, oracle rows, {M}x{N}x{K} b{bits}")
+        full = (xt.float() @ wd.T).bfloat16().float() + t_bf16(res, device).float()
+        assert_close(n_f32(y), n_f32(full), what=f"residual, all outputs, {M}x{N}x{K} b{bits}")
+        yn = ops.quantized_matmul(xt, qw, norm_weight=nwt, eps=1e-5)
+        xn = ops.rms_norm(xt, nwt, 1e-5)
+        assert_close(n_f32(yn), n_f32(xn.float() @ wd.T), what=f"norm, all outputs, {M}x{N}x{K} b{bits}")
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("N,K", SWEEP_SHAPES)
 def test_qmatmul_sweep_shapes(device, bits, N, K):
