@@ -34,6 +34,11 @@ class ModelConfig:
     num_experts_per_tok: int = 0
     moe_intermediate_size: int = 0
     norm_topk_prob: bool = True
+    # per-module-path entries of config.json's "quantization" map (mlx_lm writes one for
+    # every module converted at another width than the default, e.g. a MoE router kept
+    # at 8 bits): path -> {"group_size", "bits"}.  The engine itself takes each tensor's
+    # width from its shapes; this map only drives weight synthesis and round-trips.
+    quant_overrides: dict | None = None
 
     def __post_init__(self):
         if self.model_type not in SUPPORTED_MODEL_TYPES:
@@ -49,6 +54,11 @@ class ModelConfig:
     @property
     def is_moe(self) -> bool:
         return self.model_type == "qwen3_moe"
+
+    def bits_for(self, path: str) -> int:
+        """Bit width of the module at ``path`` (e.g. ``model.layers.3.mlp.gate``)."""
+        o = (self.quant_overrides or {}).get(path)
+        return int(o["bits"]) if o else self.bits
 
     @staticmethod
     def from_dict(d: dict) -> "ModelConfig":
@@ -73,6 +83,7 @@ class ModelConfig:
             num_experts_per_tok=d.get("num_experts_per_tok", 0),
             moe_intermediate_size=d.get("moe_intermediate_size", 0),
             norm_topk_prob=d.get("norm_topk_prob", True),
+            quant_overrides={k: v for k, v in q.items() if isinstance(v, dict)} or None,
         )
 
     @staticmethod
@@ -82,7 +93,8 @@ class ModelConfig:
 
     def to_dict(self) -> dict:
         d = asdict(self)
-        d["quantization"] = {"group_size": d.pop("group_size"), "bits": d.pop("bits")}
+        d["quantization"] = {"group_size": d.pop("group_size"), "bits": d.pop("bits"),
+                             **(d.pop("quant_overrides") or {})}
         return d
 
 

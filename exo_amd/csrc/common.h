@@ -80,6 +80,18 @@ __device__ __forceinline__ float run_sum(float v) {
   return v;
 }
 
+// Hand-over of results to another workgroup without a device-wide fence: the producer
+// writes its values with device-scope stores, then every storing wave waits here until all
+// of its outstanding vector-memory operations have completed (on gfx9 stores count in
+// vmcnt and are acknowledged once they are visible at the scope they were issued with),
+// then the workgroup barrier, then ONE thread bumps the arrival counter with a
+// device-scope read-modify-write.  A consumer that saw the counter value loads the values
+// at device scope.  The chain  store(sc1) -> vmcnt(0) -> s_barrier -> RMW(agent) ->
+// load(sc1)  orders the values before the counter without writing the L2 back.
+__device__ __forceinline__ void wait_own_stores_done() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // ---- host side -------------------------------------------------------------
 #define EXO_OK 0
 #define EXO_ERR_ARG (-1)

@@ -151,24 +151,7 @@ __device__ __forceinline__ void stage_x(const QmvParams& p, const bf16_t* x, uin
       if (m < p.M) {
         uint4 xv = load_word_x<BITS>(x + (size_t)m * p.K, wi);
         if (p.norm_w) norm_word<BITS>(xv, load_word_x<BITS>(p.norm_w, wi), inv[m]);
-        if (BITS == 4) {
-          o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
-          o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
-          o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
-          o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
-          truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
-                    (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
-          stored = truesum;
-        } else {
-          uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);  // (x0,x2)
-          uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u); // (x1,x3)
-          o.x = a;
-          o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
-          o.z = c2;
-          o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
-          truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
-          stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
-        }
+        o = permute_word<BITS>(xv, stored, truesum);
       }
       xs[(size_t)m * p.wpr + dst] = o;
       stored += __shfl_xor(stored, 1, 64);
@@ -258,27 +241,8 @@ __device__ __forceinline__ void stage_x_store(const QmvParams& p, XStage<BITS, M
     const int dst = (((j << 2) + t) << 6) + sl;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      const uint4 xv = st.r[m][it];
-      uint4 o;
       float stored, truesum;
-      if (BITS == 4) {
-        o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0,x4)
-        o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1,x5)
-        o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2,x6)
-        o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3,x7)
-        truesum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) +
-                  (bf_lo(o.z) + bf_hi(o.z)) + (bf_lo(o.w) + bf_hi(o.w));
-        stored = truesum;
-      } else {
-        const uint32_t a = __builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u);   // (x0,x2)
-        const uint32_t c2 = __builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u);  // (x1,x3)
-        o.x = a;
-        o.y = pack_bf2(bf_lo(a) * 16.f, bf_hi(a) * 16.f);
-        o.z = c2;
-        o.w = pack_bf2(bf_lo(c2) * 16.f, bf_hi(c2) * 16.f);
-        truesum = (bf_lo(a) + bf_hi(a)) + (bf_lo(c2) + bf_hi(c2));
-        stored = truesum + ((bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.w) + bf_hi(o.w)));
-      }
+      const uint4 o = permute_word<BITS>(st.r[m][it], stored, truesum);
       xs[m * WPR + dst] = o;
       stored += __shfl_xor(stored, 1, 64);
       truesum += __shfl_xor(truesum, 1, 64);
@@ -337,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   if (p.idx) {
     const int pair = blockIdx.y;
     int e = p.idx[pair];
-    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
     ew = (size_t)e * p.N * p.wpr;
     eg = (size_t)e * p.N * G;
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
@@ -540,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   if (p.idx) {
     const int pair = blockIdx.y;
     int e = p.idx[pair];
-    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
     ew = (size_t)e * p.N * p.wpr;
     eg = (size_t)e * p.N * G;
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
@@ -950,7 +914,7 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
   const int row0 = (int)blockIdx.x * (kDownRW * rpwi);
 
   int e = p.idx[(size_t)t * p.topk + slot];
-  e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);
+  e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
   const float score = bf2f(p.scores[(size_t)t * p.topk + slot]);
 
   // every weight load of this wave goes out first

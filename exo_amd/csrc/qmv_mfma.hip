@@ -445,7 +445,7 @@ __global__ __launch_bounds__(64 * KW * NG) void qmv_mfma_kernel(const MfmaParams
   // order (the result does not depend on arrival order), and writes y.  One counter round
   // trip per workgroup, after the streaming, instead of one per row block inside it.
   __shared__ int s_last;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this wave's partials are out
+  wait_own_stores_done();  // this wave's device-scope partial stores have completed
   __syncthreads();
   if (tid == 0) {
     int* cnt = &p.counters[blockIdx.x];

@@ -362,9 +362,9 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
   // The last workgroup of this (sequence, kv head) to finish merges the splits.  The
   // counter returns to zero, so the launch can be replayed without re-initialising it.
   // No device-wide fence (an L2 write-back on this chip): the partials were stored and
-  // are loaded at device scope, and the workgroup-scope release below only waits for
-  // this workgroup's stores to complete before the counter is bumped.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  // are loaded at device scope; every wave waits for its own stores to complete, the
+  // barrier collects the waves, and only then is the counter bumped.
+  wait_own_stores_done();
   __syncthreads();
   if (threadIdx.x == 0) {
     int* cnt = &p.counters[b * p.Hkv * p.hgroups + blockIdx.y];
@@ -683,7 +683,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
     }
   }
   // the last workgroup of this (sequence, kv head) merges the splits (see sdpa_kernel)
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  wait_own_stores_done();
   __syncthreads();
   if (threadIdx.x == 0) {
     int* cnt = &p.counters[b * p.Hkv + blockIdx.y];

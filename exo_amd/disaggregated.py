@@ -25,6 +25,7 @@ import time
 from collections import defaultdict
 from collections.abc import Callable
 from dataclasses import dataclass, field, fields
+import struct
 from typing import BinaryIO
 
 import msgpack
@@ -166,29 +167,44 @@ def _unpack(payload: bytes, what: str):
 # ------------------------------------------------------------------------- frames
 
 
-def _read_exactly(stream: BinaryIO, n: int) -> bytes:
-    buf = bytearray()
-    while len(buf) < n:
-        chunk = stream.read(n - len(buf))
-        if not chunk:
-            if len(buf) == 0:
-                return b""
-            raise ConnectionError(f"Connection closed after {len(buf)}/{n} bytes")
-        buf.extend(chunk)
-    return bytes(buf)
+_LEN = struct.Struct(">I")  # frame prefix: payload length, 4 bytes big-endian
+
+
+def _fill(stream: BinaryIO, want: int) -> bytes:
+    """``want`` bytes from a stream whose reads may come back short.  End of stream before
+    the first byte gives b"" (the peer closed between frames); end of stream inside the
+    block is an error."""
+    block = memoryview(bytearray(want))
+    have = 0
+    while have < want:
+        piece = stream.read(want - have)
+        if not piece:
+            if have:
+                raise ConnectionError(f"Connection closed after {have}/{want} bytes")
+            return b""
+        block[have : have + len(piece)] = piece
+        have += len(piece)
+    return block.tobytes()
 
 
 def write_frame(stream: BinaryIO, payload: bytes) -> None:
-    stream.write(len(payload).to_bytes(4, "big"))
-    stream.write(payload)
+    """One frame = length prefix + payload (protocol.py:76-79), flushed as a unit."""
+    prefix = _LEN.pack(len(payload))
+    if len(payload) <= 1 << 16:  # small frames go out in one write call
+        stream.write(prefix + payload)
+    else:  # KV chunks: no copy of the payload
+        stream.write(prefix)
+        stream.write(payload)
     stream.flush()
 
 
 def read_frame(stream: BinaryIO) -> bytes:
-    raw = _read_exactly(stream, 4)
-    if not raw:
+    """The next frame's payload, or b"" at a clean end of stream (protocol.py:81-86)."""
+    prefix = _fill(stream, _LEN.size)
+    if not prefix:
         return b""
-    return _read_exactly(stream, int.from_bytes(raw, "big"))
+    (size,) = _LEN.unpack(prefix)
+    return _fill(stream, size) if size else b""
 
 
 def encode(obj) -> bytes:

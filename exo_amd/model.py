@@ -53,21 +53,31 @@ def rope_inv_freq(cfg: ModelConfig) -> torch.Tensor:
     return inv.to(torch.float32)
 
 
+def _qw(w: dict, prefix: str, cfg: ModelConfig) -> QuantizedWeight:
+    """The (weight, scales, biases) triple under ``prefix``; the bit width comes from the
+    tensor shapes, so per-module overrides of the checkpoint's quantisation are honoured
+    and a malformed tensor fails here, at load, not at the first forward."""
+    return QuantizedWeight.from_tensors(w[prefix + ".weight"], w[prefix + ".scales"],
+                                        w[prefix + ".biases"], cfg.group_size, prefix)
+
+
 class _Layer:
     """Weights of one transformer block (device resident)."""
 
     def __init__(self, cfg: ModelConfig, w: dict, i: int):
         p = f"model.layers.{i}."
-        bits = cfg.bits
 
         def q(name: str) -> QuantizedWeight:
-            return QuantizedWeight(w[p + name + ".weight"], w[p + name + ".scales"],
-                                   w[p + name + ".biases"], bits, cfg.group_size)
+            return _qw(w, p + name, cfg)
 
         self.index = i
         self.in_norm = w[p + "input_layernorm.weight"]
         self.post_norm = w[p + "post_attention_layernorm.weight"]
         qp, kp, vp = q("self_attn.q_proj"), q("self_attn.k_proj"), q("self_attn.v_proj")
+        if not (qp.bits == kp.bits == vp.bits):
+            raise ValueError(f"{p}self_attn: q/k/v projections quantised at different widths "
+                             f"({qp.bits}/{kp.bits}/{vp.bits} bits) cannot share one launch")
+        bits = qp.bits
         # q|k|v concatenated along the output rows: one launch instead of three
         self.qkv = QuantizedWeight(
             torch.cat([qp.weight, kp.weight, vp.weight]).contiguous(),
@@ -133,15 +143,12 @@ class ShardModel:
         self.layers = [_Layer(cfg, weights, i) for i in range(self.start_layer, self.end_layer)]
         self.embed_tokens = None
         if self.is_first or (self.is_last and cfg.tie_word_embeddings):
-            self.embed_tokens = QuantizedWeight(
-                weights["model.embed_tokens.weight"], weights["model.embed_tokens.scales"],
-                weights["model.embed_tokens.biases"], cfg.bits, cfg.group_size)
+            self.embed_tokens = _qw(weights, "model.embed_tokens", cfg)
         self.norm = self.lm_head = None
         if self.is_last:
             self.norm = weights["model.norm.weight"]
-            self.lm_head = self.embed_tokens if cfg.tie_word_embeddings else QuantizedWeight(
-                weights["lm_head.weight"], weights["lm_head.scales"], weights["lm_head.biases"],
-                cfg.bits, cfg.group_size)
+            self.lm_head = self.embed_tokens if cfg.tie_word_embeddings else _qw(
+                weights, "lm_head", cfg)
         self.inv_freq = rope_inv_freq(cfg).to(self.device)
         self.scale = cfg.head_dim ** -0.5
         # inputs of up to this many rows take the GEMV family with fused norms; 8-bit
@@ -150,6 +157,7 @@ class ShardModel:
         self._bufs: dict[tuple[int, int], _Buffers] = {}
         self._graphs: dict[int, tuple] = {}
         self._rope_tab: torch.Tensor | None = None
+        self._retired_rope_tabs: list[torch.Tensor] = []
 
     # ------------------------------------------------------------------ properties
     @property
@@ -163,6 +171,8 @@ class ShardModel:
     def _rope_table(self, n: int) -> torch.Tensor:
         """(cos, sin) table covering n positions, built once on the device."""
         if self._rope_tab is None or self._rope_tab.shape[0] < n:
+            if self._rope_tab is not None:  # a captured graph may still point at the old table
+                self._retired_rope_tabs.append(self._rope_tab)
             self._rope_tab = ops.rope_table(self.inv_freq, n, self.cfg.head_dim)
         return self._rope_tab
 
@@ -214,15 +224,15 @@ class ShardModel:
         idx, sc = ops.router_topk(bf.router_logits, c.num_experts_per_tok, c.norm_topk_prob)
         k = c.num_experts_per_tok
         if not gemv:  # prefill: rows sorted by expert; gate, up and SwiGLU in one grouped GEMM
-            ws = ops.moe_group(idx, c.num_experts)
+            ws = ops.moe_group(idx, c.num_experts, check_indices=False)  # ids from router_topk
             ops.grouped_qmm_swiglu(bf.n.view(R, 1, -1), L.gate, L.up, ws, k, out=bf.act)
             ops.grouped_qmm(bf.act, L.down, ws, k, out=bf.expert_out)
             ops.moe_combine(bf.expert_out, sc, residual=bf.h, out=bf.h)
             return
         ops.gather_qmv_swiglu(bf.h, L.gate, L.up, idx, out=bf.act, norm_weight=L.post_norm,
-                              eps=c.rms_norm_eps)
+                              eps=c.rms_norm_eps, check_indices=False)
         ops.gather_qmv_combine(bf.act, L.down, idx, sc, residual=bf.h, out=bf.h,
-                               scratch=bf.expert_out)
+                               scratch=bf.expert_out, check_indices=False)
 
     def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
              rows: slice | None = None):
@@ -331,8 +341,11 @@ class ShardModel:
             key = (B, feedback)
             if key not in self._graphs or self._graphs[key][1] is not cache:
                 # warm up outside capture (lazy module loads, attribute settings), then
-                # restore the positions the warm-up advanced
+                # restore what the warm-up changed: the positions it advanced, the hidden
+                # state a later shard adds its residuals into in place, and the input
+                # tokens the feedback copy overwrote
                 saved = cache.pos.clone()
+                saved_in = bf.tokens.clone() if self.is_first else bf.h.clone()
                 s = torch.cuda.Stream()
                 s.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(s):
@@ -340,6 +353,7 @@ class ShardModel:
                 torch.cuda.current_stream().wait_stream(s)
                 torch.cuda.synchronize()
                 cache.pos.copy_(saved)
+                (bf.tokens if self.is_first else bf.h).copy_(saved_in)
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
                     body()

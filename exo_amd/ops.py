@@ -64,6 +64,22 @@ class QuantizedWeight:
             self.weight.numel() * 4 + self.scales.numel() * 2 + self.biases.numel() * 2
         )
 
+    @staticmethod
+    def from_tensors(weight: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                     group_size: int = GROUP_SIZE, name: str = "") -> "QuantizedWeight":
+        """Bits of this tensor from its own shapes (a checkpoint may quantise single modules
+        at another width than the ``quantization.bits`` of its config.json, through per-path
+        entries there): a row of K elements is K*bits/32 words and K/group_size scales."""
+        words, groups = weight.shape[-1], scales.shape[-1]
+        bits, rem = divmod(32 * words, group_size * groups)
+        if rem or bits not in (4, 8) or scales.shape != biases.shape or \
+                weight.shape[:-1] != scales.shape[:-1]:
+            raise ValueError(
+                f"{name or 'quantised tensor'}: weight {tuple(weight.shape)} with scales "
+                f"{tuple(scales.shape)} / biases {tuple(biases.shape)} is not an affine "
+                f"group-{group_size} tensor of 4 or 8 bits")
+        return QuantizedWeight(weight, scales, biases, bits, group_size)
+
     def to(self, device) -> "QuantizedWeight":
         return QuantizedWeight(
             self.weight.to(device).contiguous(),
@@ -298,7 +314,21 @@ def qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None, norm_wei
     return out
 
 
-def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, out=None):
+def check_expert_ids(idx: torch.Tensor, E: int, what: str) -> None:
+    """Reject expert ids outside [0, E).  Reads the indices back (a host synchronisation),
+    so it is skipped while the stream is being captured into a graph; callers whose indices
+    come straight from ``router_topk`` (in range by construction) pass
+    ``check_indices=False``.  The kernels clamp the id only so that a bad one cannot
+    address memory outside the weight tensor."""
+    if idx.numel() == 0 or torch.cuda.is_current_stream_capturing():
+        return
+    lo, hi = int(idx.min()), int(idx.max())
+    if lo < 0 or hi >= E:
+        raise ValueError(f"{what}: expert ids span [{lo}, {hi}], outside [0, {E})")
+
+
+def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, out=None,
+               check_indices: bool = True):
     """mx.gather_qmm(x, w, s, b, rhs_indices=idx, transpose=True) for decode-sized
     inputs: x bf16 [T, R, K] (R == 1 or topk), idx int32 [T, topk] -> bf16 [T, topk, N]."""
     lib = native.load()
@@ -306,6 +336,8 @@ def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, 
     topk = rhs_indices.shape[1]
     assert rhs_indices.dtype == torch.int32 and rhs_indices.shape[0] == T
     E = qw.weight.shape[0]
+    if check_indices:
+        check_expert_ids(rhs_indices, E, "gather_qmm")
     if out is None:
         out = torch.empty(T, topk, qw.N, dtype=torch.bfloat16, device=x.device)
     check(
@@ -318,7 +350,8 @@ def gather_qmm(x: torch.Tensor, qw: QuantizedWeight, rhs_indices: torch.Tensor, 
     return out
 
 
-def gather_qmv_combine(x, qw: QuantizedWeight, idx, scores, residual=None, out=None, scratch=None):
+def gather_qmv_combine(x, qw: QuantizedWeight, idx, scores, residual=None, out=None, scratch=None,
+                       check_indices: bool = True):
     """SwitchGLU's down projection for decode-sized inputs fused with the weighted sum over
     the top-k experts and the residual: x bf16 [T,topk,K], idx int32 [T,topk], scores bf16
     [T,topk], residual bf16 [T,N] -> bf16 [T,N].  ``scratch`` (bf16 [T,topk,N]) serves the
@@ -326,6 +359,8 @@ def gather_qmv_combine(x, qw: QuantizedWeight, idx, scores, residual=None, out=N
     lib = native.load()
     T, topk, K = x.shape
     E = qw.weight.shape[0]
+    if check_indices:
+        check_expert_ids(idx, E, "gather_qmv_combine")
     if out is None:
         out = torch.empty(T, qw.N, dtype=torch.bfloat16, device=x.device)
     check(
@@ -339,12 +374,14 @@ def gather_qmv_combine(x, qw: QuantizedWeight, idx, scores, residual=None, out=N
     return out
 
 
-def moe_group(idx: torch.Tensor, E: int) -> torch.Tensor:
+def moe_group(idx: torch.Tensor, E: int, check_indices: bool = True) -> torch.Tensor:
     """Sort the (token, slot) pairs of idx int32 [T, topk] by expert; the returned workspace
     feeds grouped_qmm for every projection that shares this routing decision."""
     lib = native.load()
     T, topk = idx.shape
     assert idx.dtype == torch.int32 and idx.is_contiguous()
+    if check_indices:
+        check_expert_ids(idx, E, "moe_group")
     nbytes = lib.exo_moe_group_workspace(T, topk, E)
     ws = torch.empty(nbytes // 4, dtype=torch.int32, device=idx.device)
     check(lib.exo_moe_group(_ptr(idx), T, topk, E, _ptr(ws), nbytes, _stream()), "moe_group")
@@ -394,13 +431,15 @@ def grouped_qmm_swiglu(x: torch.Tensor, gate: QuantizedWeight, up: QuantizedWeig
 
 
 def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=None,
-                      norm_weight=None, eps: float = 0.0):
+                      norm_weight=None, eps: float = 0.0, check_indices: bool = True):
     """SwitchGLU's gate/up + swiglu: x bf16 [T,K], idx int32 [T,topk] -> [T,topk,N];
     ``norm_weight`` fuses a preceding rms_norm(x, norm_weight, eps)."""
     lib = native.load()
     T, K = x.shape
     topk = idx.shape[1]
     E = gate.weight.shape[0]
+    if check_indices:
+        check_expert_ids(idx, E, "gather_qmv_swiglu")
     if out is None:
         out = torch.empty(T, topk, gate.N, dtype=torch.bfloat16, device=x.device)
     check(

@@ -33,7 +33,7 @@ def _qlinear(out: dict, name: str, n: int, k: int, cfg: ModelConfig, base_seed: 
     slab = max(1, (1 << 28) // k)
     for r0 in range(0, rows, slab):
         w[r0 : r0 + slab].normal_(0.0, std, generator=gen)
-    wq, s, b = quantize(w.bfloat16().float(), cfg.group_size, cfg.bits)
+    wq, s, b = quantize(w.bfloat16().float(), cfg.group_size, cfg.bits_for(name))
     del w
     if experts:
         wq = wq.reshape(experts, n, -1)

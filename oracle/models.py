@@ -145,6 +145,16 @@ class ShardModel:
     def is_last(self) -> bool:
         return self.end_layer == self.cfg.num_hidden_layers
 
+    def _bits(self, prefix: str) -> int:
+        """Bit width of one tensor from its shapes: a row of K elements is K*bits/32 words
+        and K/group_size scales (.typings/mlx/core/__init__.pyi:4180-4188).  Checkpoints may
+        quantise single modules at another width than the default of config.json."""
+        words = self.weights[prefix + ".weight"].shape[-1]
+        groups = self.weights[prefix + ".scales"].shape[-1]
+        bits, rem = divmod(32 * words, self.cfg.group_size * groups)
+        assert rem == 0 and bits in (4, 8), (prefix, words, groups)
+        return bits
+
     def _wd(self, prefix: str, expert: int | None = None) -> np.ndarray:
         """float32 dequantised matrix (cached)."""
         key = (prefix, expert)
@@ -155,7 +165,7 @@ class ShardModel:
             if expert is not None:
                 w, s, b = w[expert], s[expert], b[expert]
             self._dq[key] = affine.dequantize_f32(
-                w, s, b, self.cfg.group_size, self.cfg.bits
+                w, s, b, self.cfg.group_size, self._bits(prefix)
             )
         return self._dq[key]
 
@@ -166,7 +176,7 @@ class ShardModel:
 
             y = cref.qmm_t(
                 affine.f32_to_bf16_bits(x.reshape(rows, -1)), self.weights[prefix + ".weight"],
-                self.weights[prefix + ".scales"], self.weights[prefix + ".biases"], self.cfg.bits)
+                self.weights[prefix + ".scales"], self.weights[prefix + ".biases"], self._bits(prefix))
             return bf16_bits_to_f32(y).reshape(*x.shape[:-1], -1)
         w = self._wd(prefix)
         if self.gemm_rows is not None and rows > self.gemm_rows:
@@ -260,7 +270,7 @@ class ShardModel:
                 self.weights["model.embed_tokens.scales"],
                 self.weights["model.embed_tokens.biases"],
                 c.group_size,
-                c.bits,
+                self._bits("model.embed_tokens"),
                 self.dequant_mode,
             ).reshape(B, T, c.hidden_size)
         else:

@@ -21,7 +21,8 @@ from exo_amd.model import ShardModel  # noqa: E402
 from exo_amd.synth import write_checkpoint  # noqa: E402
 from exo_amd.types import BoundInstance, GenerationTask, ShardMetadata, TextGenerationTaskParams  # noqa: E402
 
-KINDS = [("llama", 4), ("llama_tied_d128", 8), ("qwen3_moe", 4), ("qwen3_moe", 8)]
+KINDS = [("llama", 4), ("llama_tied_d128", 8), ("qwen3_moe", 4), ("qwen3_moe", 8),
+         ("qwen3_moe_router8", 4)]
 
 
 def _load(path, cfg, start, end, device):
@@ -164,6 +165,46 @@ def test_pipeline_shards_compose(ckpt, device):
     logits = s1(None, c1, input_embeddings=hidden)
     full = gm(tt, cf)
     np.testing.assert_array_equal(n_f32(logits), n_f32(full))
+
+
+def test_decode_step_first_replay_matches_call(ckpt, device):
+    """The graph-replayed single-token step, from its very first replay after a capture,
+    gives the bits of the plain forward: on a later shard (hidden state in, residuals
+    added in place) and on the whole model with the sampled token fed back on the device."""
+    cfg, gm, path = ckpt["cfg"], ckpt["model"], ckpt["path"]
+    L = cfg.num_hidden_layers
+    w0, _ = _load(path, cfg, 0, 1, device)
+    w1, _ = _load(path, cfg, 1, L, device)
+    s0, s1 = ShardModel(cfg, w0, 0, 1, device), ShardModel(cfg, w1, 1, L, device)
+    toks = torch.from_numpy(rng(13).integers(0, cfg.vocab_size, size=(1, 12)).astype(np.int32))
+    c0, ca, cb = s0.make_cache(1, 64), s1.make_cache(1, 64), s1.make_cache(1, 64)
+    h = s0(toks, c0)
+    s1(None, ca, input_embeddings=h, logits="none")
+    s1(None, cb, input_embeddings=h, logits="none")
+    for step in range(3):
+        t = torch.tensor([[int(rng(100 + step).integers(0, cfg.vocab_size))]], dtype=torch.int32)
+        h1 = s0(t, c0)
+        want = s1(None, ca, input_embeddings=h1)
+        bufs = s1._buffers(1, 1)
+        bufs.h.copy_(h1.view(1, -1))
+        bufs = s1.decode_step(cb, 1)
+        assert torch.equal(bufs.logits.view(-1), want.view(-1)), f"later shard, step {step}"
+        assert cb.offsets[0] == ca.offsets[0] and cb.pos.tolist() == ca.pos.tolist()
+    # whole model, device-side token feedback: eager steps against graph replays
+    ce, cg = gm.make_cache(1, 64), gm.make_cache(1, 64)
+    for c in (ce, cg):
+        gm(toks, c, logits="none")
+    first = int(rng(14).integers(0, cfg.vocab_size))
+    bufs = gm._buffers(1, 1)
+    bufs.tokens[0] = first
+    want_toks = []
+    for _ in range(4):
+        want_toks.append(int(gm.decode_step(ce, 1, use_graph=False, feedback=True).next_token[0]))
+    bufs.tokens[0] = first
+    got_toks = []
+    for _ in range(4):
+        got_toks.append(int(gm.decode_step(cg, 1, feedback=True).next_token[0]))
+    assert got_toks == want_toks
 
 
 def test_batch_generator_b2_equals_b1(ckpt, device):

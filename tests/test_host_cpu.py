@@ -91,6 +91,31 @@ def test_config_round_trip_and_rejects():
         ModelConfig.from_dict(dict(d, quantization={"group_size": 32, "bits": 4}))
 
 
+def test_per_module_bit_width_comes_from_the_tensor_shapes(tmp_path):
+    """A checkpoint that keeps single modules at another width (per-path entries of
+    config.json's quantization map): the map round-trips, the synthesised router tensor
+    has the 8-bit shape, and a tensor's width is read off its own shapes."""
+    from exo_amd.ops import QuantizedWeight
+    c = tiny_config("qwen3_moe_router8")
+    d = json.loads(json.dumps(c.to_dict()))
+    assert d["quantization"]["bits"] == 4
+    assert d["quantization"]["model.layers.1.mlp.gate"] == {"group_size": 64, "bits": 8}
+    assert ModelConfig.from_dict(d) == c and c.bits_for("model.layers.0.mlp.gate") == 8
+    assert c.bits_for("model.layers.0.self_attn.o_proj") == 4
+    w = synth_weights(c, seed=2)
+    H, E = c.hidden_size, c.num_experts
+    assert w["model.layers.0.mlp.gate.weight"].shape == (E, H * 8 // 32)
+    assert w["model.layers.0.self_attn.o_proj.weight"].shape[-1] == c.num_attention_heads * c.head_dim * 4 // 32
+    gate = QuantizedWeight.from_tensors(*(w[f"model.layers.0.mlp.gate.{k}"] for k in ("weight", "scales", "biases")))
+    o = QuantizedWeight.from_tensors(*(w[f"model.layers.0.self_attn.o_proj.{k}"] for k in ("weight", "scales", "biases")))
+    ex = QuantizedWeight.from_tensors(*(w[f"model.layers.0.mlp.switch_mlp.up_proj.{k}"] for k in ("weight", "scales", "biases")))
+    assert (gate.bits, gate.K, o.bits, ex.bits, ex.K) == (8, H, 4, 4, H)
+    with pytest.raises(ValueError):  # 3 words per group of 64: no 4- or 8-bit layout
+        QuantizedWeight.from_tensors(torch.zeros(4, 6, dtype=torch.int32),
+                                     torch.zeros(4, 2, dtype=torch.bfloat16),
+                                     torch.zeros(4, 2, dtype=torch.bfloat16), name="bad")
+
+
 def test_shard_tensor_selection_rule():
     c = tiny_config("llama")
     assert layer_index_of("model.layers.12.self_attn.q_proj.weight") == 12

@@ -146,6 +146,11 @@ def tiny_config(kind: str, bits: int = 4):
     if kind == "qwen3_moe":
         return ModelConfig("qwen3_moe", 256, 2, 8, 2, 128, 0, 600, 1e-6, 1e6, None, False, 64, bits,
                            8, 2, 128, True)
+    if kind == "qwen3_moe_router8":  # 4-bit experts and attention, router kept at 8 bits
+        c = tiny_config("qwen3_moe", 4)
+        c.quant_overrides = {f"model.layers.{i}.mlp.gate": {"group_size": 64, "bits": 8}
+                             for i in range(c.num_hidden_layers)}
+        return c
     raise KeyError(kind)
 
 
