@@ -16,6 +16,7 @@
 //          writes the output directly.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
+#include <mutex>
 #include "sdpa_internal.h"
 
 namespace {
@@ -806,6 +807,73 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_sdpa_decode");
   return EXO_OK;
+}
+
+// ---------------------------------------------------------------- no-allocation variant
+// exo_sdpa_decode for callers that cannot allocate (code under graph capture, serving
+// loops, harnesses that forbid it): the split-KV partials and arrival counters live in a
+// file-scope device array instead of a caller workspace.  The array's name is only a
+// host-side handle; its device address is looked up once per device and kept.
+constexpr int kStaticMaxHeads = EXO_SDPA_DECODE_STATIC_MAX_HEADS;  // B * Hq of one call
+constexpr int kStaticMaxD = 128;
+constexpr int64_t kStaticFloats =
+    (int64_t)kStaticMaxHeads * kMaxSplits * (kStaticMaxD + 2) + kStaticMaxHeads;
+static __device__ __align__(256) float scratch[kStaticFloats];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device
+static std::mutex g_scratch_mutex;
+
+// device address of this device's copy of `scratch` (resolved on first use)
+static int scratch_address(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    exo_set_error("exo_sdpa_decode_static: cannot identify the current device: %s",
+                  e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return EXO_ERR_HIP;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      exo_set_error("exo_sdpa_decode_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                    hipGetErrorString(e));
+      return EXO_ERR_HIP;
+    }
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return EXO_OK;
+}
+
+__global__ __launch_bounds__(256) void zero_ints_kernel(int* __restrict__ p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+extern "C" int exo_sdpa_decode_static(const uint16_t* q, const uint16_t* k_cache,
+                                      const uint16_t* v_cache, const int32_t* pos,
+                                      uint16_t* out, float scale, int B, int Hq, int Hkv, int D,
+                                      int S_max, exo_stream_t stream) {
+  int rc = check("exo_sdpa_decode_static", B, 1, Hq, Hkv, D, S_max);
+  if (rc) return rc;
+  EXO_REQUIRE((int64_t)B * Hq <= kStaticMaxHeads,
+              "exo_sdpa_decode_static: B*Hq = %lld query heads exceed the static scratch "
+              "(at most %d); use exo_sdpa_decode with a workspace",
+              (long long)B * Hq, kStaticMaxHeads);
+  EXO_REQUIRE(q && k_cache && v_cache && pos && out, "exo_sdpa_decode_static: null pointer");
+  float* ws = nullptr;
+  rc = scratch_address(&ws);
+  if (rc) return rc;
+  // The counters of this call's layout sit right behind its partials, where an earlier
+  // call of another shape may have left partial sums: they are cleared by a small kernel
+  // (no memset node, so the call can be captured into a graph).
+  const int n_cnt = B * Hq;
+  int* cnt = reinterpret_cast<int*>(ws + ws_partial_floats(B, Hq, D));
+  zero_ints_kernel<<<dim3(exo_ceil_div(n_cnt, 256)), 256, 0, (hipStream_t)stream>>>(cnt, n_cnt);
+  return exo_sdpa_decode(q, k_cache, v_cache, pos, out, ws, scale, B, Hq, Hkv, D, S_max, stream);
 }
 
 __global__ __launch_bounds__(256) void rope_table_kernel(const float* __restrict__ inv_freq,

@@ -217,6 +217,21 @@ int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache, const uint16_t* 
                     const int32_t* pos, uint16_t* out, float* workspace, float scale, int B,
                     int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
 
+/* exo_sdpa_decode for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the
+ * reference.  Same arguments and same results, bit for bit, as exo_sdpa_decode, minus the
+ * workspace: the split-KV partials and arrival counters live in a static device array
+ * inside the library (about 2.1 MB per GPU, held until the process ends).  The call
+ * allocates and frees nothing.  Limit: B * Hq <= EXO_SDPA_DECODE_STATIC_MAX_HEADS query
+ * heads per call (head_dim <= 128); larger calls return -1 with a message.  All calls on
+ * one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
+ * order them on one stream.  The first call on a device looks the array's address up and
+ * must not run under stream capture; later ones may be captured. */
+#define EXO_SDPA_DECODE_STATIC_MAX_HEADS 256
+int exo_sdpa_decode_static(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache,
+                           const int32_t* pos, uint16_t* out, float scale, int B, int Hq,
+                           int Hkv, int D, int S_max, exo_stream_t stream);
+
 /* K6+K10+K7 fused for decode: one launch per layer does what exo_rope_kv_append followed
  * by exo_sdpa_decode do for T == 1: q and k heads of the fused qkv row [B,(Hq+2Hkv)*D] are
  * (head-normalised and) rotated at position pos[b], the new k,v are appended to the

@@ -51,6 +51,9 @@ def test_argument_errors_without_gpu():
     assert lib.exo_qmm(None, None, None, None, None, None, 1, 64, 100, 4, 64, None) == -1
     assert lib.exo_sdpa_decode(None, None, None, None, None, None, 1.0, 1, 8, 3, 128, 64, None) == -1
     assert lib.exo_router_topk(None, None, None, 1, 300, 8, 1, None) == -1
+    # the no-allocation decode attention rejects sizes beyond its static scratch
+    assert lib.exo_sdpa_decode_static(None, None, None, None, None, 1.0, 9, 32, 8, 128, 64, None) == -1
+    assert b"exceed the static scratch" in lib.exo_last_error()
     assert lib.exo_sdpa_decode_workspace(2, 32, 128) == (2 * 32 * 16 * 130 + 2 * 32) * 4
     with pytest.raises(ValueError):
         native.check(-1, "x")
