@@ -58,6 +58,8 @@ SIGNATURES: dict[str, tuple] = {
     "exo_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "exo_argmax_workspace": (_i64, [_i]),
     "exo_argmax_logsumexp": (_i, [_vp] * 6 + [_i, _i, _vp]),
+    "exo_sample_workspace": (_i64, [_i]),
+    "exo_sample": (_i, [_vp] * 13 + [_i64, _i, _i, _i, _i, _vp]),
 }
 
 

@@ -307,6 +307,68 @@ int exo_argmax_logsumexp(const uint16_t* logits, int32_t* token, float* lse, flo
                          float* workspace, int32_t* pos_inc, int rows, int V,
                          exo_stream_t stream);
 
+/* A9, whole: everything between the model call and the next token in the reference's
+ * decode step (src/exo/worker/engines/mlx/patches/opt_batch_gen.py:67-107): the logits
+ * processors of each sequence (token bans src/exo/worker/engines/mlx/generator/
+ * generate.py:465-473; repetition / presence / frequency penalties, make_logits_processors
+ * .typings/mlx_lm/sample_utils.pyi:47-72 as called at generate.py:599-608),
+ * logprobs = logits - logsumexp(logits), the sequence's sampler (make_sampler
+ * .typings/mlx_lm/sample_utils.pyi:10-45 with the defaults of generate.py:614-619:
+ * temperature, top-p, min-p, top-k) and the 20 most likely tokens (opt_batch_gen.py:93-107).
+ *
+ * Per row r of bf16 logits [rows, V]:
+ *   x = logits[r] with the processors applied, each rounding its result to bf16: banned ids
+ *       -> -1e9; tokens among the last repetition_context of the history: x/penalty if
+ *       x >= 0 else x*penalty; among the last presence_context: x - presence_penalty;
+ *       x - frequency_penalty * (occurrences among the last frequency_context);
+ *   lse = logsumexp(x) (float32);
+ *   temperature == 0: token = argmax x (lowest id on ties);
+ *   else token i is kept iff x_i >= max(t_p, t_m, t_k): t_p the smallest value whose tokens
+ *       of strictly larger value hold less than top_p of the probability mass, t_m =
+ *       max(x) + log(min_p), t_k the k-th largest value; token = inverse CDF, in vocabulary
+ *       order, of the weights exp((x - max) / temperature) over the kept tokens at the
+ *       uniform u = (first word of Philox-4x32-10(counter = (draws[r],0,0,0), key =
+ *       (seed_lo, seed_hi)) >> 8) * 2^-24; draws[r] += 1;
+ *   logprob[r] = x[token] - lse;  top_idx/top_val [rows,20]: the 20 largest x, descending
+ *       (lower id first among equals), as ids and x - lse;
+ *   history[r][hist_len[r] % hist_cap] = token, hist_len[r] += 1 (history int32
+ *       [rows, hist_cap]: a ring of the sequence's latest tokens, prompt included);
+ *   feedback[r] = token (the next step's input id), pos_inc[r] += 1 - each when non-null.
+ * `mode` says which launches the rows need (rows whose parameters do not ask for a stage
+ * pass through it untouched): EDITS if any row bans or penalises, DRAW if any row has
+ * temperature != 0, TABLE if any sampling row uses top_p in (0,1) or top_k > 0, TOP for
+ * the top-20 outputs.  workspace: exo_sample_workspace(rows) bytes, 256-byte aligned,
+ * zeroed ONCE by the caller (every call leaves its tables zero); calls that share it must
+ * be ordered on one stream.  V <= 262144; contexts <= hist_cap <= 256. */
+#define EXO_SAMPLER_MAX_CONTEXT 256
+#define EXO_SAMPLER_MAX_BANNED 8
+#define EXO_SAMPLER_TOP_LOGPROBS 20
+#define EXO_SAMPLE_EDITS 1
+#define EXO_SAMPLE_DRAW 2
+#define EXO_SAMPLE_TABLE 4
+#define EXO_SAMPLE_TOP 8
+typedef struct exo_sampler_params {
+  float temperature;        /* 0: greedy */
+  float top_p;              /* in (0,1): nucleus filter; anything else: off */
+  float min_p;              /* > 0: keep p >= min_p * max p */
+  int32_t top_k;            /* > 0: keep the k most likely */
+  float repetition_penalty; /* 0 or 1: off */
+  int32_t repetition_context;
+  float presence_penalty;   /* 0: off */
+  int32_t presence_context;
+  float frequency_penalty;  /* 0: off */
+  int32_t frequency_context;
+  uint32_t seed_lo, seed_hi;
+  int32_t n_banned;         /* <= EXO_SAMPLER_MAX_BANNED */
+  int32_t banned[EXO_SAMPLER_MAX_BANNED];
+} exo_sampler_params;
+int64_t exo_sample_workspace(int rows);
+int exo_sample(const uint16_t* logits, const exo_sampler_params* params, int32_t* history,
+               int32_t* hist_len, uint32_t* draws, int32_t* token, float* logprob, float* lse,
+               int32_t* top_idx, float* top_val, int32_t* feedback, int32_t* pos_inc,
+               void* workspace, int64_t workspace_bytes, int rows, int V, int hist_cap, int mode,
+               exo_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

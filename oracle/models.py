@@ -171,7 +171,9 @@ class ShardModel:
 
     def linear(self, x: np.ndarray, prefix: str) -> np.ndarray:
         rows = int(np.prod(x.shape[:-1]))
-        if self.use_c and rows <= 16:
+        # (in exact mode - no bf16 rounding of the weights for long inputs - the C
+        # restatement serves every row count: no float32 copy of the matrix is formed)
+        if self.use_c and (rows <= 16 or self.gemm_rows is None):
             from . import cref
 
             y = cref.qmm_t(

@@ -181,3 +181,282 @@ def test_decode_attention_at_config_lengths(device, Hq, Hkv, S):
     ref = torch.nn.functional.scaled_dot_product_attention(
         q.view(B, Hq, 1, D).float(), k.float(), v.float(), enable_gqa=True)
     assert_close(n_f32(out.view(B, Hq, D)), n_f32(ref.view(B, Hq, D)), what=f"decode sdpa S={S}")
+
+
+# ------------------------------------------------------------------ workload-size attention
+
+
+def _causal_ref(q, k, v, pos, T, heads, Hq, Hkv, D):
+    """float32 library attention for a subset of query heads: q [T, Hq*D] of one sequence,
+    k/v [Hkv, S_max, D], query t attends keys j <= pos + t."""
+    S = pos + T
+    G = Hq // Hkv
+    qh = q.view(T, Hq, D)[:, heads].permute(1, 0, 2).float()              # [h, T, D]
+    kv = torch.as_tensor([h // G for h in heads], device=q.device)
+    kk, vv = k[kv, :S].float(), v[kv, :S].float()                          # [h, S, D]
+    mask = torch.arange(S, device=q.device)[None, :] <= (pos + torch.arange(T, device=q.device))[:, None]
+    return torch.nn.functional.scaled_dot_product_attention(qh, kk, vv, attn_mask=mask)  # [h, T, D]
+
+
+@pytest.mark.parametrize("Hq,Hkv,T,pos,S_max", [
+    (32, 8, 2046, 0, 2304),      # Llama-3.1-8B prompt chunk
+    (32, 4, 1022, 0, 1280),      # Qwen3-30B-A3B prompt chunk
+    (64, 4, 4094, 0, 4224),      # Qwen3-235B-A22B prompt chunk
+    (32, 8, 2048, 1500, 8192),   # a later chunk of a long prompt in the engine's default cache
+    (32, 8, 4096, 4096, 8192),   # a full-size chunk ending exactly at the end of the cache
+])
+def test_prefill_attention_at_config_lengths(device, Hq, Hkv, T, pos, S_max):
+    """The matrix-core flash kernel over thousands of keys (many key tiles, the causal edge
+    inside the last tiles) against float32 library attention, on the first, a middle and the
+    last query head of the first and the last kv head."""
+    D = 128
+    g = torch.Generator(device=device).manual_seed(T + pos)
+    q = torch.randn(T, Hq * D, device=device, generator=g).bfloat16()
+    k = torch.randn(1, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    v = torch.randn(1, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    out = torch.empty_like(q)
+    ops.sdpa_prefill(q, k, v, torch.tensor([pos], dtype=torch.int32, device=device), out,
+                     D ** -0.5, 1, T, Hq, Hkv, D)
+    G = Hq // Hkv
+    heads = sorted({0, G // 2, G - 1, Hq - G, Hq - 1})
+    ref = _causal_ref(q, k[0], v[0], pos, T, heads, Hq, Hkv, D)
+    got = out.view(T, Hq, D)[:, heads].permute(1, 0, 2)
+    assert_close(n_f32(got), n_f32(ref), what=f"prefill sdpa T={T} pos={pos} {Hq}/{Hkv}")
+
+
+def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed):
+    """exo_attn_decode (rope + append + attention) for B sequences at the given lengths,
+    against: rope by the oracle, float32 library attention over the cache."""
+    from oracle import ops as O
+    D = 128
+    g = torch.Generator(device=device).manual_seed(seed)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, device=device, generator=g).bfloat16()
+    kc = torch.randn(B, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    vc = torch.randn(B, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    k0, v0 = kc.clone(), vc.clone()
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=device)
+    inv = O.rope_inv_freq(D, 5e5, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                   "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
+    inv_t = torch.from_numpy(inv).to(device)
+    out = torch.empty(B, Hq * D, dtype=torch.bfloat16, device=device)
+    ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+    tab = ops.rope_table(inv_t, S_max, D)
+    for _ in range(2):  # twice: the arrival counters must be back at zero
+        ops.attn_decode(qkv, kc, vc, pos, inv_t, out, ws, D ** -0.5, B, Hq, Hkv, D, rope_tab=tab)
+    x = n_f32(qkv).reshape(B, 1, Hq + 2 * Hkv, D)
+    for b in range(B):
+        p = lens[b] - 1
+        qr = O.rope(x[b:b + 1, :, :Hq].transpose(0, 2, 1, 3), inv, p)               # [1,Hq,1,D]
+        kr = O.rope(x[b:b + 1, :, Hq:Hq + Hkv].transpose(0, 2, 1, 3), inv, p)       # [1,Hkv,1,D]
+        vn = x[b, 0, Hq + Hkv:]                                                     # [Hkv,D]
+        kk = torch.cat([k0[b, :, :p].float(), t_bf16(kr[0], device).float()], dim=1)  # [Hkv,p+1,D]
+        vv = torch.cat([v0[b, :, :p].float(), t_bf16(vn, device).float()[:, None]], dim=1)
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            t_bf16(qr[0], device).float()[None], kk[None], vv[None], enable_gqa=True)[0, :, 0]
+        assert_close(n_f32(out[b].view(Hq, D)), n_f32(ref), what=f"attn_decode B={B} len {lens[b]}")
+        assert torch.equal(kc[b, :, :p], k0[b, :, :p]) and torch.equal(kc[b, :, p + 1:], k0[b, :, p + 1:])
+        assert_close(n_f32(kc[b, :, p]), kr[0, :, 0], rtol=1e-2, what="appended k")
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,lens,S_max", [
+    (8, 32, 8, [2304, 2050, 2049, 2048, 1999, 1025, 130, 1], 2304),   # Llama-8B batch 8: matrix-core kernel
+    (4, 32, 4, [1280, 1026, 1025, 513], 1280),                        # Qwen3-30B batch 4: matrix-core kernel
+    (1, 32, 8, [2050], 8192),                                         # batch 1 in the engine's default cache
+    (1, 32, 8, [8191], 8192),
+    (4, 32, 8, [8191, 2050, 4097, 3], 8192),
+    (8, 32, 8, [8192, 8191, 2050, 2049, 4097, 4096, 65, 64], 8192),
+    (2, 64, 4, [4224, 4097], 4224),                                   # Qwen3-235B shard heads
+])
+def test_fused_decode_attention_at_config_lengths(device, B, Hq, Hkv, lens, S_max):
+    _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0])
+
+
+# ------------------------------------------------------------------ batched decode blocks
+
+
+@pytest.mark.parametrize("name,B,T0", [("llama-3.1-8b", 8, 24), ("qwen3-30b-a3b", 4, 6)])
+def test_block_batched_decode_at_real_shape(device, name, B, T0):
+    """One block at the real shapes with B sequences decoded together (8 rows: matrix-core
+    GEMV and matrix-core decode attention; MoE at 4 rows: gather kernels over 32 (token,
+    slot) pairs): a chunk per sequence, then three single-token steps, against the oracle."""
+    cfg, gm, om = _one_layer(name, device)
+    oc, gc = OM.make_kv_cache(1), gm.make_cache(B, 64)
+    h = rand_bf16((B, T0, cfg.hidden_size), seed=B + T0)
+    om.router_margins.clear()
+    want = om(None, oc, input_hidden=h)
+    got = n_f32(gm(None, gc, input_embeddings=t_bf16(h, device)))
+    tied = False
+    if cfg.is_moe:
+        tied = check_tokens(got, want, om, f"{name} B={B} chunk")
+    else:
+        assert_close(got, want, what=f"{name} B={B} chunk", tail_frac=1e-5)  # 786432 elements
+    for step in range(3):
+        if tied:
+            break
+        h1 = rand_bf16((B, 1, cfg.hidden_size), seed=300 + step)
+        om.router_margins.clear()
+        want = om(None, oc, input_hidden=h1)
+        got = n_f32(gm(None, gc, input_embeddings=t_bf16(h1, device)))
+        if cfg.is_moe:
+            tied = check_tokens(got, want, om, f"{name} B={B} step {step}")
+        else:
+            assert_close(got, want, what=f"{name} B={B} step {step}")
+    assert gc[0].offset == oc[0].offset
+
+
+# ------------------------------------------------------------------ configs[0], whole
+
+
+def _config0(device):
+    from exo_amd.synth import synth_weights as sw
+    cfg = named_config("llama-3.2-1b")
+    w = sw(cfg, seed=0, device=device)
+    om = OM.ShardModel(OM.Config.from_json(cfg.to_dict()), weights_to_numpy(w), use_c=True)  # exact mode
+    prompt = torch.randint(0, cfg.vocab_size, (128,), generator=torch.Generator().manual_seed(1234)).tolist()
+    return cfg, w, om, prompt
+
+
+@pytest.mark.timeout(900)
+def test_llama_1b_every_layer_at_depth(device):
+    """Every one of the 16 layers of the first benchmark configuration at its real shape and
+    on the activations it really sees at its depth: the oracle (exact mode: un-rounded float32
+    weights for every row count) walks the model layer by layer, each GPU layer is fed the
+    ORACLE's input of that layer - the 126-token prompt chunk (matrix-core GEMM + flash
+    attention), then three single-token steps (GEMV + decode attention on the cache the chunk
+    left).  Errors cannot compound across layers here.  The single-token steps (un-rounded
+    weights on both sides) are held to the single-layer elementwise bound at every depth.
+    The chunk goes through the matrix-core GEMM, whose operands are the weights rounded to
+    bf16; against the exact oracle that alone moves a layer's output by about 1e-2 relative
+    RMS with 0.4 % of the elements past the elementwise bound (the oracle differs from ITSELF
+    by that much when told to round its weights: 9.6e-3 and 0.38 % on layer 0), so the chunk
+    is held to relative RMS <= 2e-2 and <= 1 % outliers; the mirrored oracle (weights rounded
+    where the GEMM rounds them) holds the chunk to the elementwise bound in
+    test_llama_block_at_real_shape.  Then the final norm + tied 128256-row head."""
+    from oracle import ops as O
+    cfg, w, om, prompt = _config0(device)
+    L = cfg.num_hidden_layers
+    toks = np.array(prompt[:126])[None]
+    steps = [prompt[126], prompt[127], 4242]
+    ocache = OM.make_kv_cache(L)
+    emb = lambda t: affine.embed(np.asarray(t).reshape(-1), om.weights["model.embed_tokens.weight"],  # noqa: E731
+                                 om.weights["model.embed_tokens.scales"], om.weights["model.embed_tokens.biases"],
+                                 64, 4, "M1").reshape(1, -1, cfg.hidden_size)
+    # oracle pass: inputs[i][c] = hidden state entering layer i for call c (chunk, 3 steps)
+    inputs = [[] for _ in range(L + 1)]
+    for call in [toks] + [np.array([[t]]) for t in steps]:
+        h = emb(call)
+        for i in range(L):
+            inputs[i].append(h)
+            h = om.layer(h, i, ocache[i])
+        inputs[L].append(h)
+    worst, worst_chunk = 0.0, 0.0
+    for i in range(L):
+        gl = ShardModel(cfg, w, i, i + 1, device)
+
+        def run(gc, c, lo=0, hi=None):
+            if i == 0:
+                ids = toks[:, lo:hi] if c == 0 else np.array([[steps[c - 1]]])
+                return n_f32(gl(torch.from_numpy(ids.astype(np.int32)), gc))
+            x = inputs[i][c][:, lo:hi]
+            return n_f32(gl(None, gc, input_embeddings=t_bf16(x, device), logits="none"))
+
+        # the chunk in one call: matrix-core GEMM (bf16-rounded weights) + flash attention
+        rel, _ = assert_close_stat(run(gl.make_cache(1, 160), 0), inputs[i + 1][0], max_outlier_frac=1e-2,
+                                   what=f"config0 layer {i}, 126-token chunk through the GEMM")
+        worst_chunk = max(worst_chunk, rel)
+        # the same chunk in slices of 16 rows (matrix-core GEMV, un-rounded weights, short
+        # causal attention chunks), then the single-token steps on that cache: elementwise
+        gc = gl.make_cache(1, 160)
+        got = np.concatenate([run(gc, 0, lo, min(lo + 16, 126)) for lo in range(0, 126, 16)], axis=1)
+        e, atol = assert_close(got, inputs[i + 1][0], tail_frac=2e-4,
+                               what=f"config0 layer {i}, chunk in slices of 16 rows")
+        worst = max(worst, e / atol)
+        for c in range(1, 4):
+            e, atol = assert_close(run(gc, c), inputs[i + 1][c], what=f"config0 layer {i} step {c}")
+            worst = max(worst, e / atol)
+        del gl, gc
+    print(f"[config0] 16 layers: GEMV-path calls worst |err| = {worst:.2f} x atol; 126-token GEMM chunk worst "
+          f"relative RMS {worst_chunk:.2e}", flush=True)
+    head = ShardModel(cfg, w, L - 1, L, device)
+    hc = head.make_cache(1, 160)
+    for c in range(1, 4):
+        if c == 1:
+            head(None, hc, input_embeddings=t_bf16(inputs[L - 1][0], device), logits="none")
+        got = head(None, hc, input_embeddings=t_bf16(inputs[L - 1][c], device))
+        hn = O.rms_norm(inputs[L][c], om._norm_w("model.norm.weight"), cfg.rms_norm_eps)
+        want = om.linear(hn, "model.embed_tokens")
+        assert_close_stat(n_f32(got), want, what=f"config0 last layer + norm + head, call {c}")
+
+
+@pytest.mark.timeout(900)
+def test_llama_1b_whole_model_greedy_64_tokens(device):
+    """The first benchmark configuration end to end: the 16-layer Llama-3.2-1B architecture
+    (tied 128256-row head, llama3 rope factor 32), seeded 128-token prompt, 64 greedy tokens
+    through generate(), against the oracle in its EXACT mode.
+
+    1. free running: tokens identical up to the first step where they differ; that step must
+       be a near-tie of the oracle's own top two logits: their margin within the sum of the
+       two logits' tolerances, each rtol * |logit| + rtol * rms(logits) with rtol = 2e-2 (the
+       top logits of this random-weight model sit near 4, where one bf16 step is 0.031; the
+       margin of every step is printed);
+    2. teacher forced on the oracle's tokens for all 64 steps: the argmax agrees wherever the
+       oracle's margin is not a near-tie, and the logits agree to a relative RMS of 4e-2.
+       That is twice the single-op tolerance: through 16 layers of bf16-rounded ops two
+       correct evaluation orders drift apart by that much on their own (the same prompt
+       prefilled through this engine's GEMV path in chunks of 16 and of 1 token - identical
+       un-rounded weights, different summation order - gives logits 2.2e-2 apart); the
+       per-layer test above holds every layer to the tight bound."""
+    from exo_amd.generate import generate, prefill
+    from exo_amd.types import TextGenerationTaskParams
+    cfg, w, om, prompt = _config0(device)
+    gm = ShardModel(cfg, w, device=device)
+    del w
+    N, n_new = 128, 64
+    print(f"[config0] oracle: prefill {N - 1} + {n_new} greedy steps", flush=True)
+    want, wl = OM.greedy_generate(om, prompt, n_new)
+    rms = np.sqrt(np.mean(wl.astype(np.float64) ** 2, axis=1))
+    top2 = np.sort(wl, axis=1)[:, -2:]
+    margin = top2[:, 1] - top2[:, 0]
+    tol = 2e-2 * (np.abs(top2[:, 0]) + np.abs(top2[:, 1])) + 2 * 2e-2 * rms
+    near_tie = margin <= tol
+    task = TextGenerationTaskParams(model="llama-3.2-1b", max_output_tokens=n_new, temperature=0.0)
+    got = [r.token for r in generate(gm, None, task, prompt)]
+    assert len(got) == n_new
+    first_bad = next((i for i in range(n_new) if got[i] != want[i]), None)
+    for i in range(n_new):
+        print(f"[config0] step {i:2d}: oracle {want[i]:6d} gpu {got[i]:6d} margin {margin[i]:.4f} "
+              f"(tolerance {tol[i]:.4f}){' near-tie' if near_tie[i] else ''}"
+              f"{'  <- first difference' if i == first_bad else ''}", flush=True)
+    if first_bad is not None:
+        assert near_tie[first_bad], (f"free-running tokens differ at step {first_bad} where the oracle's "
+                                     f"margin {margin[first_bad]:.4f} is clear")
+    print(f"[config0] free running: identical for {n_new if first_bad is None else first_bad} steps; "
+          f"{int(near_tie[:32].sum())} near-ties among the first 32 oracle steps", flush=True)
+    # teacher forced: the GPU follows the oracle's token sequence
+    cache = gm.make_cache(1, N + n_new + 8)
+    prefill(gm, prompt[:-1], cache)
+    gm(torch.tensor([[prompt[-2]]], dtype=torch.int32), cache, logits="none")
+    fed = [prompt[-1]] + want[:-1]
+    agree, clear = 0, 0
+    for i in range(n_new):
+        bufs = gm._buffers(1, 1)
+        bufs.tokens[0] = fed[i]
+        bufs = gm.decode_step(cache, 1)
+        lg = n_f32(bufs.logits[0])
+        assert_close_stat(lg, wl[i], max_rel_rms=4e-2, max_outlier_frac=0.5,
+                          what=f"config0 teacher-forced logits step {i}")
+        tok = int(bufs.next_token[0])
+        if i == first_bad:
+            a, b = want[i], got[i]
+            print(f"[config0] step {i}: oracle logits ({wl[i][a]:.4f}, {wl[i][b]:.4f}) for tokens ({a}, {b}); "
+                  f"gpu logits ({lg[a]:.4f}, {lg[b]:.4f})", flush=True)
+        if not near_tie[i]:
+            clear += 1
+            assert tok == want[i], f"step {i}: argmax {tok} vs oracle {want[i]} at margin {margin[i]:.4f}"
+        agree += tok == want[i]
+    print(f"[config0] teacher forced: argmax agrees on {agree}/{n_new} steps ({clear} with a clear margin)", flush=True)
+    if first_bad is None or first_bad >= 32:
+        return
+    pytest.xfail(f"free-running tokens identical for {first_bad} < 32 steps: the oracle's own top-2 margin at "
+                 f"step {first_bad} is {margin[first_bad]:.4f}, inside the tolerance {tol[first_bad]:.4f}; every "
+                 f"teacher-forced step passed")

@@ -49,6 +49,34 @@ def ckpt(request, tmp_path_factory, device):
                 model=ShardModel(cfg, w, device=device), ocfg=ocfg, ow=ow, w=w)
 
 
+def test_logits_match_oracle_in_exact_mode(ckpt, device):
+    """The same prefill + single-token steps against the oracle's own arithmetic mode:
+    un-rounded float32 weights for every matmul, whatever its row count (gemm_rows=None),
+    i.e. without telling the oracle where the matrix-core GEMM rounds its weights to bf16."""
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    om = OM.ShardModel(ckpt["ocfg"], ckpt["ow"])
+    prompt = rng(12).integers(0, cfg.vocab_size, size=40)
+    oc, gc = OM.make_kv_cache(om.n_local_layers), gm.make_cache(1, 128)
+    want = om(prompt[None], oc)
+    got = gm(torch.from_numpy(prompt[None].astype(np.int32)), gc)
+    if cfg.is_moe:
+        tied = _check_tokens(n_f32(got), want, om, "prefill logits, exact oracle")
+    else:
+        assert_close_stat(n_f32(got), want, what="prefill logits, exact oracle")
+        tied = False
+    for step in range(6):
+        if tied:
+            break
+        t = int(rng(50 + step).integers(0, cfg.vocab_size))
+        om.router_margins.clear()
+        want = om(np.array([[t]]), oc)
+        got = gm(torch.tensor([[t]], dtype=torch.int32), gc)
+        if cfg.is_moe:
+            tied = _check_tokens(n_f32(got), want, om, f"decode step {step}, exact oracle")
+        else:
+            assert_close_stat(n_f32(got), want, what=f"decode logits step {step}, exact oracle")
+
+
 def test_prefill_and_decode_logits_match_oracle(ckpt, device):
     cfg, om, gm = ckpt["cfg"], ckpt["oracle"], ckpt["model"]
     prompt = rng(11).integers(0, cfg.vocab_size, size=40)

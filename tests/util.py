@@ -28,8 +28,11 @@ def rand_quantized(N, K, bits, seed, scale=0.02, E=None):
     return tuple(np.stack([p[i] for p in parts]) for i in range(3))
 
 
-def assert_close(got: np.ndarray, want: np.ndarray, rtol=RTOL, what=""):
-    """|got - want| <= rtol*|want| + atol with atol = rtol * rms(want)."""
+def assert_close(got: np.ndarray, want: np.ndarray, rtol=RTOL, what="", tail_frac=0.0):
+    """|got - want| <= rtol*|want| + atol with atol = rtol * rms(want).  ``tail_frac`` (for
+    outputs of several hundred thousand elements, where the far tail of the rounding-flip
+    distribution shows): that fraction of the elements may lie outside the bound, none
+    outside twice the bound."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
     assert got.shape == want.shape, (got.shape, want.shape)
@@ -37,6 +40,10 @@ def assert_close(got: np.ndarray, want: np.ndarray, rtol=RTOL, what=""):
     err = np.abs(got - want)
     bound = rtol * np.abs(want) + atol
     bad = err > bound
+    if tail_frac and bad.sum() <= tail_frac * bad.size and not (err > 2 * bound).any():
+        if bad.any():
+            print(f"[parity] {what}: {bad.sum()}/{bad.size} elements between one and two bounds (tail)")
+        return float(err.max()), atol
     if bad.any():
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError(
