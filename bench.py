@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-engine", action="store_true", help="skip the run through the Engine")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (1..16)")
     ap.add_argument("--shard-layers", type=int, default=None,
                     help="run layers [0, n) as a first pipeline shard (output: hidden state)")
@@ -105,18 +106,33 @@ def measure_kernels(model, torch, reps: int = 20):
         us = st.elapsed_time(en) * 1e3 / (reps * len(model.layers))
         out.append(dict(name=name, kernel=kname, launches_per_token=len(model.layers),
                         bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
-    # lm_head: one launch per token; rotate nothing (295 MB >> caches)
-    ops.quantized_matmul(xh, model.lm_head, out=y_v)
+    # lm_head: once per token, with 4 GB of layer weights streamed since its last use, so
+    # the 256 MB last-level cache holds none of it when it runs.  Re-reading ONE matrix back to
+    # back would find most of it there (5.0 against 4.7 TB/s measured), so the launches of the
+    # timed graph rotate over four copies of the matrix (1.2 GB).
+    from exo_amd.ops import QuantizedWeight
+    hd = model.lm_head
+    heads = [hd] + [QuantizedWeight(hd.weight.clone(), hd.scales.clone(), hd.biases.clone(), hd.bits)
+                    for _ in range(3)]
+    for q in heads:
+        ops.quantized_matmul(xh, q, out=y_v, norm_weight=nw, eps=eps)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for q in heads:
+            ops.quantized_matmul(xh, q, out=y_v, norm_weight=nw, eps=eps)
+    g.replay()
     torch.cuda.synchronize()
     st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     st.record()
     for _ in range(reps):
-        ops.quantized_matmul(xh, model.lm_head, out=y_v)
+        g.replay()
     en.record()
     torch.cuda.synchronize()
-    us = st.elapsed_time(en) * 1e3 / reps
-    nbytes = qbytes(c.vocab_size, H, c.bits) + 2 * (H + c.vocab_size)
-    out.append(dict(name="lm_head", kernel=kernel_name(1, H), launches_per_token=1,
+    us = st.elapsed_time(en) * 1e3 / (reps * len(heads))
+    del heads
+    nbytes = qbytes(c.vocab_size, H, c.bits) + 2 * (2 * H + c.vocab_size)
+    out.append(dict(name="norm_lm_head", kernel=kernel_name(1, H), launches_per_token=1,
                     bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
     return out
 
@@ -198,28 +214,78 @@ def cpu_baseline(model, torch, seconds: float, context: int):
     t_head /= n_head
     t_layer = max(t_full - t_head, 1e-9) / n_sample
     t_token = t_layer * c.num_hidden_layers + t_head
+    import importlib.util
+    have = {m: importlib.util.find_spec(m) is not None for m in ("mlx", "mlx_lm")}
+    mlx_note = ("mlx_lm: unavailable on this box (importlib finds neither mlx nor mlx_lm), so the baseline "
+                "is this repository's own CPU restatement; " if not all(have.values()) else
+                "mlx / mlx_lm are importable here but are not driven by this build; ")
     return dict(value=1.0 / t_token, unit="tok/s", cores=cref.num_threads(), kind="port",
-                sample=(f"{n_full} decode steps of {n_sample} layers + lm_head at context {context} "
+                mlx_importable=have,
+                sample=(mlx_note +
+                        f"{n_full} decode steps of {n_sample} layers + lm_head at context {context} "
                         f"(layer {t_layer * 1e3:.1f} ms, head {t_head * 1e3:.1f} ms), layer time "
                         f"scaled to {c.num_hidden_layers} layers; oracle/qmm_ref.c with OpenMP + numpy"),
                 host_cpus=os.cpu_count(), affinity=len(os.sched_getaffinity(0)))
 
 
+PMC_SUMMARY = "profiles/decode_llama8b_4bit_bs1_pmc_traffic.md"
+
+
 def pmc_traffic(launch: str):
     """HBM bytes per launch of one GEMV group as measured by the committed
     `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` passes of this command (a text summary
-    under profiles/; counters cannot be read from inside the process).  None if absent."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
-                        "decode_llama8b_4bit_bs1_pmc_traffic.md")
+    under profiles/; counters cannot be read from inside the process).  Returns (bytes,
+    where the figure comes from) or (None, None): it is a recorded measurement of that
+    earlier run, not of this one."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), PMC_SUMMARY)
+    val, commit = None, "unknown"
     try:
         with open(path) as fh:
             for line in fh:
                 parts = line.split()
                 if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == launch:
-                    return int(parts[2])
+                    val = int(parts[2])
+                if len(parts) >= 2 and parts[0] == "measured_at_commit":
+                    commit = parts[1]
     except OSError:
         pass
-    return None
+    if val is None:
+        return None, None
+    return val, f"{PMC_SUMMARY} (rocprofv3 --pmc passes recorded at commit {commit}; not re-measured by this run)"
+
+
+def engine_rates(model, cfg, args, torch):
+    """The same workload through the Engine the runner drives (BatchGenerator.step(): queue,
+    prefill, double-buffered graph replays with device sampling, detokeniser, chunks):
+    `generation_tps` as the reference defines it, (n-1)/(t_last - t_first) per request
+    (src/exo/worker/engines/mlx/generator/batch_generate.py:418-426), summed over the
+    requests of the batch; once greedy, once with the reference's default sampler
+    (temperature 0.7, min-p 0.05)."""
+    from exo_amd.engine import BatchGenerator
+    from exo_amd.types import GenerationTask, TextGenerationTaskParams
+
+    B, K = args.batch, args.steps + args.warmup
+    eng = BatchGenerator(model=model, tokenizer=None, model_id=args.config,
+                         max_seq=args.prompt + K + 72)
+    g = torch.Generator().manual_seed(1234)
+    prompts = [torch.randint(0, cfg.vocab_size, (args.prompt,), generator=g).tolist() for _ in range(B)]
+    res = {}
+    for label, temp in (("engine_tok_s", 0.0), ("engine_tok_s_sampled", 0.7)):
+        for i, p in enumerate(prompts):
+            eng.submit(GenerationTask(f"{label}-{i}", f"cmd-{i}", TextGenerationTaskParams(
+                model=args.config, input=p, max_output_tokens=K, temperature=temp, bench=True)))
+        tps, n_done = 0.0, 0
+        while n_done < B:
+            for _tid, ev in eng.step():
+                st = getattr(ev, "stats", None)
+                if st is not None:
+                    tps += st.generation_tps
+                    n_done += 1
+        res[label] = tps
+    res["engine_note"] = (f"{B} request(s) of {K} tokens through BatchGenerator.step(); generation_tps per "
+                          "request as the reference defines it, summed")
+    eng.close()
+    return res
 
 
 def active_token_bytes(model, cfg, ctx: int, batch: int) -> int:
@@ -397,11 +463,12 @@ def main():
             k["frac_of_8TBps"] = k["GBps"] / 8000.0
             k["us_per_token"] = k["avg_us"] * k["launches_per_token"]
         dom = max(kernels, key=lambda k: k["us_per_token"])
+        traffic, traffic_src = pmc_traffic(dom["name"]) if headline else (None, None)
         gemv_us = sum(k["us_per_token"] for k in kernels)
         gemv_bytes = sum(k["bytes_per_launch"] * k["launches_per_token"] for k in kernels)
         roofline = dict(bound="hbm", achieved=dom["GBps"], peak=8000.0, unit="GB/s",
                         frac=dom["GBps"] / 8000.0,
-                        traffic=pmc_traffic(dom["name"]) if headline else None, kernel=dom["kernel"],
+                        traffic=traffic, traffic_source=traffic_src, kernel=dom["kernel"],
                         launch=dom["name"], avg_us=dom["avg_us"], bytes_per_launch=dom["bytes_per_launch"],
                         all_gemv_GBps=gemv_bytes / gemv_us * 1e-3, all_gemv_us_per_token=gemv_us)
     else:
@@ -411,6 +478,10 @@ def main():
         roofline = dict(bound="hbm", achieved=gbps, peak=8000.0, unit="GB/s", frac=gbps / 8000.0,
                         traffic=None, kernel="all launches of one decode step",
                         bytes_per_launch=token_bytes, avg_us=dt / K * 1e6)
+
+    engine = None
+    if model.is_last and not args.no_engine:
+        engine = engine_rates(model, cfg, args, torch)
 
     what = {"llama-3.2-1b": "configs[0]", "llama-3.1-8b": "configs[2]", "qwen3-30b-a3b": "configs[3]",
             "qwen3-235b-a22b": "configs[4]"}.get(args.config, "custom")
@@ -429,6 +500,8 @@ def main():
         "token_bytes": token_bytes, "effective_GBps": token_bytes * (K / dt) * 1e-9,
         "kernels": kernels, "build_s": t_build, "last_token": last_token,
     }
+    if engine is not None:
+        out.update(engine)
     if not args.no_cpu_baseline and kernels is not None:
         out["cpu_baseline"] = cpu_baseline(model, torch, args.cpu_seconds, ctx0)
     else:

@@ -29,12 +29,13 @@ import torch
 from .cache import ShardKVCache
 from .config import ModelConfig
 from .generate import (
-    DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, ban_token_ids, extract_top_logprobs,
+    DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, TokenStream, extract_top_logprobs,
     make_sampler, prefill, processors_for,
 )
 from .loader import load_shard_weights
 from .model import ShardModel
 from .prefix_cache import KVPrefixCache, save_prefix_cache
+from .sampling import TOP_LOGPROBS, DeviceSampler, SamplerSettings
 from .tokenizer import load_tokenizer
 logger = logging.getLogger("exo_amd")
 
@@ -95,28 +96,46 @@ class _Seq:
     uid: int
     params: TextGenerationTaskParams
     prompt_tokens: list[int]
-    sampler: Callable
-    processors: list
-    greedy: bool
-    max_tokens: int
-    prefill_tps: float
-    prefill_tokens: int
+    settings: SamplerSettings
+    stream: TokenStream
     on_generation_token: Callable[[], None] | None
-    stop_sequences: list[str]
-    prefix_cache_hit: str = "none"
-    tokens: list[int] = field(default_factory=list)
-    n_gen: int = 0
-    t_first: float | None = None
-    t_last: float | None = None
-    accumulated: str = ""
+    want_top: bool
+    k_top: int
+    # host-side sampling, only for settings the device kernels do not take
+    sampler: Callable | None = None
+    processors: list | None = None
+    tokens: list[int] = field(default_factory=list)  # what the logits processors see
+
+    @property
+    def on_device(self) -> bool:
+        return self.sampler is None
+
+
+@dataclass
+class _Flight:
+    """One launched decode step whose results the host has not read yet."""
+
+    rows: list            # the sequences of the step, by batch row at launch time
+    slot: int             # which pinned host buffer set its outputs are copied into
+    event: Any
+    want_top: bool
 
 
 class ShardBatchGenerator:
     """Continuous batching over one KV pool of ``max_batch`` rows.  ``submit`` prefills
     the request into the next free row (batch-1 path) and feeds the last-but-one
-    prompt token as a single-token forward; ``step`` runs ONE graph-replayed
-    single-token forward for all active rows and maps the sampled tokens back to their
-    uids.  Active rows are kept compact at the front of the pool."""
+    prompt token as a single-token forward; ``step`` returns one token per active row.
+    Active rows are kept compact at the front of the pool.
+
+    A step is ONE graph replay: the single-token forward of all active rows followed by the
+    device sampling kernels (processors, filters, draw, top-20 log-probabilities), with the
+    chosen tokens written back as the next step's input.  Like the reference's patched step
+    (src/exo/worker/engines/mlx/patches/opt_batch_gen.py:108-124: ``async_eval`` of step n+1
+    before step n is read), ``step`` launches the NEXT replay before it waits for the results
+    of the one it returns, so the device never idles on the host's detokenising and
+    bookkeeping; the results travel through pinned host buffers guarded by an event.  When
+    the set of rows changes (a request finishes, is cancelled or joins), the chain restarts
+    from the host's tokens after the step in flight has been read."""
 
     def __init__(self, model: ShardModel, tokenizer, max_batch: int = EXO_MAX_CONCURRENT_REQUESTS,
                  max_seq: int = 8192, kv_prefix_cache: KVPrefixCache | None = None):
@@ -128,7 +147,17 @@ class ShardBatchGenerator:
         self.kv_prefix_cache = kv_prefix_cache
         self.rows: list[_Seq] = []
         self._next_uid = 0
-        self._pending_input: list[int] = []  # token to feed per active row
+        self._pending_input: list[int] = []  # latest token per active row, as the host knows it
+        self.sampler = DeviceSampler(max_batch, model.cfg.vocab_size, model.device)
+        self._flight: _Flight | None = None
+        pin = dict(pin_memory=True)
+        self._host = [dict(token=torch.zeros(max_batch, dtype=torch.int32, **pin),
+                           logprob=torch.zeros(max_batch, dtype=torch.float32, **pin),
+                           top_idx=torch.zeros(max_batch, TOP_LOGPROBS, dtype=torch.int32, **pin),
+                           top_val=torch.zeros(max_batch, TOP_LOGPROBS, dtype=torch.float32, **pin))
+                      for _ in range(2)]
+        self._slot = 0
+        self._sampler_stale = False
 
     @property
     def has_work(self) -> bool:
@@ -152,6 +181,7 @@ class ShardBatchGenerator:
             max_tokens = self.max_seq - len(toks) - 2
             if max_tokens <= 0:
                 raise ValueError(f"prompt of {len(toks)} tokens exceeds the cache ({self.max_seq})")
+        settings = SamplerSettings.from_task(task_params, self._eos())
         row = len(self.rows)
         # prefix cache lookup (batch_generate.py:164-181): bench requests opt in
         use_prefix = self.kv_prefix_cache is not None and (
@@ -189,31 +219,111 @@ class ShardBatchGenerator:
         if len(remaining) >= 2:
             self.model(torch.tensor([[remaining[-2]]], dtype=torch.int32), self.cache,
                        logits="none", rows=slice(row, row + 1))
-        gen = torch.Generator(device=self.model.device)
-        gen.manual_seed(task_params.seed or 42)
-        processors = processors_for(task_params, self._eos())
-        temp = task_params.temperature if task_params.temperature is not None else 0.7
+        k_top = task_params.top_logprobs or DEFAULT_TOP_LOGPROBS
         seq = _Seq(
-            uid=self._next_uid, params=task_params, prompt_tokens=toks,
-            sampler=make_sampler(
-                temp, task_params.top_p if task_params.top_p is not None else 1.0,
-                task_params.min_p if task_params.min_p is not None else 0.05,
-                task_params.top_k if task_params.top_k is not None else 0, gen),
-            processors=processors, greedy=(temp == 0 and not processors), max_tokens=max_tokens,
-            prefill_tps=tps, prefill_tokens=n, on_generation_token=on_generation_token,
-            prefix_cache_hit=prefix_cache_hit,
-            stop_sequences=[task_params.stop] if isinstance(task_params.stop, str)
-            else list(task_params.stop or []),
-            tokens=list(toks))
+            uid=self._next_uid, params=task_params, prompt_tokens=toks, settings=settings,
+            stream=TokenStream(self.tokenizer, task_params, self._eos(), max_tokens, len(toks), tps,
+                               prefix_cache_hit, self.model.device),
+            on_generation_token=on_generation_token, want_top=bool(task_params.logprobs), k_top=k_top,
+            # the generator is handed the last two prompt tokens (batch_generate.py:282,301):
+            # they are all the logits processors see of the prompt
+            tokens=list(toks[-2:]))
+        if settings.on_device() and k_top <= TOP_LOGPROBS:
+            self.sampler.set_row(row, settings, seq.tokens)
+        else:
+            gen = torch.Generator(device=self.model.device)
+            gen.manual_seed(settings.seed)
+            seq.processors = processors_for(task_params, self._eos())
+            seq.sampler = make_sampler(settings.temperature, settings.top_p, settings.min_p,
+                                       settings.top_k, gen)
         self._next_uid += 1
         self.rows.append(seq)
         self._pending_input.append(toks[-1])
         return seq.uid
 
-    def step(self) -> list[tuple[int, GenerationResponse]]:
+    # ------------------------------------------------------------------ the step
+    def _launch(self, from_host: bool) -> _Flight:
+        """Enqueue one decode step for the current rows and the copy of its results into
+        a pinned host buffer set.  ``from_host``: the input tokens are uploaded; otherwise
+        they are where the previous replay of the same rows left them."""
         B = len(self.rows)
-        if B == 0:
+        bufs = self.model._buffers(B, 1)
+        if from_host:
+            bufs.tokens.copy_(torch.tensor(self._pending_input, dtype=torch.int32))
+        want_top = any(s.want_top for s in self.rows)
+        self.model.decode_step(self.cache, B, feedback=True, sampler=self.sampler,
+                               mode=self.sampler.mode(B, want_top))
+        slot, self._slot = self._slot, self._slot ^ 1
+        h, d = self._host[slot], self.sampler
+        h["token"][:B].copy_(d.token[:B], non_blocking=True)
+        h["logprob"][:B].copy_(d.logprob[:B], non_blocking=True)
+        if want_top:
+            h["top_idx"][:B].copy_(d.top_idx[:B], non_blocking=True)
+            h["top_val"][:B].copy_(d.top_val[:B], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        return _Flight(rows=list(self.rows), slot=slot, event=ev, want_top=want_top)
+
+    def step(self) -> list[tuple[int, GenerationResponse]]:
+        if not self.rows:
+            self._flight = None
             return []
+        if not all(s.on_device for s in self.rows):
+            if self._flight is not None:  # drain the device-side chain first
+                cur, self._flight = self._flight, None
+                return self._collect(cur)
+            return self._step_host()
+        if self._flight is None:
+            if self._sampler_stale:  # steps were taken on the host meanwhile
+                for r, q in enumerate(self.rows):
+                    self.sampler.set_row(r, q.settings, q.tokens, draws=q.stream.n_gen)
+                self._sampler_stale = False
+            self._flight = self._launch(from_host=True)
+        cur = self._flight
+        # the next replay goes out before this one is read, if the same rows will still be
+        # there: nothing joined or left since the launch and nobody reaches its token limit
+        same = len(cur.rows) == len(self.rows) and all(a is b for a, b in zip(cur.rows, self.rows))
+        go_on = same and all(s.stream.n_gen + 2 <= s.stream.max_tokens for s in cur.rows)
+        self._flight = self._launch(from_host=False) if go_on else None
+        return self._collect(cur)
+
+    def _collect(self, fl: _Flight) -> list[tuple[int, GenerationResponse]]:
+        """Wait for a launched step and turn its tokens into responses."""
+        fl.event.synchronize()
+        h = self._host[fl.slot]
+        B = len(fl.rows)
+        toks = h["token"][:B].tolist()
+        lps = h["logprob"][:B].tolist()
+        now = time.perf_counter()
+        out: list[tuple[int, GenerationResponse]] = []
+        finished: list[_Seq] = []
+        for r, seq in enumerate(fl.rows):
+            cur_row = next((i for i, s in enumerate(self.rows) if s is seq), None)
+            if cur_row is None:
+                continue  # finished or cancelled while this step was in flight
+            tok = int(toks[r])
+            logprob = top = None
+            if seq.want_top:
+                logprob = float(lps[r])
+                top = seq.stream.top_items(h["top_idx"][r].tolist(), h["top_val"][r].tolist(), seq.k_top)
+            seq.tokens.append(tok)
+            self._pending_input[cur_row] = tok
+            resp = seq.stream.push(tok, now, logprob, top)
+            if seq.on_generation_token is not None:
+                seq.on_generation_token()
+            out.append((seq.uid, resp))
+            if resp.finish_reason is not None:
+                finished.append(seq)
+        self._drop_rows([i for i, s in enumerate(self.rows) if any(s is f for f in finished)])
+        if not self.rows:
+            self._flight = None
+        return out
+
+    def _step_host(self) -> list[tuple[int, GenerationResponse]]:
+        """A step with the processors and samplers of every row run on the host with torch:
+        taken only while a row's settings are outside what the sampling kernels accept."""
+        B = len(self.rows)
+        self._sampler_stale = True
         bufs = self.model._buffers(B, 1)
         bufs.tokens.copy_(torch.tensor(self._pending_input, dtype=torch.int32))
         bufs = self.model.decode_step(self.cache, B)
@@ -222,57 +332,37 @@ class ShardBatchGenerator:
         out: list[tuple[int, GenerationResponse]] = []
         finished: list[int] = []
         for r, seq in enumerate(self.rows):
-            logprobs = None
-            if seq.greedy:
-                tok = int(greedy_tokens[r])
+            logits = bufs.logits[r : r + 1].float()
+            if seq.on_device:  # its settings on the host all the same, for this step
+                procs = processors_for(seq.params, self._eos())
+                if seq.settings.temperature == 0 and not procs:
+                    tok, logprobs = int(greedy_tokens[r]), None
+                else:
+                    for p in procs:
+                        logits = p(torch.tensor(seq.tokens), logits)
+                    logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
+                    gen = torch.Generator(device=self.model.device)
+                    gen.manual_seed(seq.settings.seed + seq.stream.n_gen)
+                    tok = int(make_sampler(seq.settings.temperature, seq.settings.top_p,
+                                           seq.settings.min_p, seq.settings.top_k, gen)(logprobs)[0])
             else:
-                logits = bufs.logits[r : r + 1].float()
                 for p in seq.processors:
                     logits = p(torch.tensor(seq.tokens), logits)
                 logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
                 tok = int(seq.sampler(logprobs)[0])
-            seq.n_gen += 1
-            seq.tokens.append(tok)
-            seq.t_first = seq.t_first or now
-            seq.t_last = now
-            self._pending_input[r] = tok
-            text = self.tokenizer.decode([tok]) if self.tokenizer is not None else ""
-            seq.accumulated += text
-            finish = None
-            if tok in self._eos() and not seq.params.bench:
-                finish = "stop"
-            elif seq.n_gen >= seq.max_tokens:
-                finish = "length"
-            for s in seq.stop_sequences:
-                if s and s in seq.accumulated:
-                    cut = seq.accumulated.find(s)
-                    text = seq.accumulated[:cut][len(seq.accumulated) - len(text):]
-                    finish = "stop"
-                    break
             logprob = top = None
-            if seq.params.logprobs:
+            if seq.want_top:
                 if logprobs is None:
-                    lg = bufs.logits[r].float()
-                    logprobs = (lg - torch.logsumexp(lg, dim=-1, keepdim=True))[None]
-                logprob, top = extract_top_logprobs(
-                    logprobs[0], self.tokenizer, seq.params.top_logprobs or DEFAULT_TOP_LOGPROBS, tok)
-            stats = usage = None
-            if finish is not None:
-                dt = (seq.t_last - seq.t_first) if seq.n_gen > 1 else 0.0
-                stats = GenerationStats(
-                    prompt_tps=float(seq.prefill_tps),
-                    generation_tps=float((seq.n_gen - 1) / dt) if dt > 0 else 0.0,
-                    prompt_tokens=len(seq.prompt_tokens), generation_tokens=seq.n_gen,
-                    peak_memory_usage=int(torch.cuda.max_memory_allocated(self.model.device)),
-                    prefix_cache_hit=seq.prefix_cache_hit)
-                n_p = len(seq.prompt_tokens)
-                usage = Usage(n_p, seq.n_gen, n_p + seq.n_gen)
-                finished.append(r)
+                    logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
+                logprob, top = extract_top_logprobs(logprobs[0], self.tokenizer, seq.k_top, tok)
+            seq.tokens.append(tok)
+            self._pending_input[r] = tok
+            resp = seq.stream.push(tok, now, logprob, top)
             if seq.on_generation_token is not None:
                 seq.on_generation_token()
-            out.append((seq.uid, GenerationResponse(text=text, token=tok, logprob=logprob,
-                                                    top_logprobs=top, finish_reason=finish,
-                                                    stats=stats, usage=usage)))
+            out.append((seq.uid, resp))
+            if resp.finish_reason is not None:
+                finished.append(r)
         self._drop_rows(finished)
         return out
 
@@ -281,6 +371,8 @@ class ShardBatchGenerator:
             last = len(self.rows) - 1
             if r != last:  # keep active rows compact: move the last row into the hole
                 self.cache.copy_row(last, r)
+                if self.rows[last].on_device:
+                    self.sampler.move_row(last, r)
                 self.rows[r] = self.rows[last]
                 self._pending_input[r] = self._pending_input[last]
             self.rows.pop()
@@ -288,10 +380,13 @@ class ShardBatchGenerator:
 
     def cancel(self, uids: list[int]) -> None:
         self._drop_rows([r for r, s in enumerate(self.rows) if s.uid in set(uids)])
+        if not self.rows:
+            self._flight = None
 
     def close(self) -> None:
         self.rows.clear()
         self._pending_input.clear()
+        self._flight = None
         self.cache = None  # type: ignore[assignment]
 
 

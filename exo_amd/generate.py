@@ -202,6 +202,90 @@ def prefill(model: ShardModel, prompt_tokens, cache: ShardKVCache,
     return (n / dt if dt > 0 else 0.0), n
 
 
+# ---------------------------------------------------------------------- per-sequence host state
+
+
+class _NoTokenizer:
+    eos_token_ids: list = []
+
+    def decode(self, ids) -> str:
+        return ""
+
+
+class TokenStream:
+    """Host-side bookkeeping of one generating sequence, the part of the reference's decode
+    loop that runs after a token is known (src/exo/worker/engines/mlx/generator/
+    batch_generate.py:337-460, generate.py:735-827): streaming detokenisation, EOS / length /
+    stop-sequence finish, log-probability items, statistics and usage at the end."""
+
+    def __init__(self, tokenizer, task: TextGenerationTaskParams, eos_token_ids, max_tokens: int,
+                 n_prompt: int, prefill_tps: float, prefix_cache_hit: str, device,
+                 prompt_tokens_stat: int | None = None):
+        from .tokenizer import StreamingDetokenizer
+        self.tokenizer = tokenizer if tokenizer is not None else _NoTokenizer()
+        self.task, self.eos, self.max_tokens = task, set(eos_token_ids or []), max_tokens
+        self.n_prompt, self.prefill_tps, self.prefix_cache_hit = n_prompt, prefill_tps, prefix_cache_hit
+        self.prompt_tokens_stat = n_prompt if prompt_tokens_stat is None else prompt_tokens_stat
+        self.device = device
+        self.detok = StreamingDetokenizer(self.tokenizer)
+        self.stop_sequences = [task.stop] if isinstance(task.stop, str) else list(task.stop or [])
+        self.max_stop_len = max((len(s) for s in self.stop_sequences), default=0)
+        self.pending_stop_text = ""
+        self.n_gen = 0
+        self.t_first: float | None = None
+        self.t_last: float | None = None
+
+    def top_items(self, ids, values, k: int) -> list[TopLogprobItem]:
+        """generate.py:513-529: ids and log-probabilities (most likely first) -> items."""
+        items = []
+        for i, v in list(zip(ids, values))[:k]:
+            if i < 0 or v != v:
+                continue
+            text = self.tokenizer.decode([int(i)]) if not isinstance(self.tokenizer, _NoTokenizer) else str(int(i))
+            items.append(TopLogprobItem(token=text, logprob=float(v), bytes=list(text.encode("utf-8"))))
+        return items
+
+    def push(self, tok: int, now: float, logprob: float | None = None,
+             top_logprobs: list[TopLogprobItem] | None = None) -> GenerationResponse:
+        self.n_gen += 1
+        if self.t_first is None:
+            self.t_first = now
+        self.t_last = now
+        finish = None
+        if tok in self.eos and not self.task.bench:
+            finish = "stop"
+        elif self.n_gen >= self.max_tokens:
+            finish = "length"
+        if finish != "stop":
+            self.detok.add_token(tok)
+        if finish is not None:
+            self.detok.finalize()
+        text = self.detok.last_segment
+        self.pending_stop_text += text
+        for s in self.stop_sequences:
+            if s and s in self.pending_stop_text:
+                cut = self.pending_stop_text.find(s)
+                chunk_start = len(self.pending_stop_text) - len(text)
+                text = self.pending_stop_text[:cut][chunk_start:]
+                finish = "stop"
+                break
+        stats = usage = None
+        if finish is not None:
+            # generation_tps = (n-1)/(t_last - t_first)  (batch_generate.py:418-426)
+            dt = (self.t_last - self.t_first) if self.n_gen > 1 else 0.0
+            stats = GenerationStats(
+                prompt_tps=float(self.prefill_tps),
+                generation_tps=float((self.n_gen - 1) / dt) if dt > 0 else 0.0,
+                prompt_tokens=int(self.prompt_tokens_stat), generation_tokens=self.n_gen,
+                peak_memory_usage=int(torch.cuda.max_memory_allocated(self.device)),
+                prefix_cache_hit=self.prefix_cache_hit)
+            usage = Usage(self.n_prompt, self.n_gen, self.n_prompt + self.n_gen)
+        elif self.max_stop_len and len(self.pending_stop_text) > self.max_stop_len:
+            self.pending_stop_text = self.pending_stop_text[-self.max_stop_len:]
+        return GenerationResponse(text=text, token=tok, logprob=logprob, top_logprobs=top_logprobs,
+                                  finish_reason=finish, stats=stats, usage=usage)
+
+
 # ---------------------------------------------------------------------- generate
 
 
@@ -213,12 +297,15 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     """Sequential (batch 1) generation for a full-model shard: yields one
     GenerationResponse per token; the last carries finish_reason, stats and usage.
     ``kv_prefix_cache`` (a KVPrefixCache) is consulted and updated the way the reference's
-    mlx_generate does (generate.py:577-706): bench requests only with use_prefix_cache."""
+    mlx_generate does (generate.py:577-706): bench requests only with use_prefix_cache.
+
+    Every step is one graph replay that ends in the device sampling kernels; the host only
+    reads the sampled token (and log-probabilities when asked for).  Settings the kernels do
+    not take (penalty contexts beyond 256 tokens, more than 8 banned ids) run the processors
+    and the sampler on the host with torch instead."""
+    from .sampling import DeviceSampler, SamplerSettings
     if not (model.is_first and model.is_last):
         raise ValueError("generate() needs a shard that holds the whole model")
-    seed = task.seed or 42
-    gen = torch.Generator(device=model.device)
-    gen.manual_seed(seed)
     max_tokens = task.max_output_tokens or MAX_TOKENS
     n_prompt = len(prompt_tokens)
     if n_prompt == 0:
@@ -227,14 +314,7 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     torch.cuda.reset_peak_memory_stats(model.device)
 
     eos = list(eos_token_ids or [])
-    processors = processors_for(task, eos)
-    sampler = make_sampler(
-        temp=task.temperature if task.temperature is not None else 0.7,
-        top_p=task.top_p if task.top_p is not None else 1.0,
-        min_p=task.min_p if task.min_p is not None else 0.05,
-        top_k=task.top_k if task.top_k is not None else 0, generator=gen)
-    greedy = (task.temperature == 0) and not processors
-    stop_sequences = [task.stop] if isinstance(task.stop, str) else list(task.stop or [])
+    settings = SamplerSettings.from_task(task, eos)
 
     if task.bench and not task.use_prefix_cache:
         kv_prefix_cache = None
@@ -254,64 +334,50 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
         save_prefix_cache(kv_prefix_cache, prompt_tokens, cache, 0, prefix_hit_length,
                           matched_index, prefill_tps=prefill_tps)
 
-    # the last two prompt tokens, one forward each (generate.py:710-733)
+    # the last two prompt tokens, one forward each (generate.py:710-733); they are also all
+    # the logits processors see of the prompt (stream_generate is handed prompt[-2:])
     if len(remaining) >= 2:
         model(torch.tensor([[remaining[-2]]], dtype=torch.int32), cache, logits="none")
     tok = int(prompt_tokens[-1])
-    history = list(prompt_tokens)
-    accumulated = ""
-    t_first = t_last = None
-    for n_gen in range(1, max_tokens + 1):
-        bufs = model._buffers(1, 1)
-        bufs.tokens[0] = tok
-        bufs = model.decode_step(cache, 1)
-        if greedy:
-            tok = int(bufs.next_token[0])
-            logprobs = None
+    history = [int(t) for t in prompt_tokens[-2:]]
+    stream = TokenStream(tokenizer, task, eos, max_tokens, n_prompt, prefill_tps, prefix_cache_hit,
+                         model.device, prompt_tokens_stat=prefill_tokens + min(n_prompt, 2))
+    want_top = bool(task.logprobs)
+    k_top = task.top_logprobs or DEFAULT_TOP_LOGPROBS
+    on_device = settings.on_device() and k_top <= 20
+    if on_device:
+        ds = DeviceSampler(1, model.cfg.vocab_size, model.device)
+        ds.set_row(0, settings, history)
+        mode = ds.mode(1, want_top)
+    else:
+        gen = torch.Generator(device=model.device)
+        gen.manual_seed(settings.seed)
+        processors = processors_for(task, eos)
+        sampler = make_sampler(settings.temperature, settings.top_p, settings.min_p, settings.top_k, gen)
+    bufs = model._buffers(1, 1)
+    bufs.tokens[0] = tok
+    for _ in range(max_tokens):
+        logprob = top = None
+        if on_device:
+            model.decode_step(cache, 1, feedback=True, sampler=ds, mode=mode)
+            tok = int(ds.token[0])  # synchronises
+            if want_top:
+                logprob = float(ds.logprob[0])
+                top = stream.top_items(ds.top_idx[0].tolist(), ds.top_val[0].tolist(), k_top)
         else:
+            bufs.tokens[0] = tok
+            bufs = model.decode_step(cache, 1)
             logits = bufs.logits[0:1].float()
             for p in processors:
                 logits = p(torch.tensor(history), logits)
             logprobs = logits - torch.logsumexp(logits, dim=-1, keepdim=True)
             tok = int(sampler(logprobs)[0])
-        now = time.perf_counter()
-        t_first = t_first or now
-        t_last = now
-        history.append(tok)
-        text = tokenizer.decode([tok]) if tokenizer is not None else ""
-        accumulated += text
-        finish = None
-        if tok in eos and not task.bench:
-            finish = "stop"
-        elif n_gen >= max_tokens:
-            finish = "length"
-        for s in stop_sequences:
-            if s and s in accumulated:
-                cut = accumulated.find(s)
-                chunk_start = len(accumulated) - len(text)
-                text = accumulated[:cut][chunk_start:]
-                finish = "stop"
-                break
-        logprob = top = None
-        if task.logprobs:
-            if logprobs is None:
-                lg = bufs.logits[0].float()
-                logprobs = (lg - torch.logsumexp(lg, dim=-1, keepdim=True))[None]
-            logprob, top = extract_top_logprobs(logprobs[0], tokenizer,
-                                                task.top_logprobs or DEFAULT_TOP_LOGPROBS, tok)
-        stats = usage = None
-        if finish is not None:
-            # generation_tps = (n-1)/(t_last - t_first)  (batch_generate.py:418-426)
-            dt = (t_last - t_first) if n_gen > 1 else 0.0
-            stats = GenerationStats(
-                prompt_tps=float(prefill_tps), generation_tps=float((n_gen - 1) / dt) if dt > 0 else 0.0,
-                prompt_tokens=int(prefill_tokens + min(n_prompt, 2)), generation_tokens=n_gen,
-                peak_memory_usage=int(torch.cuda.max_memory_allocated(model.device)),
-                prefix_cache_hit=prefix_cache_hit)
-            usage = Usage(n_prompt, n_gen, n_prompt + n_gen)
+            history.append(tok)
+            if want_top:
+                logprob, top = extract_top_logprobs(logprobs[0], tokenizer, k_top, tok)
+        resp = stream.push(tok, time.perf_counter(), logprob, top)
         if on_generation_token is not None:
             on_generation_token()
-        yield GenerationResponse(text=text, token=tok, logprob=logprob, top_logprobs=top,
-                                 finish_reason=finish, stats=stats, usage=usage)
-        if finish is not None:
+        yield resp
+        if resp.finish_reason is not None:
             break

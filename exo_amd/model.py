@@ -314,20 +314,27 @@ class ShardModel:
 
     # ------------------------------------------------------------------ graph decode
     def decode_step(self, cache: ShardKVCache, B: int, use_graph: bool = True,
-                    feedback: bool = False) -> _Buffers:
+                    feedback: bool = False, sampler=None, mode: int = 0) -> _Buffers:
         """One single-token step for cache rows [0,B): reads ``bufs.tokens`` (first shard)
         or ``bufs.h``, leaves logits / next_token / lse / logprob (last shard) or the
         hidden state in the returned buffers, advances the device positions.  The kernel
         sequence is captured once per B into a HIP graph and replayed.  ``feedback``
-        (last shard, greedy): the graph also copies next_token into tokens, so steps
-        can be chained without the host."""
+        (last shard): the graph also writes the chosen token into ``tokens``, so steps
+        can be chained without the host.  ``sampler`` (a DeviceSampler, last shard): the step
+        ends in the device sampling kernels with the stages ``mode`` names instead of the
+        plain argmax; results are then in the sampler's ``token`` / ``logprob`` / ``top_*``."""
         bf = self._buffers(B, 1)
         if max(cache.offsets[:B]) + 1 > cache.max_seq:
             raise ValueError("KV cache overflow")
+        if sampler is not None and not self.is_last:
+            raise ValueError("sampling needs the shard that holds the lm_head")
 
         def body():
             out = self._run(B, 1, cache, bf, "all")
-            if self.is_last:
+            if self.is_last and sampler is not None:
+                sampler.sample(out, B, mode, feedback=bf.tokens if feedback else None,
+                               pos_inc=cache.pos[:B])
+            elif self.is_last:
                 ops.argmax_logsumexp(out, bf.next_token, bf.lse, bf.logprob, bf.argmax_ws,
                                      cache.pos[:B])
                 if feedback:
@@ -338,14 +345,16 @@ class ShardModel:
         if not use_graph:
             body()
         else:
-            key = (B, feedback)
-            if key not in self._graphs or self._graphs[key][1] is not cache:
+            key = (B, feedback, sampler is not None, mode)
+            hit = self._graphs.get(key)
+            if hit is None or hit[1] is not cache or hit[2] is not sampler:
                 # warm up outside capture (lazy module loads, attribute settings), then
                 # restore what the warm-up changed: the positions it advanced, the hidden
-                # state a later shard adds its residuals into in place, and the input
-                # tokens the feedback copy overwrote
+                # state a later shard adds its residuals into in place, the input tokens
+                # the feedback overwrote, the sampler's counters and history ring
                 saved = cache.pos.clone()
                 saved_in = bf.tokens.clone() if self.is_first else bf.h.clone()
+                saved_sampler = sampler.snapshot() if sampler is not None else None
                 s = torch.cuda.Stream()
                 s.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(s):
@@ -354,11 +363,13 @@ class ShardModel:
                 torch.cuda.synchronize()
                 cache.pos.copy_(saved)
                 (bf.tokens if self.is_first else bf.h).copy_(saved_in)
+                if sampler is not None:
+                    sampler.restore(saved_sampler)
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
                     body()
                 cache.pos.copy_(saved)
-                self._graphs[key] = (g, cache)
+                self._graphs[key] = (g, cache, sampler)
             self._graphs[key][0].replay()
         cache.advance_host(1, range(B))
         return bf

@@ -136,9 +136,9 @@ class DeviceSampler:
         self.settings: list[SamplerSettings | None] = [None] * max_rows
 
     # ---- rows
-    def set_row(self, row: int, settings: SamplerSettings, tokens_so_far) -> None:
-        """Install a request in ``row``: its parameters, the ring holding the latest
-        tokens of its prompt, a fresh draw counter."""
+    def set_row(self, row: int, settings: SamplerSettings, tokens_so_far, draws: int = 0) -> None:
+        """Install a request in ``row``: its parameters, the ring holding the latest of
+        the tokens its processors have seen so far, the draw counter."""
         if not settings.on_device():
             raise ValueError("sampler settings outside what the device kernels take")
         n = PARAMS_DTYPE.itemsize
@@ -150,7 +150,7 @@ class DeviceSampler:
             ring[a % self.hist_cap] = toks[a]  # token at absolute position a sits at a mod cap
         self.history[row].copy_(torch.from_numpy(ring))
         self.hist_len[row : row + 1].copy_(torch.tensor([len(toks)], dtype=torch.int32))
-        self.draws[row : row + 1].zero_()
+        self.draws[row : row + 1].copy_(torch.tensor([draws], dtype=torch.int32))
         self.settings[row] = settings
 
     def move_row(self, src: int, dst: int) -> None:
@@ -160,6 +160,15 @@ class DeviceSampler:
         self.hist_len[dst : dst + 1].copy_(self.hist_len[src : src + 1])
         self.draws[dst : dst + 1].copy_(self.draws[src : src + 1])
         self.settings[dst] = self.settings[src]
+
+    def snapshot(self):
+        """The state a launch advances (history ring, its fill count, the draw counters)."""
+        return self.history.clone(), self.hist_len.clone(), self.draws.clone()
+
+    def restore(self, snap) -> None:
+        self.history.copy_(snap[0])
+        self.hist_len.copy_(snap[1])
+        self.draws.copy_(snap[2])
 
     def mode(self, rows: int, want_top: bool = False) -> int:
         s = [x for x in self.settings[:rows] if x is not None]

@@ -259,6 +259,107 @@ def test_batch_generator_b2_equals_b1(ckpt, device):
     assert len(a1) == 12 and a1 == b1 and a2 == b2
 
 
+def _run_batch(gm, reqs, max_batch=4, force_host=False, stagger=0):
+    """reqs = [(params, prompt)]; returns per request the list of responses.  ``stagger``:
+    the second and later requests join after that many steps."""
+    g = ShardBatchGenerator(gm, None, max_batch=max_batch, max_seq=256)
+    out, uids = {}, []
+
+    def submit(params, prompt):
+        u = g.submit(params, prompt)
+        if force_host:  # pretend the kernels do not take this request's settings
+            from exo_amd.generate import make_sampler, processors_for
+            seq = g.rows[-1]
+            gen = torch.Generator(device=gm.device)
+            gen.manual_seed(seq.settings.seed)
+            seq.processors = processors_for(params, [])
+            seq.sampler = make_sampler(seq.settings.temperature, seq.settings.top_p, seq.settings.min_p,
+                                       seq.settings.top_k, gen)
+        uids.append(u)
+        out[u] = []
+
+    submit(*reqs[0])
+    pending = list(reqs[1:])
+    steps = 0
+    while g.has_work or pending:
+        if pending and (steps >= stagger or not g.has_work):
+            submit(*pending.pop(0))
+        for u, r in g.step():
+            out[u].append(r)
+        steps += 1
+    return [out[u] for u in uids]
+
+
+def test_device_sampling_is_per_request_and_survives_compaction(ckpt, device):
+    """Sampled requests (temperature, min-p, top-k, top-p, penalties; different seeds) give
+    the same tokens whether they run alone, together, or join a running batch, and whichever
+    row they are moved to when another request finishes: the sampling state (parameters,
+    history ring, draw counter) travels with the request."""
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    P = TextGenerationTaskParams
+    reqs = [
+        (P(model="t", max_output_tokens=5, temperature=0.9, seed=7), [int(t) for t in rng(101).integers(0, cfg.vocab_size, size=11)]),
+        (P(model="t", max_output_tokens=14, temperature=0.7, top_k=20, seed=8, repetition_penalty=1.3,
+           frequency_penalty=0.5), [int(t) for t in rng(102).integers(0, cfg.vocab_size, size=17)]),
+        (P(model="t", max_output_tokens=9, temperature=1.1, top_p=0.8, min_p=0.0, seed=9, presence_penalty=0.7),
+         [int(t) for t in rng(103).integers(0, cfg.vocab_size, size=9)]),
+    ]
+    solo = [[r.token for r in _run_batch(gm, [q])[0]] for q in reqs]
+    assert [len(s) for s in solo] == [5, 14, 9]
+    assert len(set(solo[1])) > 3  # it does sample
+    together = [[r.token for r in rs] for rs in _run_batch(gm, reqs)]
+    assert [len(t) for t in together] == [5, 14, 9]
+    # Alone, a request runs the single-row kernels, and in another row of a batch its sums
+    # are formed in another order (log-probabilities move by a few 1e-3): a draw that falls
+    # on the edge between two tokens may then go the other way, so across placements only the
+    # beginning is compared; the same placement again must give the same tokens exactly.
+    flipped = [[r.token for r in rs] for rs in _run_batch(gm, reqs[::-1])][::-1]
+    assert [len(t) for t in flipped] == [5, 14, 9]
+    assert all(t[:3] == s[:3] == f[:3] for t, s, f in zip(together, solo, flipped))
+    staggered = [[r.token for r in rs] for rs in _run_batch(gm, reqs, stagger=3)]
+    assert [len(t) for t in staggered] == [5, 14, 9] and staggered[0] == solo[0]
+    assert staggered == [[r.token for r in rs] for rs in _run_batch(gm, reqs, stagger=3)]
+    again = [[r.token for r in rs] for rs in _run_batch(gm, reqs)]
+    assert again == together  # same seeds, same tokens
+    other_seed = _run_batch(gm, [(P(model="t", max_output_tokens=14, temperature=0.7, top_k=20, seed=88,
+                                    repetition_penalty=1.3, frequency_penalty=0.5), reqs[1][1])])[0]
+    assert [r.token for r in other_seed] != solo[1]
+    # sequential generate() runs the same kernels with the same seed
+    assert [r.token for r in generate(gm, None, reqs[1][0], reqs[1][1])] == solo[1]
+
+
+def test_device_logprobs_match_host_path(ckpt, device):
+    """Greedy requests with log-probabilities: the device step (top-20 table, selected
+    log-probability) against the same requests stepped with the processors and torch.topk on
+    the host; a request whose settings the kernels do not take switches the whole batch to the
+    host for as long as it runs and the others carry on unchanged."""
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    P = TextGenerationTaskParams
+    reqs = [(P(model="t", max_output_tokens=6, temperature=0.0, logprobs=True, top_logprobs=5),
+             [int(t) for t in rng(111).integers(0, cfg.vocab_size, size=13)]),
+            (P(model="t", max_output_tokens=9, temperature=0.0, logprobs=True, top_logprobs=20,
+               repetition_penalty=1.5), [int(t) for t in rng(112).integers(0, cfg.vocab_size, size=8)])]
+    dev = _run_batch(gm, reqs)
+    host = _run_batch(gm, reqs, force_host=True)
+    for d, h in zip(dev, host):
+        assert [r.token for r in d] == [r.token for r in h]
+        assert len(d[0].top_logprobs) == len(h[0].top_logprobs)
+        for rd, rh in zip(d, h):
+            assert abs(rd.logprob - rh.logprob) < 2e-2  # a penalised logit is rounded to bf16 on the device
+            # bf16 processors on the device, float32 on the host: the order of near-equal
+            # entries may differ, the values may not
+            np.testing.assert_allclose([i.logprob for i in rd.top_logprobs],
+                                       [i.logprob for i in rh.top_logprobs], atol=2e-2)
+            assert rd.top_logprobs[0].token == rh.top_logprobs[0].token
+        assert d[-1].finish_reason == "length" and d[-1].stats.generation_tokens == len(d)
+    # a context the history ring does not hold: that request samples on the host
+    wide = (P(model="t", max_output_tokens=4, temperature=0.0, repetition_penalty=1.2,
+              repetition_context_size=1000), reqs[0][1])
+    mixed = _run_batch(gm, [reqs[1], wide], stagger=2)
+    assert [r.token for r in mixed[0]] == [r.token for r in dev[1]]
+    assert len(mixed[1]) == 4
+
+
 def test_batch_generator_slot_compaction_and_cancel(ckpt, device):
     cfg, gm = ckpt["cfg"], ckpt["model"]
     short = TextGenerationTaskParams(model="tiny", max_output_tokens=3, temperature=0.0)

@@ -461,3 +461,79 @@ def test_logits_processors():
     procs = processors_for(p, [3])
     assert len(procs) == 3 and procs[0](None, logits)[0, 3] == -1e9
     assert processors_for(TextGenerationTaskParams(model="m", bench=True), []) == []
+
+
+# ------------------------------------------------------------------ detokeniser, token stream
+
+
+def _byte_level_tokenizer():
+    """A byte-level BPE without merges: one id per UTF-8 byte, decoded by the ByteLevel
+    decoder - the smallest tokenizer in which a character is split over several ids."""
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+    from exo_amd.tokenizer import HFTokenizer
+    vocab = {ch: i for i, ch in enumerate(sorted(pre_tokenizers.ByteLevel.alphabet()))}
+    tok = Tokenizer(models.BPE(vocab=vocab, merges=[]))
+    tok.pre_tokenizer = pre_tokenizers.ByteLevel(add_prefix_space=False)
+    tok.decoder = decoders.ByteLevel()
+    return HFTokenizer(tok, [])
+
+
+def test_streaming_detokenizer_holds_back_incomplete_characters():
+    from exo_amd.tokenizer import StreamingDetokenizer
+    t = _byte_level_tokenizer()
+    text = "h\u00e9llo \u4e16\u754c \U0001f600!"
+    ids = t.encode(text)
+    assert len(ids) > len(text)                       # multi-byte characters span ids
+    assert "\ufffd" in "".join(t.decode([i]) for i in ids)  # one by one they would be garbled
+    d = StreamingDetokenizer(t)
+    segs = []
+    for i in ids:
+        d.add_token(i)
+        segs.append(d.last_segment)
+    d.finalize()
+    segs.append(d.last_segment)
+    assert "".join(segs) == text and not any("\ufffd" in s for s in segs)
+    assert segs[1] == "" and segs[2] == "\u00e9"     # the first byte of the e-acute is held back
+    # a sequence cut inside a character: finalize releases what there is
+    d = StreamingDetokenizer(t)
+    for i in ids[:2]:
+        d.add_token(i)
+    assert d.last_segment == "h"
+    d.finalize()
+    assert d.last_segment == "\ufffd"
+
+
+def test_token_stream_finish_reasons_and_stop_sequences():
+    from exo_amd.generate import TokenStream
+    t = _byte_level_tokenizer()
+    ids = t.encode("ab\u00e9cd STOP tail")
+    task = TextGenerationTaskParams(model="m", stop=["STOP"])
+    ts = TokenStream(t, task, [], 100, 5, 10.0, "none", "cpu")
+    out = []
+    with pytest.MonkeyPatch.context() as mp:
+        mp.setattr(torch.cuda, "max_memory_allocated", lambda d=None: 0)
+        for k, i in enumerate(ids):
+            r = ts.push(i, float(k))
+            out.append(r)
+            if r.finish_reason:
+                break
+    # as in the reference (batch_generate.py:371-385) only the chunk that completes the stop
+    # sequence is trimmed: the characters of it that earlier chunks carried are already out
+    assert "".join(r.text for r in out) == "ab\u00e9cd STO" and out[-1].finish_reason == "stop"
+    assert out[-1].text == "" and out[-1].token == ids[len(out) - 1]
+    assert out[-1].usage.completion_tokens == len(out) and out[-1].stats.generation_tokens == len(out)
+    assert out[-1].stats.generation_tps == pytest.approx((len(out) - 1) / (len(out) - 1.0))
+    # EOS: the token is not detokenised; length: the last token is
+    eos = t.encode("z")[0]
+    with pytest.MonkeyPatch.context() as mp:
+        mp.setattr(torch.cuda, "max_memory_allocated", lambda d=None: 0)
+        ts = TokenStream(t, TextGenerationTaskParams(model="m"), [eos], 100, 5, 10.0, "none", "cpu")
+        assert ts.push(t.encode("q")[0], 0.0).text == "q"
+        r = ts.push(eos, 1.0)
+        assert r.finish_reason == "stop" and r.text == ""
+        ts = TokenStream(t, TextGenerationTaskParams(model="m", bench=True), [eos], 2, 5, 10.0, "none", "cpu")
+        assert ts.push(eos, 0.0).finish_reason is None   # bench mode: EOS does not stop
+        r = ts.push(t.encode("q")[0], 1.0)
+        assert r.finish_reason == "length" and r.text == "q"
+        items = ts.top_items([t.encode("a")[0], -1, t.encode("b")[0]], [-0.5, float("nan"), -1.5], 5)
+        assert [(i.token, i.logprob) for i in items] == [("a", -0.5), ("b", -1.5)]
