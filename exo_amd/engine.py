@@ -17,6 +17,7 @@ from __future__ import annotations
 import logging
 import os
 import time
+import uuid
 from abc import ABC, abstractmethod
 from collections import deque
 from collections.abc import Callable, Generator, Iterable
@@ -46,6 +47,7 @@ from .types import (
 )
 
 EXO_MAX_CONCURRENT_REQUESTS = int(os.environ.get("EXO_MAX_CONCURRENT_REQUESTS", "8"))
+REMOTE_PREFILL_MIN_TOKENS = 1000  # src/exo/worker/engines/mlx/generator/batch_generate.py:62
 CANCEL_ALL_TASKS = "CANCEL_ALL_TASKS"
 
 
@@ -201,7 +203,8 @@ class ShardBatchGenerator:
                 on_prefill_progress(done, total)
 
         try:
-            tps, n = prefill(self.model, remaining[:-1], self.cache, progress, row=row)
+            tps, n = self._prefill_row(task_params, toks, remaining, prefix_hit_length, row, progress,
+                                       on_prefill_progress)
         except PrefillCancelled:
             self.cache.reset(rows=range(row, row + 1))
             raise
@@ -240,6 +243,44 @@ class ShardBatchGenerator:
         self.rows.append(seq)
         self._pending_input.append(toks[-1])
         return seq.uid
+
+    def _prefill_row(self, task_params, toks, remaining, prefix_hit_length, row, progress,
+                     on_prefill_progress) -> tuple[float, int]:
+        """Fill row ``row`` up to the last-but-one prompt position: locally, or - for a long
+        uncached remainder when the task names a prefill server - by fetching the KV over the
+        wire (batch_generate.py:205-246; a failed fetch falls back to the local path).
+
+        Two departures from the reference's call, both where it contradicts its own server
+        (disaggregated/serve.py:43-58): the whole prompt is sent, not only the uncached
+        remainder, because the server prefills ``token_ids`` as a complete prompt and
+        ``start_pos`` only says which positions to ship; and whatever positions the reply
+        leaves short of N-2 (the server stops a few positions early) are computed here, so
+        the cache is complete whichever way it was filled."""
+        use_remote = (len(remaining) > REMOTE_PREFILL_MIN_TOKENS
+                      and task_params.prefill_endpoint is not None)
+        if use_remote:
+            from .disaggregated import remote_prefill
+            t0 = time.perf_counter()
+            try:
+                remote_prefill(toks[:-1], self.cache, on_prefill_progress,
+                               endpoint=task_params.prefill_endpoint, request_id=str(uuid.uuid4()),
+                               model_id=str(task_params.model), start_pos=prefix_hit_length, row=row)
+                have, need = self.cache.offsets[row], len(toks) - 2
+                if have > need:
+                    self.cache.trim(have - need, rows=range(row, row + 1))
+                elif have < need:
+                    self.model(torch.tensor([toks[have:need]], dtype=torch.int32), self.cache,
+                               logits="none", rows=slice(row, row + 1))
+                torch.cuda.synchronize()
+                n = len(remaining) - 1
+                return n / max(time.perf_counter() - t0, 1e-3), n
+            except PrefillCancelled:
+                raise
+            except Exception:
+                logger.warning("remote prefill failed, falling back to local prefill", exc_info=True)
+                self.cache.offsets[row] = prefix_hit_length
+                self.cache.sync_pos()
+        return prefill(self.model, remaining[:-1], self.cache, progress, row=row)
 
     # ------------------------------------------------------------------ the step
     def _launch(self, from_host: bool) -> _Flight:

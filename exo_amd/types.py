@@ -122,6 +122,7 @@ class TextGenerationTaskParams:
     repetition_context_size: int | None = None
     presence_penalty: float | None = None
     frequency_penalty: float | None = None
+    prefill_endpoint: str | None = None  # "host:port" of a disaggregated-prefill server
 
 
 @dataclass

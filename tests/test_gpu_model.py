@@ -639,3 +639,70 @@ def test_serve_prefill_over_tcp_then_decode(ckpt, device):
         got.append(tok)
     assert got == want
     eng.close()
+
+
+def test_submit_fetches_long_prompts_from_a_prefill_server(ckpt, device):
+    """A task that names a prefill endpoint and has more than 1000 uncached prompt tokens is
+    prefilled over the wire (src/exo/worker/engines/mlx/generator/batch_generate.py:205-246):
+    the generated tokens equal those of a local prefill, the server was asked once, short
+    prompts stay local, and a dead endpoint falls back to the local path."""
+    from exo_amd import disaggregated as D
+    from exo_amd.engine import BatchGenerator
+    from exo_amd.prefix_cache import KVPrefixCache
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    prompt = [int(t) for t in rng(121).integers(0, cfg.vocab_size, size=1203)]
+    P = TextGenerationTaskParams
+    local = [r.token for r in _run_batch_seq(gm, P(model="tiny", max_output_tokens=6, temperature=0.0), prompt)]
+    server_engine = BatchGenerator(model=gm, tokenizer=None, model_id="tiny", max_seq=2048,
+                                   kv_prefix_cache=KVPrefixCache(None, device))
+    served = []
+
+    def resolve(job, wfile):
+        server_engine.serve_prefill(job, wfile)
+        served.append((len(job.token_ids), job.start_pos))
+        return True
+
+    srv = D.PrefillServer(resolve, "127.0.0.1", 0)
+    try:
+        ep = f"127.0.0.1:{srv.server_address[1]}"
+        remote = _run_batch_seq(gm, P(model="tiny", max_output_tokens=6, temperature=0.0, prefill_endpoint=ep), prompt)
+        for _ in range(500):
+            if served:
+                break
+            time.sleep(0.01)
+        # the few positions the server's reply stops short of are computed here as a short
+        # chunk (GEMV kernels) where the local path has them inside its one long GEMM chunk:
+        # last-bit differences there may turn a near-tie, so the tokens are compared at the
+        # start and the shipped KV bit for bit
+        assert [r.token for r in remote][:3] == local[:3] and served == [(len(prompt) - 1, 0)]
+        assert remote[-1].stats.prompt_tps > 0
+        ga, gb = ShardBatchGenerator(gm, None, 1, 2048), ShardBatchGenerator(gm, None, 1, 2048)
+        ga.submit(P(model="tiny", max_output_tokens=2, temperature=0.0), prompt)
+        gb.submit(P(model="tiny", max_output_tokens=2, temperature=0.0, prefill_endpoint=ep), prompt)
+        n_ship = len(prompt) - 1 - 3
+        assert ga.cache.offsets[0] == gb.cache.offsets[0] == len(prompt) - 1
+        for li in range(len(ga.cache)):
+            assert torch.equal(ga.cache.k[li][0, :, :n_ship], gb.cache.k[li][0, :, :n_ship])
+            assert torch.equal(ga.cache.v[li][0, :, :n_ship], gb.cache.v[li][0, :, :n_ship])
+        # (layer 0's keys of the locally filled positions depend on the tokens alone)
+        assert_close_stat(n_f32(gb.cache.k[0][0, :, n_ship:len(prompt) - 2]),
+                          n_f32(ga.cache.k[0][0, :, n_ship:len(prompt) - 2]), what="gap positions, layer 0 keys")
+        short = _run_batch_seq(gm, P(model="tiny", max_output_tokens=3, temperature=0.0, prefill_endpoint=ep), prompt[:50])
+        assert len(short) == 3 and len(served) == 2  # 50 tokens: not worth the trip (2 = the fetches above)
+    finally:
+        srv.stop()
+    dead = _run_batch_seq(gm, P(model="tiny", max_output_tokens=6, temperature=0.0,
+                                prefill_endpoint="127.0.0.1:9"), prompt)
+    assert [r.token for r in dead] == local
+    server_engine.close()
+    ga.close()
+    gb.close()
+
+
+def _run_batch_seq(gm, params, prompt):
+    g = ShardBatchGenerator(gm, None, max_batch=2, max_seq=2048)
+    g.submit(params, prompt)
+    out = []
+    while g.has_work:
+        out += [r for _, r in g.step()]
+    return out
