@@ -24,8 +24,18 @@
 //  * grouped mode (MoE prefill): blockIdx.y is a tile of one expert's sorted rows.
 //  * up to 128 rows and few column tiles: blockIdx.z splits K; float32 partial tiles and a
 //    small reduce launch.
+//  * up to 32 rows (64 on matrices of 8192 rows or more): the four waves sit side by side on
+//    a (32 or 64) x 256 tile, so no weight row is dequantised twice, and K is split until the
+//    launch has up to two workgroups per CU (14336x4096 4-bit at 32 rows: 31 -> 21 us,
+//    4096x14336: 32.5 -> 23 us; at 96 rows and more the 128-row tile is level or faster).
+//    Without the arithmetic that launch still takes 3/4 of its time, and re-reading one
+//    weight block from L2 changes nothing: a wave instruction that touches 32 rows x 32 bytes
+//    is bound by line requests, not by bytes.  A ring of eight register stages (every load of
+//    a K range requested before the first product) was slower than two stages.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
+
+#include <algorithm>
 
 namespace {
 
@@ -51,6 +61,7 @@ struct QmmParams {
   // float32 partial tile; qmm_reduce_kernel adds them
   int ksplit, kc;
   float* part;  // [ksplit][M][N]
+  bool wide = false;  // host only: launch the (32*MI) x 256 tile (up to 128 rows)
   // pair mode (Llama MLP, prefill): w/s/b is the gate matrix, w2/s2/b2 the up matrix, both
   // [N, K]; y[M,N] = silu(x gate^T) * (x up^T) with both projections rounded to bf16 first
   const uint32_t* w2 = nullptr;
@@ -146,18 +157,24 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // PAIR: the workgroup's 128 weight rows are 64 rows of the gate matrix and the same 64 rows
 // of the up matrix - a wave's two column tiles are (gate, up) of the same 32 output columns,
 // so the SwiGLU happens in the epilogue and neither projection is written to memory.
-template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false>
+// WIDE (inputs of up to 64 rows): the four waves sit side by side - the workgroup tile is
+// (32*MI) x 256, every wave owns 64 weight rows of its own, so nothing is dequantised twice;
+// blockIdx.z always owns a K range and the tile leaves as a float32 partial.
+template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false,
+          bool WIDE = false>
 __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
+  static_assert(!WIDE || (!GROUPED && !PAIR), "the wide tile is for the plain GEMM");
   constexpr int kThreads = 256;
-  constexpr int BM = 64 * MI, BN = PAIR ? 64 : 128;  // BN: output columns per workgroup
-  constexpr int WN = PAIR ? 32 : 64;                 // output columns per wave
+  constexpr int BM = WIDE ? 32 * MI : 64 * MI;
+  constexpr int BN = PAIR ? 64 : WIDE ? 256 : 128;  // output columns per workgroup
+  constexpr int WN = PAIR ? 32 : 64;                // output columns per wave
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * BN;
-  const int wm = (wave >> 1) * (32 * MI), wn = (wave & 1) * WN;
+  const int wm = WIDE ? 0 : (wave >> 1) * (32 * MI), wn = WIDE ? wave * WN : (wave & 1) * WN;
   const int G = p.K >> 6;
   const int wpr = p.K * BITS / 32;
   int m0 = blockIdx.y * BM, m_end = p.M;
@@ -292,7 +309,8 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     // seven vector instructions of the same wave.  The order is pinned slot by slot (one
     // MFMA, one register of the next B operand, one LDS read) with scheduling barriers;
     // left alone, the compiler clumps the MFMAs behind all the vector work.
-    static_assert(MI == 2 || MI == 4, "eight operand registers are spread over 2*MI slots");
+    static_assert(MI == 2 || MI == 4 || (WIDE && MI == 1),
+                  "eight operand registers are spread over 2*MI slots");
     const char* arow = tiles + buf * TILE_BYTES + (wm + frow) * 128;
     bf16x8_t a[2][MI];
     uint4 bq[2][2];
@@ -374,7 +392,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     buf ^= 1;
   }
 
-  if (!GROUPED && !PAIR && p.ksplit > 1) {
+  if (WIDE || (!GROUPED && !PAIR && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel)
     float* mine = p.part + (size_t)blockIdx.z * part_stride(p.M, p.N);
@@ -477,7 +495,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   }
 }
 
-constexpr int kQmmMaxSplit = 8;
+constexpr int kQmmMaxSplit = 16;  // K ranges the reduce kernel adds
 
 // y = bf16(sum over the K ranges, in order) (+ residual): four outputs per thread
 __global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict__ part,
@@ -536,7 +554,7 @@ void plan_split(int M, int N, int K, bool have_ws, int* ksplit, int* kc) {
   const int tiles = exo_ceil_div(N, 128) * exo_ceil_div(M, 128);
   if (tiles >= kQmmSplitTiles) return;
   int ks = 1;
-  while (ks < kQmmMaxSplit && tiles * ks < 256 && K / (ks * 2) >= 512) ks *= 2;
+  while (ks < 8 && tiles * ks < 256 && K / (ks * 2) >= 512) ks *= 2;
   if (ks == 1) return;
   int c = exo_ceil_div(K, ks);
   c = (c + 255) / 256 * 256;
@@ -544,9 +562,46 @@ void plan_split(int M, int N, int K, bool have_ws, int* ksplit, int* kc) {
   *ksplit = exo_ceil_div(K, c);
 }
 
+// The wide tile (no weight row dequantised twice), K split so that the launch has up to two
+// workgroups per CU.  Matrices of more than kQmmWideMaxN rows have enough column tiles for
+// the 128-column tile without partials.
+constexpr int kQmmWideMaxN = 32768;
+
+int wide_max_split(int N) {
+  const int tiles = exo_ceil_div(N, 256);
+  int ks = 1;
+  while (ks < kQmmMaxSplit && tiles * ks * 2 <= 512) ks *= 2;
+  return ks;
+}
+
+bool plan_wide(int M, int N, int K, const QmmParams& p, bool have_ws, int* ksplit, int* kc) {
+  if (!have_ws || M > 64 || (M > 32 && N < 8192) || N > kQmmWideMaxN || K % 256 != 0) return false;
+  if ((((uintptr_t)p.s | (uintptr_t)p.b) & 7) != 0) return false;
+  const int cap = wide_max_split(N);
+  int ks = 1;
+  while (ks < cap && K / (ks * 2) >= 256) ks *= 2;
+  int c = exo_ceil_div(K, ks);
+  c = (c + 255) / 256 * 256;
+  *kc = c;
+  *ksplit = exo_ceil_div(K, c);
+  return true;
+}
+
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
+  if (p.wide) {
+    const dim3 g(exo_ceil_div(N, 256), 1, p.ksplit);
+    if (M <= 32)
+      qmm_kernel<BITS, 1, false, true, false, true><<<g, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 2, false, true, false, true><<<g, 256, 0, st>>>(p);
+    const int64_t total = (int64_t)M * N;
+    const int vec_ok = (((uintptr_t)p.y | (uintptr_t)p.residual) & 7) == 0;
+    qmm_reduce_kernel<<<dim3(exo_ceil_div(exo_ceil_div(total, 4), 256)), 256, 0, st>>>(
+        p.part, p.residual, p.y, total, (int64_t)part_stride(M, N), p.ksplit, vec_ok);
+    return;
+  }
   // taller inputs: 256-row tiles halve the dequantisation work and the LDS reads per output
   const dim3 g2(exo_ceil_div(N, 128), exo_ceil_div(M, 128), p.ksplit), g4(exo_ceil_div(N, 128), exo_ceil_div(M, 256));
   const bool sb4 = p.K % 256 == 0 && (((uintptr_t)p.s | (uintptr_t)p.b) & 7) == 0;
@@ -778,8 +833,10 @@ extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const u
 
 extern "C" int64_t exo_qmm_workspace(int M, int N) {
   if (M <= 0 || N <= 0) return 0;
-  if ((int64_t)exo_ceil_div(N, 128) * exo_ceil_div(M, 128) >= kQmmSplitTiles) return 0;
-  return (int64_t)kQmmMaxSplit * (int64_t)part_stride(M, N) * 4;
+  int64_t ranges = 0;
+  if ((int64_t)exo_ceil_div(N, 128) * exo_ceil_div(M, 128) < kQmmSplitTiles) ranges = 8;
+  if (M <= 64 && N <= kQmmWideMaxN) ranges = std::max<int64_t>(ranges, wide_max_split(N));
+  return ranges * (int64_t)part_stride(M, N) * 4;
 }
 
 extern "C" int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
@@ -809,7 +866,8 @@ extern "C" int exo_qmm_ws(const uint16_t* x, const uint32_t* w, const uint16_t* 
   p.tiles = nullptr;
   p.x_div = 1;
   p.w_stride = p.s_stride = 0;
-  plan_split(M, N, K, workspace != nullptr, &p.ksplit, &p.kc);
+  p.wide = plan_wide(M, N, K, p, workspace != nullptr, &p.ksplit, &p.kc);
+  if (!p.wide) plan_split(M, N, K, workspace != nullptr, &p.ksplit, &p.kc);
   p.part = reinterpret_cast<float*>(workspace);
   EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm: M=%d too large", M);
   EXO_REQUIRE((int64_t)M * K < (1ll << 31), "exo_qmm: M*K=%lld exceeds 32-bit byte offsets",
