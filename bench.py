@@ -330,7 +330,7 @@ def qmatmul_sweep(args):
                 sc = (torch.rand(N, K // 64, device=dev, generator=g) * 0.01).bfloat16()
                 bi = (torch.rand(N, K // 64, device=dev, generator=g) * -0.08).bfloat16()
                 ws.append(QuantizedWeight(w, sc, bi, bits))
-            for M in (1, 4, 16, 128, 2048):
+            for M in (1, 4, 16, 32, 64, 128, 2048):
                 if M >= 128 and N * M * 2 > (1 << 30):
                     continue  # 128256 x 2048 outputs: not a shape the models produce
                 x = torch.randn(M, K, device=dev, generator=g).bfloat16()
@@ -367,7 +367,7 @@ def qmatmul_sweep(args):
         "n_gpus": 1, "steps": len(rows), "warmup": 1, "ms_per_step": dom["us"] * 1e-3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: quantised matmul sweep, bits {4,8} x 5 shapes x M {1,4,16,128,2048}; "
+        "config": {"workload": "configs[1]: quantised matmul sweep, bits {4,8} x 5 shapes x M {1,4,16,32,64,128,2048}; "
                                "value = 4-bit 14336x4096 at M=1"},
         "roofline": {"bound": "hbm", "achieved": dom["GBps"], "peak": 8000.0, "unit": "GB/s",
                      "frac": dom["GBps"] / 8000.0, "traffic": None},
