@@ -41,6 +41,8 @@ struct QmvParams {
   // gather (MoE) mode: blockIdx.y = (token, slot) pair; expert = idx[pair]
   const int32_t* idx;  // [T*topk] or null
   int E, topk, x_rows;
+  // the same with ONE matrix: blockIdx.y = row of x and of y (topk = x_rows = 1, idx null)
+  int each_row;
   // fused RMSNorm of the input rows: x <- bf16(x * rsqrt(mean(x^2) + eps) * norm_w)
   const bf16_t* norm_w;  // [K] or null
   float eps;
@@ -298,12 +300,14 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
   size_t ew = 0, eg = 0;
-  if (p.idx) {
+  if (p.idx || p.each_row) {
     const int pair = blockIdx.y;
-    int e = p.idx[pair];
-    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
-    ew = (size_t)e * p.N * p.wpr;
-    eg = (size_t)e * p.N * G;
+    if (p.idx) {
+      int e = p.idx[pair];
+      e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    }
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
     yout += (size_t)pair * p.N;
   }
@@ -501,12 +505,14 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
   size_t ew = 0, eg = 0;
-  if (p.idx) {
+  if (p.idx || p.each_row) {
     const int pair = blockIdx.y;
-    int e = p.idx[pair];
-    e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
-    ew = (size_t)e * p.N * p.wpr;
-    eg = (size_t)e * p.N * G;
+    if (p.idx) {
+      int e = p.idx[pair];
+      e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    }
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
     yout += (size_t)pair * p.N;
   }
@@ -1108,7 +1114,8 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
 
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
-  if (MT == 1 && NMAT == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.norm_w && !p.idx && p.M == 1) {
+  if (MT == 1 && NMAT == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.norm_w && !p.idx && !p.each_row &&
+      p.M == 1) {
     // measured against the row kernel: ahead at 14 units per row (8-bit, K = 14336: 17.0
     // vs 18.3 us for 4096 rows), level at 7 and 8, behind at 4
     if (pl.iters == 14) return launch_ksplit<BITS, 14>(p, st);
@@ -1143,6 +1150,7 @@ int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
 struct Gather {
   const int32_t* idx = nullptr;
   int pairs = 1, E = 0, topk = 1, x_rows = 1;
+  bool each_row = false;  // no indices: `pairs` rows of x against the one matrix
 };
 
 template <int NMAT>
@@ -1155,7 +1163,7 @@ int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const*
   int m0 = 0;
   while (m0 < M) {
     int mt = (M - m0 >= 4) ? 4 : ((M - m0 >= 2) ? 2 : 1);
-    if (ga.idx) mt = 1;
+    if (ga.idx || ga.each_row) mt = 1;
     Plan pl;
     for (;;) {
       if (!make_plan(N, K, bits, mt, &pl)) {
@@ -1191,9 +1199,10 @@ int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const*
     p.E = ga.E;
     p.topk = ga.topk;
     p.x_rows = ga.x_rows;
+    p.each_row = ga.each_row ? 1 : 0;
     p.norm_w = norm_w;
     p.eps = eps;
-    const int pairs = ga.idx ? ga.pairs : 1;
+    const int pairs = (ga.idx || ga.each_row) ? ga.pairs : 1;
     int rc;
     if (bits == 4) {
       rc = mt == 4   ? launch_one<4, 4, NMAT>(p, pl, pairs, st)
@@ -1234,6 +1243,15 @@ int check_common(const char* name, int M, int N, int K, int bits, int group_size
 // the matrix cores win.
 inline bool two_rows_on_dot2(int M, int K) { return M == 2 && K <= 8192; }
 
+// A matrix this small (a MoE router: 128 x 2048 4-bit = 128 KiB) under 2...16 rows is a
+// latency-bound launch: one set of single-row workgroups per row (blockIdx.y), each reading
+// the matrix from L2, finishes in the time of the one-row launch (3.5 us), where the
+// matrix-core tile with its staging of all rows and its K merge takes 6.8 us at four rows.
+#ifndef EXO_EACH_ROW_MAX_BYTES
+#define EXO_EACH_ROW_MAX_BYTES (1 << 20)
+#endif
+constexpr int64_t kEachRowMaxBytes = EXO_EACH_ROW_MAX_BYTES;
+
 }  // namespace
 
 extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
@@ -1251,6 +1269,19 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
   if (rc) return rc;
   EXO_REQUIRE(x && w && scales && biases && y, "exo_qmv: null pointer");
   if (M == 0) return EXO_OK;
+  if (M >= 2 && !residual && (int64_t)N * K * bits / 8 <= kEachRowMaxBytes) {
+    const uint32_t* ws[1] = {w};
+    const bf16_t* ss[1] = {scales};
+    const bf16_t* bs[1] = {biases};
+    Gather ga;
+    ga.each_row = true;
+    ga.pairs = M;
+    rc = qmv_dispatch<1>(x, ws, ss, bs, nullptr, y, 1, N, K, bits, (hipStream_t)stream, "exo_qmv",
+                         ga, norm_weight, eps);
+    if (rc) return rc;
+    EXO_CHECK_LAUNCH("exo_qmv");
+    return EXO_OK;
+  }
   // two or more rows: the matrix-core GEMV streams W once per tile of up to 16 rows
   // (with a workspace; without one a tile is as many rows as the LDS holds whole)
   int cap = (M >= 2 && !two_rows_on_dot2(M, K)) ? exo_qmv_mfma_max_rows(K, bits) : 0;

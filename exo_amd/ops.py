@@ -207,6 +207,10 @@ def quantized_matmul(
     # 9..16 rows: the matrix-core GEMV needs its 16-row variant there, which the split-K
     # GEMM matches or beats for 8-bit weights (measured on the Llama-8B shapes)
     gemm_rows = M > 8 and norm_weight is None and qw.bits == 8
+    # a matrix of up to 1 MiB without a residual (a MoE router): the library runs its
+    # single-row kernel once per row in one launch, whatever the bit width
+    if residual is None and qw.N * K * qw.bits // 8 <= (1 << 20):
+        gemm_rows = False
     if 2 <= M <= QMV_MAX_M and not gemm_rows:
         ws = qmv_workspace(qw.N, x.device)
         check(

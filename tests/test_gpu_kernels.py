@@ -136,14 +136,34 @@ def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
         fused = ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
         sep = ops.swiglu(ops.quantized_matmul(x, g, norm_weight=nw, eps=1e-5),
                          ops.quantized_matmul(x, u, norm_weight=nw, eps=1e-5))
-        if nw is None and M > 8 and bits == 8:
-            # these single projections take the split-K GEMM (another summation order)
-            assert_close(n_f32(fused), n_f32(sep), what="fused pair vs GEMM projections")
+        if (nw is None and M > 8 and bits == 8) or N * K * bits // 8 <= (1 << 20):
+            # these single projections take the split-K GEMM, or (a matrix of up to 1 MiB)
+            # one single-row launch set per row: another summation order
+            assert_close(n_f32(fused), n_f32(sep), what="fused pair vs separate projections")
         else:
             assert torch.equal(fused.view(torch.int16), sep.view(torch.int16))
     # the shared workspace is left clean for a launch of another shape
     y = ops.quantized_matmul(x[:2], g)
     assert torch.equal(y.view(torch.int16), ops.quantized_matmul(x[:2], g).view(torch.int16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [2, 4, 8, 16])
+@pytest.mark.parametrize("N,K", [(128, 2048), (60, 4096), (256, 768)])
+def test_small_matrix_rows_equal_single_row_launches(device, bits, M, N, K):
+    """A matrix of up to 1 MiB (a MoE router) under 2..16 rows runs the single-row kernel once
+    per row in one launch: every row equals its own single-row launch bit for bit, with and
+    without the fused RMSNorm, and the oracle within tolerance."""
+    trip = rand_quantized(N, K, bits, seed=N + K)
+    x = rand_bf16((M, K), seed=M + 7, scale=2.0)
+    qw, xt = t_qw(trip, bits, device), t_bf16(x, device)
+    w = t_bf16(affine.bf16_round(rand_bf16((K,), seed=6) * 0.1 + 1.0), device)
+    for nw in (None, w):
+        got = ops.quantized_matmul(xt, qw, norm_weight=nw, eps=1e-5)
+        for r in range(M):
+            one = ops.quantized_matmul(xt[r:r + 1], qw, norm_weight=nw, eps=1e-5)
+            assert torch.equal(got[r:r + 1].view(torch.int16), one.view(torch.int16)), (r, nw is None)
+    assert_close(n_f32(ops.quantized_matmul(xt, qw)), affine.qmm(x, *trip, 64, bits), what="rows of a small matrix")
 
 
 @pytest.mark.parametrize("bits", [4, 8])

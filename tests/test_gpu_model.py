@@ -287,6 +287,26 @@ def _run_batch(gm, reqs, max_batch=4, force_host=False, stagger=0):
         for u, r in g.step():
             out[u].append(r)
         steps += 1
+        if not force_host and g.rows and all(q.on_device for q in g.rows):
+            # the device-side state of every row belongs to the request that sits there now:
+            # its seed, and a draw counter at the request's token count (or one step ahead
+            # of it, while the next replay is in flight)
+            from exo_amd.sampling import PARAMS_DTYPE
+            torch.cuda.synchronize()
+            n = len(g.rows)
+            recs = np.frombuffer(g.sampler.params[: n * PARAMS_DTYPE.itemsize].cpu().numpy().tobytes(), PARAMS_DTYPE)
+            draws = g.sampler.draws[:n].tolist()
+            hist_len, ring = g.sampler.hist_len[:n].tolist(), g.sampler.history[:n].tolist()
+            for r, q in enumerate(g.rows):
+                assert int(recs[r]["seed_lo"]) == q.settings.seed & 0xFFFFFFFF, (steps, r)
+                if g._sampler_stale:
+                    continue
+                if q.settings.draws:
+                    assert draws[r] - q.stream.n_gen in (0, 1), (steps, r, draws[r], q.stream.n_gen)
+                toks, cap = [int(t) for t in q.tokens], g.sampler.hist_cap
+                assert hist_len[r] - len(toks) in (0, 1), (steps, r, hist_len[r], len(toks))
+                for a in range(max(0, len(toks) - cap + 1), len(toks)):
+                    assert ring[r][a % cap] == toks[a], (steps, r, a)
     return [out[u] for u in uids]
 
 
@@ -311,13 +331,14 @@ def test_device_sampling_is_per_request_and_survives_compaction(ckpt, device):
     assert [len(t) for t in together] == [5, 14, 9]
     # Alone, a request runs the single-row kernels, and in another row of a batch its sums
     # are formed in another order (log-probabilities move by a few 1e-3): a draw that falls
-    # on the edge between two tokens may then go the other way, so across placements only the
-    # beginning is compared; the same placement again must give the same tokens exactly.
+    # on the edge between two tokens may then go the other way, so sampled tokens are only
+    # compared between runs of the SAME placement (exactly); that the state travels with the
+    # request (seed, draw counter, history ring) is checked row by row after every step
+    # (_run_batch).
     flipped = [[r.token for r in rs] for rs in _run_batch(gm, reqs[::-1])][::-1]
     assert [len(t) for t in flipped] == [5, 14, 9]
-    assert all(t[:3] == s[:3] == f[:3] for t, s, f in zip(together, solo, flipped))
     staggered = [[r.token for r in rs] for rs in _run_batch(gm, reqs, stagger=3)]
-    assert [len(t) for t in staggered] == [5, 14, 9] and staggered[0] == solo[0]
+    assert [len(t) for t in staggered] == [5, 14, 9]
     assert staggered == [[r.token for r in rs] for rs in _run_batch(gm, reqs, stagger=3)]
     again = [[r.token for r in rs] for rs in _run_batch(gm, reqs)]
     assert again == together  # same seeds, same tokens
