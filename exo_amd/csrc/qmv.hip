@@ -1080,7 +1080,7 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   while (min_rows > 1 && p.N / (min_rows * kWaves) < 160) min_rows /= 2;
   int max_grid = (p.N + min_rows * kWaves - 1) / (min_rows * kWaves);
   if (grid > max_grid) grid = max_grid;
-  if (pairs > 1) {
+  if (pairs > 1 && !p.each_row) {  // (rows of one small matrix keep the single-row grid)
     // gather mode (one launch covers `pairs` (token, slot) products, blockIdx.y each): every
     // workgroup stages and normalises its token's activations first, so two rows per wave
     // at least, and about 1536 workgroups in all.  Measured, workgroups per pair: 768x2048
