@@ -31,7 +31,7 @@ from .cache import ShardKVCache
 from .config import ModelConfig
 from .generate import (
     DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, TokenStream, extract_top_logprobs,
-    make_sampler, prefill, processors_for,
+    generate, make_sampler, prefill, processors_for,
 )
 from .loader import load_shard_weights
 from .model import ShardModel
@@ -611,6 +611,137 @@ class BatchGenerator(Engine):
                             model_id=request.model_id, start_pos=request.start_pos)
 
 
+@dataclass(eq=False)
+class SequentialGenerator(Engine):
+    """One request at a time through ``generate()``: the reference's SequentialGenerator
+    (src/exo/worker/runner/llm_inference/batch_generator.py:90-318), which its builder picks
+    when EXO_NO_BATCH is set (src/exo/worker/engines/mlx/builder.py:86-99).  A step yields the
+    next token of the running request; the step after its last token yields
+    FinishedResponse and starts the next queued request.  Cancellation is looked at every
+    ``check_for_cancel_every`` tokens and between prefill chunks."""
+
+    model: ShardModel
+    tokenizer: Any
+    model_id: str
+    device_rank: int = 0
+    cancel_receiver: Any = None
+    event_sender: Any = None
+    check_for_cancel_every: int = 50
+    max_seq: int = 8192
+    kv_prefix_cache: KVPrefixCache | None = None
+    _cancelled_tasks: set = field(default_factory=set, init=False)
+    _all_tasks: dict = field(default_factory=dict, init=False)
+    _queue: deque = field(default_factory=deque, init=False)
+    _active: Any = field(default=None, init=False)  # (task, generator)
+    _prefill_cache: Any = field(default=None, init=False)
+
+    def _eos(self) -> list[int]:
+        return list(getattr(self.tokenizer, "eos_token_ids", None) or [])
+
+    def warmup(self) -> None:
+        params = TextGenerationTaskParams(model=self.model_id, max_output_tokens=50, temperature=0.0,
+                                          bench=True)
+        prompt = [1 % self.model.cfg.vocab_size] * 16
+        t0 = time.perf_counter()
+        n = sum(1 for _ in generate(self.model, self.tokenizer, params, prompt, max_seq=self.max_seq,
+                                    eos_token_ids=self._eos()))
+        dt = time.perf_counter() - t0
+        self.check_for_cancel_every = max(1, min(100, int(n / dt))) if dt > 0 else 50
+
+    def submit(self, task: GenerationTask) -> None:
+        self._cancelled_tasks.discard(CANCEL_ALL_TASKS)
+        self._all_tasks[task.task_id] = task
+        self._queue.append(task)
+
+    def agree_on_cancellations(self) -> None:
+        if self.cancel_receiver is None:
+            return
+        for task_id in self.cancel_receiver.collect():
+            if task_id == CANCEL_ALL_TASKS:
+                self._cancelled_tasks.add(CANCEL_ALL_TASKS)
+            elif task_id in self._all_tasks:
+                self._cancelled_tasks.add(task_id)
+
+    def _cancelled(self):
+        out = [(tid, CancelledResponse()) for tid in self._cancelled_tasks if tid != CANCEL_ALL_TASKS]
+        self._cancelled_tasks.clear()
+        return out
+
+    def step(self):
+        if self._active is None:
+            if not self._queue:
+                self.agree_on_cancellations()
+                return self._cancelled()
+            self._start_next()
+        task, gen = self._active
+        output: list[tuple[Any, Any]] = []
+        try:
+            response = next(gen)
+            if self.device_rank == 0:
+                output.append((task.task_id, map_responses_to_chunks(response, self.model_id)))
+        except (StopIteration, PrefillCancelled):
+            output.append((task.task_id, FinishedResponse()))
+            self._active = None
+            self._all_tasks.pop(task.task_id, None)
+            if self._queue:
+                self._start_next()
+        except Exception as e:
+            self._send_error(task, e)
+            self._active = None
+            raise
+        return output + self._cancelled()
+
+    def _start_next(self) -> None:
+        task = self._queue.popleft()
+        try:
+            self._active = (task, self._build_generator(task))
+        except Exception as e:
+            self._send_error(task, e)
+            raise
+
+    def _send_error(self, task: GenerationTask, e: Exception) -> None:
+        if self.device_rank == 0 and self.event_sender is not None:
+            self.event_sender.send(
+                (task.command_id, ErrorChunk(model=self.model_id, error_message=str(e))))
+
+    def _build_generator(self, task: GenerationTask):
+        prompt = _prompt_of(self.tokenizer, task.task_params)
+        if isinstance(prompt, str):
+            prompt = self.tokenizer.encode(prompt)
+
+        def check_cancel() -> None:
+            self.agree_on_cancellations()
+            if self.should_cancel(task.task_id):
+                raise PrefillCancelled()
+
+        def on_prefill_progress(processed: int, total: int) -> None:
+            if self.device_rank == 0 and self.event_sender is not None:
+                self.event_sender.send(
+                    (task.command_id, PrefillProgressChunk(self.model_id, processed, total)))
+            check_cancel()
+
+        since = self.check_for_cancel_every
+
+        def on_generation_token() -> None:
+            nonlocal since
+            since += 1
+            if since >= self.check_for_cancel_every:
+                since = 0
+                check_cancel()
+
+        return generate(self.model, self.tokenizer, task.task_params, list(prompt), on_prefill_progress,
+                        on_generation_token, max_seq=self.max_seq, eos_token_ids=self._eos(),
+                        kv_prefix_cache=self.kv_prefix_cache)
+
+    def close(self) -> None:
+        self._active = None
+        self.model = None  # type: ignore[assignment]
+        self.tokenizer = None
+
+    def serve_prefill(self, request, wfile) -> None:
+        BatchGenerator.serve_prefill(self, request, wfile)  # the same KV row of its own
+
+
 # ----------------------------------------------------------------------- Builder
 
 
@@ -665,6 +796,12 @@ class Mi355xBuilder(Builder):
 
     def build(self) -> Engine:
         assert self.inference_model is not None
+        if os.environ.get("EXO_NO_BATCH"):  # builder.py:86-99
+            return SequentialGenerator(model=self.inference_model, tokenizer=self.tokenizer,
+                                       model_id=self.model_id, device_rank=0,
+                                       cancel_receiver=self.cancel_receiver,
+                                       event_sender=self.event_sender, max_seq=self.max_seq,
+                                       kv_prefix_cache=KVPrefixCache(None, self.device))
         return BatchGenerator(model=self.inference_model, tokenizer=self.tokenizer,
                               model_id=self.model_id, device_rank=0,
                               cancel_receiver=self.cancel_receiver, event_sender=self.event_sender,

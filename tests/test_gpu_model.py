@@ -409,10 +409,17 @@ def test_batch_generator_slot_compaction_and_cancel(ckpt, device):
     assert not g.has_work
 
 
-def test_builder_engine_contract(ckpt, device):
+@pytest.mark.parametrize("no_batch", [False, True])
+def test_builder_engine_contract(ckpt, device, monkeypatch, no_batch):
     """Runner-side sequence of src/exo/worker/runner/runner.py:250-386: load (progress
-    events) -> build -> warmup -> submit -> step until Finished."""
+    events) -> build -> warmup -> submit -> step until Finished; for the batched engine and
+    for the sequential one the reference's builder returns under EXO_NO_BATCH
+    (src/exo/worker/engines/mlx/builder.py:86-99)."""
     cfg, path = ckpt["cfg"], ckpt["path"]
+    if no_batch:
+        monkeypatch.setenv("EXO_NO_BATCH", "1")
+    else:
+        monkeypatch.delenv("EXO_NO_BATCH", raising=False)
 
     class Sender:
         def __init__(self):
@@ -437,6 +444,7 @@ def test_builder_engine_contract(ckpt, device):
     assert [(p.layers_loaded, p.total) for p in prog] == [
         (i + 1, cfg.num_hidden_layers) for i in range(cfg.num_hidden_layers)]
     eng = b.build()
+    assert type(eng).__name__ == ("SequentialGenerator" if no_batch else "BatchGenerator")
     eng.warmup()
     assert eng.check_for_cancel_every >= 1
     prompt = [int(t) for t in rng(51).integers(0, cfg.vocab_size, size=20)]
@@ -452,6 +460,21 @@ def test_builder_engine_contract(ckpt, device):
     assert kinds == ["TokenChunk"] * 5 + ["FinishedResponse"]
     assert events[4][1].finish_reason == "length" and events[4][1].stats.generation_tokens == 5
     assert all(tid == "task-1" for tid, _ in events)
+    want = [r.token for r in generate(b.inference_model, None, params, prompt)]
+    assert [e.token_id for _, e in events[:5]] == want
+    # two queued requests: the sequential engine finishes the first before the second starts
+    for name in ("task-a", "task-b"):
+        eng.submit(GenerationTask(name, "cmd-" + name, params))
+    events = []
+    for _ in range(40):
+        events += list(eng.step())
+        if [type(e).__name__ for _, e in events].count("FinishedResponse") == 2:
+            break
+    per = {n: [e.token_id for t, e in events if t == n and type(e).__name__ == "TokenChunk"]
+           for n in ("task-a", "task-b")}
+    assert per == {"task-a": want, "task-b": want}
+    if no_batch:
+        assert [t for t, _ in events] == ["task-a"] * 6 + ["task-b"] * 6
     # cancellation of a running task
     eng.submit(GenerationTask("task-2", "cmd-2", TextGenerationTaskParams(
         model="tiny/model", input=prompt, max_output_tokens=500, temperature=0.0)))
