@@ -28,10 +28,14 @@
 //    a (32 or 64) x 256 tile, so no weight row is dequantised twice, and K is split until the
 //    launch has up to two workgroups per CU (14336x4096 4-bit at 32 rows: 31 -> 21 us,
 //    4096x14336: 32.5 -> 23 us; at 96 rows and more the 128-row tile is level or faster).
-//    Without the arithmetic that launch still takes 3/4 of its time, and re-reading one
-//    weight block from L2 changes nothing: a wave instruction that touches 32 rows x 32 bytes
-//    is bound by line requests, not by bytes.  A ring of eight register stages (every load of
-//    a K range requested before the first product) was slower than two stages.
+//    Where that launch's time goes (14336x4096 4-bit, 32 rows, 22 us with the reduce launch):
+//    the weights alone, requested as they are, take 10 us (what the one-row GEMV takes for the
+//    same matrix); the dequantisation and products add 5 us that do not overlap (all
+//    workgroups run in step: one round of 448 workgroups, two K ranges of loads each); the
+//    float32 partial tiles 3.4 us to store and 4 us to reduce; the activation tiles 1 us.
+//    Requesting the weights as whole 128-byte lines (8 rows x 128 B per wave instruction
+//    instead of 32 rows x 32 B) gained 8 %, re-reading one weight block from L2 nothing, a ring
+//    of eight register stages nothing, four K steps per barrier nothing: none was kept.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 
