@@ -111,7 +111,9 @@ int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
  * 128 x 128: a short prompt, or a narrow matrix such as a MoE router under a long one): the
  * tiles alone do not fill the chip, so K is split over up to 8 workgroups per tile, the
  * float32 partial tiles go to `workspace` and a second small launch adds them in a fixed
- * order.  exo_qmm_workspace(M, N) bytes (0: this shape never splits),
+ * order.  Inputs of up to 32 rows (64 on matrices of 8192 rows or more; matrices of at most
+ * 32768 rows) take a 256-column tile whose four waves own 64 weight rows each, with K split
+ * up to 16 ways.  exo_qmm_workspace(M, N) bytes (0: this shape never splits),
  * 256-byte aligned, no initialisation needed.  Launches that share a workspace must be
  * ordered on one stream.  workspace == NULL behaves like exo_qmm. */
 int64_t exo_qmm_workspace(int M, int N);
