@@ -27,8 +27,10 @@ commonly stated ones and are "parity unpinned" against mlx_lm itself:
 The random stream is this build's own (Philox-4x32-10 keyed by the request seed, one block
 per draw): MLX's generator cannot be reproduced without MLX.  What IS pinned: Philox
 against the published known-answer vectors, the filters against independent torch
-restatements (sort / cumsum / topk), top-k log-probabilities against ``torch.topk``, the
-inverse-CDF draw against hand-worked cases.
+restatements (sort / cumsum / topk) and against the logits warpers of ``transformers``
+(TopP / TopK / MinP: same kept sets), the repetition penalty against
+``transformers.RepetitionPenaltyLogitsProcessor``, top-k log-probabilities against
+``torch.topk``, the inverse-CDF draw against hand-worked cases.
 """
 
 from __future__ import annotations

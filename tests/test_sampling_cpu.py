@@ -132,3 +132,42 @@ def test_sampler_record_layout():
     assert b.banned == [2, 3] and b.edits and not b.draws
     assert not SamplerSettings(repetition_penalty=1.2, repetition_context=1000).on_device()
     assert PARAMS_DTYPE.names[-1] == "banned"
+
+
+def test_filters_and_repetition_against_transformers():
+    """The same definitions as implemented by another library: transformers' logits warpers
+    (`TopPLogitsWarper`, `TopKLogitsWarper`, `MinPLogitsWarper`) and its
+    `RepetitionPenaltyLogitsProcessor` - the kept set of every filter and of their composition,
+    and the penalised values (penalty 2 and 0.5: results exact in bf16)."""
+    from transformers.generation.logits_process import (
+        MinPLogitsWarper, RepetitionPenaltyLogitsProcessor, TopKLogitsWarper, TopPLogitsWarper)
+    rng = np.random.default_rng(5)
+    for trial in range(40):
+        V = int(rng.integers(5, 400))
+        x = bf16_round((rng.standard_normal(V) * rng.uniform(0.5, 4.0)).astype(np.float32))
+        if trial % 3 == 0:  # distinct values, so that no tie sits on a filter's edge
+            x = bf16_round((np.argsort(np.argsort(x)) * 0.0625 - 3.0).astype(np.float32))
+        xt = torch.from_numpy(x)[None].double()
+        for top_p, min_p, top_k in [(0.9, 0.0, 0), (0.5, 0.0, 0), (1.0, 0.05, 0), (1.0, 0.3, 0),
+                                    (1.0, 0.0, 1), (1.0, 0.0, 7), (0.8, 0.1, 0), (0.7, 0.0, 5), (0.95, 0.02, 40)]:
+            y = xt.clone()
+            if top_k > 0:
+                y = TopKLogitsWarper(top_k=min(top_k, V))(None, y)
+            if top_p < 1.0:
+                y = TopPLogitsWarper(top_p=top_p)(None, xt.clone()).where(torch.isfinite(y), y)
+            if min_p > 0.0:
+                y = MinPLogitsWarper(min_p=min_p)(None, xt.clone()).where(torch.isfinite(y), y)
+            want = torch.isfinite(y[0]).numpy()
+            thr = S.keep_threshold(x, S.SamplerParams(temperature=1.0, top_p=top_p, min_p=min_p, top_k=top_k))
+            got = x >= thr
+            if len(np.unique(x)) == V:
+                assert (got == want).all(), (trial, top_p, min_p, top_k)
+            else:
+                # values tied at a filter's edge: the library keeps some of them (by sort
+                # position), this build all of them
+                assert got[want].all() and (x[got & ~want] == x[want].min()).all(), (trial, top_p, min_p, top_k)
+        hist = [int(t) for t in rng.integers(0, V, size=12)]
+        for pen in (2.0, 0.5):
+            want = RepetitionPenaltyLogitsProcessor(penalty=pen)(torch.tensor([hist]), torch.from_numpy(x)[None].clone())[0].numpy()
+            got = S.apply_processors(x, hist, S.SamplerParams(repetition_penalty=pen, repetition_context=12))
+            assert (got == want).all(), (trial, pen)
