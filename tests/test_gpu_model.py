@@ -623,16 +623,18 @@ def test_send_and_ingest_kv_cache(ckpt, device):
     assert res.kv_chunks == {} and res.total_tokens == 0
 
 
-def test_serve_prefill_over_tcp_then_decode(ckpt, device):
-    """The engine as prefill server: a request over the TCP front is resolved by
+@pytest.mark.parametrize("engine_cls", ["BatchGenerator", "SequentialGenerator"])
+def test_serve_prefill_over_tcp_then_decode(ckpt, device, engine_cls):
+    """The engine (batched or sequential) as prefill server: a request over the TCP front is resolved by
     Engine.serve_prefill; the KV that arrives is bit-identical to a local prefill of the
     same tokens and a decoder continuing from it produces the local tokens.  The server
     stops three positions short of the tokens it is given (serve.py:43-58: target n-2,
     and the prefill routine leaves one more out), so the client asks with one padding
     token to receive N-2 positions."""
     from exo_amd import disaggregated as D
-    from exo_amd.engine import BatchGenerator
+    import exo_amd.engine as E
     from exo_amd.prefix_cache import KVPrefixCache
+    BatchGenerator = getattr(E, engine_cls)
     cfg, gm = ckpt["cfg"], ckpt["model"]
     prompt = [int(t) for t in rng(91).integers(0, cfg.vocab_size, size=45)]
     params = TextGenerationTaskParams(model="tiny", max_output_tokens=6, temperature=0.0)
