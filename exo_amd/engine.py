@@ -280,7 +280,7 @@ class ShardBatchGenerator:
                 logger.warning("remote prefill failed, falling back to local prefill", exc_info=True)
                 self.cache.offsets[row] = prefix_hit_length
                 self.cache.sync_pos()
-        return prefill(self.model, remaining[:-1], self.cache, progress, row=row)
+        return prefill(self.model, remaining[:-1], self.cache, progress, row=row, graph_steps=True)
 
     # ------------------------------------------------------------------ the step
     def _launch(self, from_host: bool) -> _Flight:

@@ -169,7 +169,7 @@ def extract_top_logprobs(logprobs: torch.Tensor, tokenizer, top_logprobs: int,
 def prefill(model: ShardModel, prompt_tokens, cache: ShardKVCache,
             on_prefill_progress: Callable[[int, int], None] | None = None,
             step: int = PREFILL_STEP_SIZE, faithful_extra_steps: bool = True,
-            row: int = 0) -> tuple[float, int]:
+            row: int = 0, graph_steps: bool = False) -> tuple[float, int]:
     """Fill cache row ``row`` from ``prompt_tokens`` (n ids).  After it the row holds
     n-1 entries (invariant asserted by the reference's test_kv_prefix_cache.py:157).
 
@@ -177,7 +177,9 @@ def prefill(model: ShardModel, prompt_tokens, cache: ShardKVCache,
     n-1 tokens; token n-1 is then run as a single-token forward whose sample is
     discarded, the generator it came from had already computed one more single-token
     forward, and ``trim(2)`` removes both entries.  ``faithful_extra_steps=False``
-    skips those two forwards (same cache contents, less work).
+    skips those two forwards (same cache contents, less work).  ``graph_steps``: run them as
+    replays of the captured single-token step of this cache row instead of launch by launch
+    (same kernels; worth it for a cache that serves many requests).
     Returns (tokens_per_sec, n)."""
     n = len(prompt_tokens)
     if n == 0:
@@ -193,9 +195,17 @@ def prefill(model: ShardModel, prompt_tokens, cache: ShardKVCache,
         if on_prefill_progress is not None:
             on_prefill_progress(done, n)
     if faithful_extra_steps:
-        lg = model(toks[:, done : done + 1], cache, logits="last", rows=rows)
-        nxt = torch.argmax(lg[0, -1].float()).reshape(1, 1)
-        model(nxt, cache, logits="last", rows=rows)
+        if graph_steps and model.is_first and model.is_last:
+            # the same two single-token forwards as graph replays (a cache that outlives the
+            # call keeps its captured step per row): the second consumes the first's argmax
+            bufs = model._buffers(1, 1)
+            bufs.tokens.copy_(toks[0, done : done + 1])
+            model.decode_step(cache, 1, feedback=True, row0=row)
+            model.decode_step(cache, 1, feedback=True, row0=row)
+        else:
+            lg = model(toks[:, done : done + 1], cache, logits="last", rows=rows)
+            nxt = torch.argmax(lg[0, -1].float()).reshape(1, 1)
+            model(nxt, cache, logits="last", rows=rows)
         cache.trim(2, rows=range(row, row + 1))
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0

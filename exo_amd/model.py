@@ -314,8 +314,8 @@ class ShardModel:
 
     # ------------------------------------------------------------------ graph decode
     def decode_step(self, cache: ShardKVCache, B: int, use_graph: bool = True,
-                    feedback: bool = False, sampler=None, mode: int = 0) -> _Buffers:
-        """One single-token step for cache rows [0,B): reads ``bufs.tokens`` (first shard)
+                    feedback: bool = False, sampler=None, mode: int = 0, row0: int = 0) -> _Buffers:
+        """One single-token step for cache rows [row0, row0+B): reads ``bufs.tokens`` (first shard)
         or ``bufs.h``, leaves logits / next_token / lse / logprob (last shard) or the
         hidden state in the returned buffers, advances the device positions.  The kernel
         sequence is captured once per B into a HIP graph and replayed.  ``feedback``
@@ -324,28 +324,33 @@ class ShardModel:
         ends in the device sampling kernels with the stages ``mode`` names instead of the
         plain argmax; results are then in the sampler's ``token`` / ``logprob`` / ``top_*``."""
         bf = self._buffers(B, 1)
-        if max(cache.offsets[:B]) + 1 > cache.max_seq:
+        rsl = slice(row0, row0 + B)
+        if row0 < 0 or row0 + B > cache.batch:
+            raise ValueError(f"rows [{row0}, {row0 + B}) outside the cache's {cache.batch} rows")
+        if max(cache.offsets[rsl]) + 1 > cache.max_seq:
             raise ValueError("KV cache overflow")
         if sampler is not None and not self.is_last:
             raise ValueError("sampling needs the shard that holds the lm_head")
+        if sampler is not None and row0 != 0:
+            raise ValueError("the sampling state is indexed by cache row: row0 must be 0 with a sampler")
 
         def body():
-            out = self._run(B, 1, cache, bf, "all")
+            out = self._run(B, 1, cache, bf, "all", rsl if row0 else None)
             if self.is_last and sampler is not None:
                 sampler.sample(out, B, mode, feedback=bf.tokens if feedback else None,
-                               pos_inc=cache.pos[:B])
+                               pos_inc=cache.pos[rsl])
             elif self.is_last:
                 ops.argmax_logsumexp(out, bf.next_token, bf.lse, bf.logprob, bf.argmax_ws,
-                                     cache.pos[:B])
+                                     cache.pos[rsl])
                 if feedback:
                     bf.tokens.copy_(bf.next_token)
             else:
-                cache.pos[:B] += 1
+                cache.pos[rsl] += 1
 
         if not use_graph:
             body()
         else:
-            key = (B, feedback, sampler is not None, mode)
+            key = (B, feedback, sampler is not None, mode, row0)
             hit = self._graphs.get(key)
             if hit is None or hit[1] is not cache or hit[2] is not sampler:
                 # warm up outside capture (lazy module loads, attribute settings), then
@@ -371,5 +376,5 @@ class ShardModel:
                 cache.pos.copy_(saved)
                 self._graphs[key] = (g, cache, sampler)
             self._graphs[key][0].replay()
-        cache.advance_host(1, range(B))
+        cache.advance_host(1, range(row0, row0 + B))
         return bf
