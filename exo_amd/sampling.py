@@ -22,6 +22,7 @@ import torch
 
 from . import native
 from .native import check
+from .ops import _stream
 
 MAX_CONTEXT = 256   # EXO_SAMPLER_MAX_CONTEXT
 MAX_BANNED = 8      # EXO_SAMPLER_MAX_BANNED
@@ -197,4 +198,4 @@ class DeviceSampler:
             self.logprob.data_ptr(), self.lse.data_ptr(), self.top_idx.data_ptr(),
             self.top_val.data_ptr(), p(feedback), p(pos_inc), self.workspace.data_ptr(),
             self.workspace.numel(), rows, self.V, self.hist_cap, mode,
-            torch.cuda.current_stream().cuda_stream), "sample")
+            _stream()), "sample")
