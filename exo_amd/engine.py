@@ -31,7 +31,7 @@ from .cache import ShardKVCache
 from .config import ModelConfig
 from .generate import (
     DEFAULT_TOP_LOGPROBS, MAX_TOKENS, PrefillCancelled, TokenStream, extract_top_logprobs,
-    generate, make_sampler, prefill, processors_for,
+    GenerateState, generate, make_sampler, prefill, processors_for,
 )
 from .loader import load_shard_weights
 from .model import ShardModel
@@ -634,6 +634,7 @@ class SequentialGenerator(Engine):
     _queue: deque = field(default_factory=deque, init=False)
     _active: Any = field(default=None, init=False)  # (task, generator)
     _prefill_cache: Any = field(default=None, init=False)
+    _state: Any = field(default=None, init=False)   # GenerateState
 
     def _eos(self) -> list[int]:
         return list(getattr(self.tokenizer, "eos_token_ids", None) or [])
@@ -643,8 +644,10 @@ class SequentialGenerator(Engine):
                                           bench=True)
         prompt = [1 % self.model.cfg.vocab_size] * 16
         t0 = time.perf_counter()
-        n = sum(1 for _ in generate(self.model, self.tokenizer, params, prompt, max_seq=self.max_seq,
-                                    eos_token_ids=self._eos()))
+        if self._state is None:
+            self._state = GenerateState(self.model, self.max_seq)
+        n = sum(1 for _ in generate(self.model, self.tokenizer, params, prompt,
+                                    eos_token_ids=self._eos(), state=self._state))
         dt = time.perf_counter() - t0
         self.check_for_cancel_every = max(1, min(100, int(n / dt))) if dt > 0 else 50
 
@@ -729,12 +732,15 @@ class SequentialGenerator(Engine):
                 since = 0
                 check_cancel()
 
+        if self._state is None:  # one cache row and sampler for all requests: graphs stay valid
+            self._state = GenerateState(self.model, self.max_seq)
         return generate(self.model, self.tokenizer, task.task_params, list(prompt), on_prefill_progress,
-                        on_generation_token, max_seq=self.max_seq, eos_token_ids=self._eos(),
-                        kv_prefix_cache=self.kv_prefix_cache)
+                        on_generation_token, eos_token_ids=self._eos(),
+                        kv_prefix_cache=self.kv_prefix_cache, state=self._state)
 
     def close(self) -> None:
         self._active = None
+        self._state = None
         self.model = None  # type: ignore[assignment]
         self.tokenizer = None
 

@@ -299,11 +299,24 @@ class TokenStream:
 # ---------------------------------------------------------------------- generate
 
 
+class GenerateState:
+    """A KV cache row and the sampling arrays that serve one request after another: the HIP
+    graphs ``generate()`` captures are bound to them, so a caller that keeps the state (the
+    sequential engine) captures once instead of once per request."""
+
+    def __init__(self, model: ShardModel, max_seq: int):
+        from .sampling import DeviceSampler
+        self.max_seq = max_seq
+        self.cache = model.make_cache(1, max_seq)
+        self.sampler = DeviceSampler(1, model.cfg.vocab_size, model.device)
+
+
 def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, prompt_tokens: list[int],
              on_prefill_progress: Callable[[int, int], None] | None = None,
              on_generation_token: Callable[[], None] | None = None,
              max_seq: int | None = None, eos_token_ids: list[int] | None = None,
-             kv_prefix_cache=None) -> Generator[GenerationResponse, None, None]:
+             kv_prefix_cache=None, state: GenerateState | None = None,
+             ) -> Generator[GenerationResponse, None, None]:
     """Sequential (batch 1) generation for a full-model shard: yields one
     GenerationResponse per token; the last carries finish_reason, stats and usage.
     ``kv_prefix_cache`` (a KVPrefixCache) is consulted and updated the way the reference's
@@ -320,7 +333,14 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     n_prompt = len(prompt_tokens)
     if n_prompt == 0:
         raise ValueError("empty prompt")
-    cache = model.make_cache(1, max_seq or (n_prompt + max_tokens + 8))
+    if state is not None:
+        cache = state.cache
+        cache.reset()
+        if n_prompt + 2 > cache.max_seq:
+            raise ValueError(f"prompt of {n_prompt} tokens exceeds the cache ({cache.max_seq})")
+        max_tokens = min(max_tokens, cache.max_seq - n_prompt - 2)
+    else:
+        cache = model.make_cache(1, max_seq or (n_prompt + max_tokens + 8))
     torch.cuda.reset_peak_memory_stats(model.device)
 
     eos = list(eos_token_ids or [])
@@ -332,7 +352,8 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     if kv_prefix_cache is not None:
         _, remaining, matched_index, is_exact_hit = kv_prefix_cache.get_kv_cache(cache, prompt_tokens)
     prefix_hit_length = n_prompt - len(remaining)
-    prefill_tps, prefill_tokens = prefill(model, remaining[:-1], cache, on_prefill_progress)
+    prefill_tps, prefill_tokens = prefill(model, remaining[:-1], cache, on_prefill_progress,
+                                          graph_steps=state is not None)
     assert cache_length(cache) == max(n_prompt - 2, prefix_hit_length)
     prefix_cache_hit = "none"
     if matched_index is not None and prefix_hit_length > 0:
@@ -347,7 +368,11 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     # the last two prompt tokens, one forward each (generate.py:710-733); they are also all
     # the logits processors see of the prompt (stream_generate is handed prompt[-2:])
     if len(remaining) >= 2:
-        model(torch.tensor([[remaining[-2]]], dtype=torch.int32), cache, logits="none")
+        if state is not None:  # the captured step of this cache (its sample is not used)
+            model._buffers(1, 1).tokens[0] = int(remaining[-2])
+            model.decode_step(cache, 1)
+        else:
+            model(torch.tensor([[remaining[-2]]], dtype=torch.int32), cache, logits="none")
     tok = int(prompt_tokens[-1])
     history = [int(t) for t in prompt_tokens[-2:]]
     stream = TokenStream(tokenizer, task, eos, max_tokens, n_prompt, prefill_tps, prefix_cache_hit,
@@ -356,7 +381,7 @@ def generate(model: ShardModel, tokenizer, task: TextGenerationTaskParams, promp
     k_top = task.top_logprobs or DEFAULT_TOP_LOGPROBS
     on_device = settings.on_device() and k_top <= 20
     if on_device:
-        ds = DeviceSampler(1, model.cfg.vocab_size, model.device)
+        ds = state.sampler if state is not None else DeviceSampler(1, model.cfg.vocab_size, model.device)
         ds.set_row(0, settings, history)
         mode = ds.mode(1, want_top)
     else:

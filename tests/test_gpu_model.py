@@ -752,3 +752,27 @@ def _run_batch_seq(gm, params, prompt):
     while g.has_work:
         out += [r for _, r in g.step()]
     return out
+
+
+def test_generate_with_persistent_state_equals_fresh_state(ckpt, device):
+    """generate() on a cache row and sampler that outlive the request (what the sequential
+    engine keeps, so that its HIP graphs are captured once): the same tokens as with fresh
+    ones, request after request, also after a request that was abandoned half way, greedy and
+    sampled."""
+    from exo_amd.generate import GenerateState
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    P = TextGenerationTaskParams
+    reqs = [(P(model="t", max_output_tokens=7, temperature=0.0), 23),
+            (P(model="t", max_output_tokens=9, temperature=0.8, top_k=12, seed=5, repetition_penalty=1.2), 9),
+            (P(model="t", max_output_tokens=5, temperature=0.0, logprobs=True, top_logprobs=3), 31)]
+    st = GenerateState(gm, 128)
+    for i, (params, n) in enumerate(reqs):
+        prompt = [int(t) for t in rng(300 + i).integers(0, cfg.vocab_size, size=n)]
+        want = [(r.token, r.finish_reason) for r in generate(gm, None, params, prompt)]
+        got = [(r.token, r.finish_reason) for r in generate(gm, None, params, prompt, state=st)]
+        assert got == want, i
+        it = generate(gm, None, params, prompt, state=st)  # abandoned after two tokens
+        next(it), next(it)
+        it.close()
+    with pytest.raises(ValueError):
+        list(generate(gm, None, reqs[0][0], list(range(1, 128)), state=st))
