@@ -12,11 +12,18 @@
 //            streaming passes patch those positions through a slice bitmap, so the logits
 //            themselves are never rewritten;
 //   stats    per slice (max, argmax, sum exp(x - max));
-//   table    (only with top-p / top-k / top-logprobs) every value is a bf16, i.e. a 16-bit
-//            key: count and probability mass per key are accumulated in a 65536-entry table
-//            with integer atomics (mass in 2^-40 fixed point: the sums are exact, so the
-//            result does not depend on arrival order), and one workgroup scans the table
-//            from the top for the k-th largest key, the nucleus edge and the 20th largest key;
+//   coarse   (only with top-p / top-k / top-logprobs) every value is a bf16, i.e. a 16-bit
+//   fine     order-preserving key.  Count and probability mass (2^-40 fixed point: integer sums
+//            are exact, so nothing depends on arrival order) are first accumulated per BUCKET
+//            of 128 keys (sign and exponent: 512 buckets) - in LDS per slice, then the few
+//            non-empty buckets with global atomics.  A scan of the 512 buckets from the top
+//            finds the bucket in which the running count reaches k (and 20), and the one in
+//            which the running mass reaches top_p; a second pass histograms only the values of
+//            those buckets by their low 7 key bits, and a scan of those 128 entries, continued
+//            from the totals above the bucket, gives the exact keys: the k-th largest value,
+//            the nucleus edge, the 20th largest value.  (A flat 65536-entry table took 85 us to
+//            fill with 2 atomics per logit and 115 us to scan and clear; the two levels take a few
+//            microseconds each.)
 //   weights  per slice the sum of exp((x - max) / T) over the kept tokens (x >= threshold);
 //            tokens at or above the 20th largest key are appended to a candidate list;
 //   select   one workgroup per row: uniform from Philox-4x32-10 (key = request seed,
@@ -35,7 +42,9 @@ constexpr int kMaxSlice = 4096;  // elements per slice (two 8-element chunks per
 constexpr int kMaxEdits = EXO_SAMPLER_MAX_CONTEXT + EXO_SAMPLER_MAX_BANNED;
 constexpr int kTop = EXO_SAMPLER_TOP_LOGPROBS;
 constexpr int kMaxCand = 320;  // top-20 candidates: up to 300 ties at the 20th place
-constexpr int kKeys = 65536;
+constexpr int kBuckets = 512;  // key >> 7: sign and exponent
+constexpr int kFine = 128;     // key & 127: mantissa, in value order inside a bucket
+constexpr int kTargets = 3;    // 0: k-th largest (top-k), 1: nucleus edge (top-p), 2: 20th largest
 constexpr float kBan = -1e9f;
 
 struct RowWs {
@@ -44,25 +53,34 @@ struct RowWs {
   float thr;    // value threshold from top-p / top-k (-inf: none)
   int key_top;  // key of the 20th largest value
   int cand_n;
+  // per target: the bucket in which the running count / mass from the top crosses it (-1:
+  // never), and the count and mass of the buckets above it
+  int bkt[kTargets];
+  unsigned int above_c[kTargets];
+  unsigned long long above_m[kTargets];
   int edit_idx[kMaxEdits];
   float edit_val[kMaxEdits];
   unsigned long long cand[kMaxCand];  // key << 32 | index
 };
 constexpr size_t kRowWsBytes = (sizeof(RowWs) + 255) / 256 * 256;
 
-// Workspace: one self-contained region per row (the row's RowWs, then its mass table, then
-// its count table), so launches of different row counts can share one workspace.
-constexpr size_t kRowStride = kRowWsBytes + (size_t)kKeys * 12;
+// mass and count per bucket, and per low key of each target's bucket; zero between steps
+struct Tables {
+  unsigned long long cm[kBuckets];
+  unsigned long long fm[kTargets][kFine];
+  unsigned int cc[kBuckets];
+  unsigned int fc[kTargets][kFine];
+};
+constexpr size_t kTablesBytes = (sizeof(Tables) + 255) / 256 * 256;
+
+// Workspace: one self-contained region per row (the row's RowWs, then its tables), so
+// launches of different row counts can share one workspace.
+constexpr size_t kRowStride = kRowWsBytes + kTablesBytes;
 __device__ __forceinline__ RowWs* row_ws(void* ws, int row) {
   return reinterpret_cast<RowWs*>(static_cast<char*>(ws) + (size_t)row * kRowStride);
 }
-__device__ __forceinline__ unsigned long long* mass_table(void* ws, int row) {
-  return reinterpret_cast<unsigned long long*>(static_cast<char*>(ws) + (size_t)row * kRowStride +
-                                               kRowWsBytes);
-}
-__device__ __forceinline__ unsigned int* count_table(void* ws, int row) {
-  return reinterpret_cast<unsigned int*>(static_cast<char*>(ws) + (size_t)row * kRowStride +
-                                         kRowWsBytes + (size_t)kKeys * 8);
+__device__ __forceinline__ Tables* row_tables(void* ws, int row) {
+  return reinterpret_cast<Tables*>(static_cast<char*>(ws) + (size_t)row * kRowStride + kRowWsBytes);
 }
 
 // order-preserving 16-bit key of a bf16 value and back
@@ -313,14 +331,186 @@ __device__ __forceinline__ bool row_needs_table(const exo_sampler_params& p, boo
   return want_top || (sampling && (p.top_k > 0 || (p.top_p > 0.f && p.top_p < 1.f)));
 }
 
-__global__ __launch_bounds__(256) void sample_table_kernel(
+// what a row asks of the tables
+struct Wanted {
+  unsigned int kk;             // top-k (0: none)
+  bool use_p;                  // top-p
+  unsigned long long target;   // top_p of the mass, fixed point
+  bool top;                    // the 20 most likely
+};
+__device__ __forceinline__ Wanted wanted_of(const exo_sampler_params& p, bool want_top) {
+  const bool sampling = p.temperature != 0.f;
+  Wanted q;
+  q.kk = (sampling && p.top_k > 0) ? (unsigned int)p.top_k : 0u;
+  q.use_p = sampling && p.top_p > 0.f && p.top_p < 1.f;
+  q.target = q.use_p ? (unsigned long long)((double)p.top_p * kMassOne) : 0ull;
+  q.top = want_top;
+  return q;
+}
+
+__device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, int o) {
+  const unsigned int lo = __shfl_up((unsigned int)v, o, 64), hi = __shfl_up((unsigned int)(v >> 32), o, 64);
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ unsigned long long shfl_u64(unsigned long long v, int src) {
+  const unsigned int lo = __shfl((unsigned int)v, src, 64), hi = __shfl((unsigned int)(v >> 32), src, 64);
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// One wave walks N = 64 * PER entries from the highest index down (lane t owns entries
+// N-1 - PER*t .. downwards), the running (count, mass) starting at (c0, m0).  For each target:
+// the entry at which the running count reaches kk / 20 (count before it below, count with it
+// at or above), or the running mass reaches `target`; found[] = entry index or -1, and
+// (fc, fm) = the totals strictly above that entry.  Every lane returns the same values.
+template <int PER>
+__device__ __forceinline__ void scan_down(const unsigned long long* __restrict__ mt,
+                                          const unsigned int* __restrict__ ct, const Wanted& q,
+                                          const unsigned int (&c0)[kTargets],
+                                          const unsigned long long (&m0)[kTargets],
+                                          const bool (&active)[kTargets], int (&found)[kTargets],
+                                          unsigned int (&fc)[kTargets],
+                                          unsigned long long (&fm)[kTargets]) {
+  const int lane = threadIdx.x & 63;
+  const int hi = 64 * PER - 1 - PER * lane;
+  unsigned long long m[PER], msum = 0;
+  unsigned int c[PER], csum = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    m[i] = mt[hi - i];
+    c[i] = ct[hi - i];
+    msum += m[i];
+    csum += c[i];
+  }
+  unsigned long long minc = msum;
+  unsigned int cinc = csum;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const unsigned long long mu = shfl_up_u64(minc, o);
+    const unsigned int cu = __shfl_up(cinc, o, 64);
+    if (lane >= o) {
+      minc += mu;
+      cinc += cu;
+    }
+  }
+  const unsigned long long mex = minc - msum;  // totals of the lanes above (higher entries)
+  const unsigned int cex = cinc - csum;
+#pragma unroll
+  for (int j = 0; j < kTargets; ++j) {
+    int f = -1;
+    unsigned int fcj = 0;
+    unsigned long long fmj = 0;
+    if (active[j]) {
+      unsigned long long ma = m0[j] + mex;
+      unsigned int ca = c0[j] + cex;
+      const unsigned int want_c = j == 0 ? q.kk : (unsigned int)kTop;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        if (c[i]) {
+          const bool hit = (j == 1) ? (ma < q.target && ma + m[i] >= q.target)
+                                    : (ca < want_c && ca + c[i] >= want_c);
+          if (hit) {
+            f = hi - i;
+            fcj = ca;
+            fmj = ma;
+          }
+        }
+        ma += m[i];
+        ca += c[i];
+      }
+    }
+    const unsigned long long mask = __ballot(f >= 0);
+    if (mask) {
+      const int src = __ffsll((long long)mask) - 1;
+      found[j] = __shfl(f, src, 64);
+      fc[j] = __shfl(fcj, src, 64);
+      fm[j] = shfl_u64(fmj, src);
+    } else {
+      found[j] = -1;
+      fc[j] = 0;
+      fm[j] = 0;
+    }
+  }
+}
+
+// ---- coarse: count and mass per bucket ------------------------------------------------
+__global__ __launch_bounds__(256) void sample_coarse_kernel(
     const bf16_t* __restrict__ logits, const exo_sampler_params* __restrict__ params, void* ws,
     int V, int want_top) {
   __shared__ EditLds ed;
+  __shared__ unsigned long long hm[kBuckets];
+  __shared__ unsigned int hc[kBuckets];
   const int row = blockIdx.y;
   if (!row_needs_table(params[row], want_top != 0)) return;
   RowWs* w = row_ws(ws, row);
   const SliceGeom g = slice_geom(logits, V, blockIdx.x);
+  for (int b = threadIdx.x; b < kBuckets; b += 256) {
+    hm[b] = 0;
+    hc[b] = 0;
+  }
+  stage_edits(w, g, ed);  // (ends in a barrier)
+  float mx, lse;
+  int mi;
+  merge_stats(w, mx, mi, lse);
+  float xv[16];
+  int i0[2];
+  load_share(logits + (size_t)row * V, g, ed, xv, i0);
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float x = xv[8 * u + k];
+      if (i0[u] + k < g.hi) {  // -inf logits are real values too (key 0x007f)
+        const int b = key_of(x) >> 7;
+        atomicAdd(&hc[b], 1u);
+        const unsigned long long q = (unsigned long long)((double)expf(x - lse) * kMassOne);
+        if (q) atomicAdd(&hm[b], q);
+      }
+    }
+  __syncthreads();
+  Tables* T = row_tables(ws, row);
+  for (int b = threadIdx.x; b < kBuckets; b += 256) {
+    if (hc[b]) atomicAdd(&T->cc[b], hc[b]);
+    if (hm[b]) atomicAdd(&T->cm[b], hm[b]);
+  }
+}
+
+// ---- fine: the buckets that hold a target, by their low key bits ----------------------
+__global__ __launch_bounds__(256) void sample_fine_kernel(
+    const bf16_t* __restrict__ logits, const exo_sampler_params* __restrict__ params, void* ws,
+    int V, int want_top) {
+  __shared__ EditLds ed;
+  __shared__ unsigned long long hm[kTargets][kFine];
+  __shared__ unsigned int hc[kTargets][kFine];
+  const int row = blockIdx.y;
+  const exo_sampler_params p = params[row];
+  if (!row_needs_table(p, want_top != 0)) return;
+  RowWs* w = row_ws(ws, row);
+  Tables* T = row_tables(ws, row);
+  const Wanted q = wanted_of(p, want_top != 0);
+  // every wave finds the target buckets for itself (512 entries, L2 resident)
+  int bkt[kTargets];
+  unsigned int ac[kTargets];
+  unsigned long long am[kTargets];
+  {
+    const unsigned int c0[kTargets] = {0u, 0u, 0u};
+    const unsigned long long m0[kTargets] = {0ull, 0ull, 0ull};
+    const bool active[kTargets] = {q.kk != 0, q.use_p, q.top};
+    scan_down<kBuckets / 64>(T->cm, T->cc, q, c0, m0, active, bkt, ac, am);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+#pragma unroll
+    for (int j = 0; j < kTargets; ++j) {
+      w->bkt[j] = bkt[j];
+      w->above_c[j] = ac[j];
+      w->above_m[j] = am[j];
+    }
+  }
+  if (bkt[0] < 0 && bkt[1] < 0 && bkt[2] < 0) return;  // (uniform over the workgroup)
+  const SliceGeom g = slice_geom(logits, V, blockIdx.x);
+  for (int i = threadIdx.x; i < kTargets * kFine; i += 256) {
+    (&hm[0][0])[i] = 0;
+    (&hc[0][0])[i] = 0;
+  }
   stage_edits(w, g, ed);
   float mx, lse;
   int mi;
@@ -328,110 +518,64 @@ __global__ __launch_bounds__(256) void sample_table_kernel(
   float xv[16];
   int i0[2];
   load_share(logits + (size_t)row * V, g, ed, xv, i0);
-  unsigned long long* mt = mass_table(ws, row);
-  unsigned int* ct = count_table(ws, row);
 #pragma unroll
   for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const float x = xv[8 * u + k];
-      if (i0[u] + k < g.hi) {  // -inf logits are real values too (key 0x007f)
-        const int key = key_of(x);
-        atomicAdd(&ct[key], 1u);
-        const unsigned long long q = (unsigned long long)((double)expf(x - lse) * kMassOne);
-        if (q) atomicAdd(&mt[key], q);
+      if (i0[u] + k < g.hi) {
+        const int key = key_of(x), b = key >> 7, f = key & (kFine - 1);
+        if (b == bkt[0] || b == bkt[1] || b == bkt[2]) {
+          const unsigned long long qm = (unsigned long long)((double)expf(x - lse) * kMassOne);
+#pragma unroll
+          for (int j = 0; j < kTargets; ++j)
+            if (b == bkt[j]) {
+              atomicAdd(&hc[j][f], 1u);
+              if (qm) atomicAdd(&hm[j][f], qm);
+            }
+        }
       }
     }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kTargets * kFine; i += 256) {
+    const unsigned int c = (&hc[0][0])[i];
+    const unsigned long long m = (&hm[0][0])[i];
+    if (c) atomicAdd(&T->fc[0][0] + i, c);
+    if (m) atomicAdd(&T->fm[0][0] + i, m);
+  }
 }
 
-// One workgroup per row walks the table from the largest key down: the k-th largest key,
-// the nucleus edge (the first key whose strictly larger keys hold less than top_p of the
-// mass and which together with them reaches it), the 20th largest key.  Leaves the table
-// zero for the next step.
-__global__ __launch_bounds__(1024) void sample_scan_kernel(
-    const exo_sampler_params* __restrict__ params, void* ws, int want_top) {
-  __shared__ unsigned long long s_mass[16];
-  __shared__ unsigned int s_cnt[16];
-  __shared__ int s_key_k, s_key_p, s_key_t;
-  const int row = blockIdx.x, t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
-  const exo_sampler_params p = params[row];
-  if (!row_needs_table(p, want_top != 0)) return;
-  RowWs* w = row_ws(ws, row);
-  unsigned long long* mt = mass_table(ws, row);
-  unsigned int* ct = count_table(ws, row);
-  // thread t owns the 64 keys from hi = 65535 - 64 t downwards
-  constexpr int PER = kKeys / 1024;
-  const int hi = kKeys - 1 - PER * t;
-  unsigned long long msum = 0;
-  unsigned int csum = 0;
-  for (int i = 0; i < PER; ++i) {
-    msum += mt[hi - i];
-    csum += ct[hi - i];
-  }
-  // exclusive prefix over the threads above this one (their keys are all larger)
-  unsigned long long minc = msum;
-  unsigned int cinc = csum;
+// The exact keys from the fine tables (one wave; the same values in every lane): the value
+// threshold of top-k / top-p (-inf: none) and the key of the 20th largest value (0: none).
+__device__ __forceinline__ void fine_thresholds(const RowWs* w, const Tables* T, const Wanted& q,
+                                                float& thr, int& key_top) {
+  thr = -INFINITY;
+  key_top = 0;
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const unsigned int mlo = __shfl_up((unsigned int)minc, o, 64);
-    const unsigned int mhi = __shfl_up((unsigned int)(minc >> 32), o, 64);
-    const unsigned int cu = __shfl_up(cinc, o, 64);
-    if (lane >= o) {
-      minc += ((unsigned long long)mhi << 32) | mlo;
-      cinc += cu;
+  for (int j = 0; j < kTargets; ++j) {
+    const int b = w->bkt[j];
+    if (b < 0) continue;  // fewer than k (20) tokens in all, or the mass never reaches top_p
+    const unsigned int c0[kTargets] = {w->above_c[j], w->above_c[j], w->above_c[j]};
+    const unsigned long long m0[kTargets] = {w->above_m[j], w->above_m[j], w->above_m[j]};
+    const bool active[kTargets] = {j == 0, j == 1, j == 2};
+    int f[kTargets];
+    unsigned int fc[kTargets];
+    unsigned long long fm[kTargets];
+    scan_down<kFine / 64>(T->fm[j], T->fc[j], q, c0, m0, active, f, fc, fm);
+    if (f[j] >= 0) {
+      const int key = (b << 7) | f[j];
+      if (j == 2)
+        key_top = key;
+      else
+        thr = fmaxf(thr, value_of(key));
     }
-  }
-  if (lane == 63) {
-    s_mass[wave] = minc;
-    s_cnt[wave] = cinc;
-  }
-  if (t == 0) {
-    s_key_k = -1;
-    s_key_p = -1;
-    s_key_t = -1;
-  }
-  __syncthreads();
-  unsigned long long ma = minc - msum;
-  unsigned int ca = cinc - csum;
-  for (int wv = 0; wv < wave; ++wv) {
-    ma += s_mass[wv];
-    ca += s_cnt[wv];
-  }
-  const bool sampling = p.temperature != 0.f;
-  const unsigned int kk = (sampling && p.top_k > 0) ? (unsigned int)p.top_k : 0u;
-  const bool use_p = sampling && p.top_p > 0.f && p.top_p < 1.f;
-  const unsigned long long target = use_p ? (unsigned long long)((double)p.top_p * kMassOne) : 0ull;
-  for (int i = 0; i < PER; ++i) {
-    const unsigned long long m = mt[hi - i];
-    const unsigned int c = ct[hi - i];
-    if (c) {
-      // counts: the key at which the running count from the top reaches k (20)
-      if (kk && ca < kk && ca + c >= kk) s_key_k = hi - i;
-      if (want_top && ca < (unsigned)kTop && ca + c >= (unsigned)kTop) s_key_t = hi - i;
-      // mass: a key is kept while the keys strictly above it hold less than top_p
-      if (use_p && ma < target && ma + m >= target) s_key_p = hi - i;
-      ct[hi - i] = 0;
-      if (m) mt[hi - i] = 0;
-    }
-    ma += m;
-    ca += c;
-  }
-  __syncthreads();
-  if (t == 0) {
-    // fewer than k (20) tokens in all, or truncation left the total mass below top_p: keep all
-    float thr = -INFINITY;
-    if (kk && s_key_k >= 0) thr = fmaxf(thr, value_of(s_key_k));
-    if (use_p && s_key_p >= 0) thr = fmaxf(thr, value_of(s_key_p));
-    w->thr = thr;
-    w->key_top = s_key_t >= 0 ? s_key_t : 0;
   }
 }
 
 // ---- weights ------------------------------------------------------------------
-__device__ __forceinline__ float keep_threshold(const exo_sampler_params& p, const RowWs* w,
+__device__ __forceinline__ float keep_threshold(const exo_sampler_params& p, float table_thr,
                                                 float mx) {
-  float thr = w->thr;
+  float thr = table_thr;
   if (p.min_p > 0.f) thr = fmaxf(thr, mx + logf(p.min_p));
   return thr;
 }
@@ -446,6 +590,25 @@ __global__ __launch_bounds__(256) void sample_weights_kernel(
   const bool sampling = p.temperature != 0.f;
   if (!sampling && !want_top) return;
   RowWs* w = row_ws(ws, row);
+  // the exact keys of this step from the fine tables (every wave for itself); the first
+  // workgroup leaves them for the select launch and clears the bucket table, whose last
+  // reader was the previous launch
+  float table_thr = -INFINITY;
+  int kt = 0;
+  if (row_needs_table(p, want_top != 0)) {
+    Tables* T = row_tables(ws, row);
+    fine_thresholds(w, T, wanted_of(p, want_top != 0), table_thr, kt);
+    if (blockIdx.x == 0) {
+      if (threadIdx.x == 0) {
+        w->thr = table_thr;
+        w->key_top = kt;
+      }
+      for (int b = threadIdx.x; b < kBuckets; b += 256) {
+        T->cm[b] = 0;
+        T->cc[b] = 0;
+      }
+    }
+  }
   const SliceGeom g = slice_geom(logits, V, blockIdx.x);
   stage_edits(w, g, ed);
   float mx, lse;
@@ -455,7 +618,6 @@ __global__ __launch_bounds__(256) void sample_weights_kernel(
   int i0[2];
   load_share(logits + (size_t)row * V, g, ed, xv, i0);
   if (want_top) {
-    const int kt = w->key_top;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -470,7 +632,7 @@ __global__ __launch_bounds__(256) void sample_weights_kernel(
         }
   }
   if (!sampling) return;
-  const float thr = keep_threshold(p, w, mx);
+  const float thr = keep_threshold(p, table_thr, mx);
   const float inv_t = 1.f / p.temperature;
   float s = 0.f;
 #pragma unroll
@@ -513,6 +675,13 @@ __global__ __launch_bounds__(256) void sample_select_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const exo_sampler_params p = params[row];
   RowWs* w = row_ws(ws, row);
+  if (row_needs_table(p, want_top != 0)) {  // the weights launch was the fine tables' last reader
+    Tables* T = row_tables(ws, row);
+    for (int i = tid; i < kTargets * kFine; i += 256) {
+      (&T->fm[0][0])[i] = 0;
+      (&T->fc[0][0])[i] = 0;
+    }
+  }
   float mx, lse;
   int mi;
   merge_stats(w, mx, mi, lse);
@@ -557,7 +726,7 @@ __global__ __launch_bounds__(256) void sample_select_kernel(
     float xv[16];
     int i0[2];
     load_share(logits + (size_t)row * V, g, ed, xv, i0);
-    const float thr = keep_threshold(p, w, mx);
+    const float thr = keep_threshold(p, w->thr, mx);
     const float inv_t = 1.f / p.temperature;
     float rem = s_rem;
 #pragma unroll
@@ -700,11 +869,13 @@ extern "C" int exo_sample(const uint16_t* logits, const exo_sampler_params* para
                                                      hist_cap > 0 ? hist_cap : 1);
   sample_stats_kernel<<<dim3(kBlocks, rows), 256, 0, st>>>(lg, workspace, V, edits ? 1 : 0);
   if (mode & (EXO_SAMPLE_TABLE | EXO_SAMPLE_TOP)) {
-    sample_table_kernel<<<dim3(kBlocks, rows), 256, 0, st>>>(lg, params, workspace, V,
-                                                            want_top ? 1 : 0);
-    sample_scan_kernel<<<dim3(rows), 1024, 0, st>>>(params, workspace, want_top ? 1 : 0);
+    sample_coarse_kernel<<<dim3(kBlocks, rows), 256, 0, st>>>(lg, params, workspace, V,
+                                                             want_top ? 1 : 0);
+    sample_fine_kernel<<<dim3(kBlocks, rows), 256, 0, st>>>(lg, params, workspace, V,
+                                                           want_top ? 1 : 0);
   }
-  if (mode & (EXO_SAMPLE_DRAW | EXO_SAMPLE_TOP))
+  // (the weights launch also resolves and clears the tables: it runs whenever they were filled)
+  if (mode & (EXO_SAMPLE_DRAW | EXO_SAMPLE_TOP | EXO_SAMPLE_TABLE))
     sample_weights_kernel<<<dim3(kBlocks, rows), 256, 0, st>>>(lg, params, workspace, V,
                                                               want_top ? 1 : 0);
   sample_select_kernel<<<dim3(rows), 256, 0, st>>>(lg, params, history, hist_len, draws, token,
