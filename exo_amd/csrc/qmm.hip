@@ -545,8 +545,9 @@ __global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict
   }
 }
 
-// launches of fewer than this many 128 x 128 output tiles may split K
-constexpr int kQmmSplitTiles = 128;
+// launches of fewer than this many 128 x 128 output tiles may split K (one tile per CU and
+// less: 2048x4096 under 1023 rows, 128 tiles, 65 -> 38 us with two K ranges)
+constexpr int kQmmSplitTiles = 256;
 
 // K split of a launch: when its 128 x 128 output tiles cover less than half the chip (a
 // short input, or a narrow matrix such as a MoE router under a long prompt); chunks of whole
@@ -613,7 +614,7 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
   // many 128-row tiles are faster there (1024x4096 at 2046 rows: 89 -> 70 us; 4096x4096 at
   // 1023 rows, exactly 128 tall tiles: 93 -> 77 us), not beyond (192 tall tiles: 88 vs 97 us)
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
-  if (M <= 128 || small_grid) {
+  if (M <= 128 || small_grid || p.ksplit > 1) {  // (only the 128-row tile splits K)
     if (sb4)
       qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
     else
@@ -838,7 +839,11 @@ extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const u
 extern "C" int64_t exo_qmm_workspace(int M, int N) {
   if (M <= 0 || N <= 0) return 0;
   int64_t ranges = 0;
-  if ((int64_t)exo_ceil_div(N, 128) * exo_ceil_div(M, 128) < kQmmSplitTiles) ranges = 8;
+  const int64_t tiles = (int64_t)exo_ceil_div(N, 128) * exo_ceil_div(M, 128);
+  if (tiles < kQmmSplitTiles) {
+    ranges = 1;
+    while (ranges < 8 && tiles * ranges < 256) ranges *= 2;  // as plan_split
+  }
   if (M <= 64 && N <= kQmmWideMaxN) ranges = std::max<int64_t>(ranges, wide_max_split(N));
   return ranges * (int64_t)part_stride(M, N) * 4;
 }

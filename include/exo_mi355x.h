@@ -107,7 +107,7 @@ int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_weight, float
 int exo_qmm(const uint16_t* x, const uint32_t* w, const uint16_t* scales,
             const uint16_t* biases, const uint16_t* residual, uint16_t* y, int M, int N,
             int K, int bits, int group_size, exo_stream_t stream);
-/* exo_qmm with a workspace for launches of few output tiles (fewer than 128 tiles of
+/* exo_qmm with a workspace for launches of few output tiles (fewer than 256 tiles of
  * 128 x 128: a short prompt, or a narrow matrix such as a MoE router under a long one): the
  * tiles alone do not fill the chip, so K is split over up to 8 workgroups per tile, the
  * float32 partial tiles go to `workspace` and a second small launch adds them in a fixed

@@ -200,7 +200,8 @@ def test_qmm_mfma(device, bits, M, N, K):
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024),
                                    (12, 256, 8192), (9, 96, 1024), (1023, 128, 2048), (300, 200, 4096),
-                                   (32, 520, 512), (64, 600, 1024), (65, 300, 768), (20, 257, 256)])
+                                   (32, 520, 512), (64, 600, 1024), (65, 300, 768), (20, 257, 256),
+                                   (300, 10880, 1024), (1023, 2048, 1024)])
 def test_qmm_split_k(device, bits, M, N, K):
     """Few output tiles (a short input, or a narrow matrix under a long one): K is split
     over workgroups and the float32 partial tiles are added by a second launch.  Against
