@@ -22,6 +22,8 @@
 //  * v_mfma_f32_32x32x16_bf16, float32 accumulators (128x64 per wave); the tile and the
 //    weights of the next K step are requested before the current one is multiplied.
 //  * grouped mode (MoE prefill): blockIdx.y is a tile of one expert's sorted rows.
+//  * 128-row tiles over K ranges of 768 or more: weights and activation chunks of four K
+//    steps in flight in registers (DEEP, below) instead of one step.
 //  * up to 128 rows and few column tiles: blockIdx.z splits K; float32 partial tiles and a
 //    small reduce launch.
 //  * up to 32 rows (64 on matrices of 8192 rows or more): the four waves sit side by side on
@@ -40,6 +42,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace {
 
@@ -164,16 +167,24 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // WIDE (inputs of up to 64 rows): the four waves sit side by side - the workgroup tile is
 // (32*MI) x 256, every wave owns 64 weight rows of its own, so nothing is dequantised twice;
 // blockIdx.z always owns a K range and the tile leaves as a float32 partial.
+// DEEP (128-row tiles with SB4): four K steps of weights and three of activations in flight
+// instead of one.  A 128-row tile holds half the arithmetic per K step of the 256-row one, so
+// with one step in flight a workgroup spends most of a step waiting for the next one's loads,
+// and the whole launch moves (bytes in flight) / (memory latency): 8 KB per workgroup and
+// step, 512 workgroups, 2 us = 2 TB/s, which is what the grouped expert GEMMs of a MoE prompt
+// ran at.
 template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false,
-          bool WIDE = false>
+          bool WIDE = false, bool DEEP = false>
 __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   static_assert(!WIDE || (!GROUPED && !PAIR), "the wide tile is for the plain GEMM");
+  static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
   constexpr int kThreads = 256;
   constexpr int BM = WIDE ? 32 * MI : 64 * MI;
   constexpr int BN = PAIR ? 64 : WIDE ? 256 : 128;  // output columns per workgroup
   constexpr int WN = PAIR ? 32 : 64;                // output columns per wave
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LDS_STRIDE];
+  constexpr int SLOTS = 2;  // activation tiles in LDS
+  __shared__ __attribute__((aligned(16))) bf16_t xs[SLOTS][BM * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -255,6 +266,11 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 #pragma unroll
     for (int r = 0; r < XR; ++r)
       load_to_lds16(rx, tiles + buf * TILE_BYTES + (wave * 64 + kThreads * r) * 16, xoff[r], k0 * 2);
+  };
+  // s_waitcnt vmcnt(n) alone (the other counters at "no wait")
+  auto wait_vm = [](auto n) {
+    constexpr int N = decltype(n)::value;
+    __builtin_amdgcn_s_waitcnt((N & 15) | 0x0F70 | ((N >> 4) << 14));
   };
   auto load_w = [&](WStage& st, int k0) {
 #pragma unroll
@@ -365,21 +381,75 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // this workgroup's K range (all of K unless split; a multiple of four K steps)
   const int kb = GROUPED ? 0 : (int)blockIdx.z * p.kc;
   const int ke = GROUPED ? p.K : min(p.K, kb + p.kc);
+  if (DEEP) {
+    // Four register stages each of weights and of activation chunks, requested four steps
+    // ahead; the activations pass through registers into the two LDS tiles one step ahead
+    // (no LDS-direct loads here: the compiler makes every LDS read wait for ALL outstanding
+    // LDS-direct loads, which would drain the pipeline in every step), so every wait count is
+    // the compiler's own and exact - the loop is straight-line, its last block of four steps
+    // peeled, no request conditional.
+    // Step s: barrier (tile s complete, tile s-1 no longer read); store the chunks of step
+    // s+1 into the other tile; request the chunks of step s+4; multiply; request the weights
+    // of step s+4 into the stage just used.
+    WStage wq[4];
+    uint4 xq[4][XR];
+    SBlock sbc, sbn;
+    auto fetch_x = [&](uint4(&dst)[XR], int k0) {
+#pragma unroll
+      for (int r = 0; r < XR; ++r)
+        dst[r] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[r], k0 * 2, 0));
+    };
+    auto store_x = [&](int buf, const uint4(&src)[XR]) {
+#pragma unroll
+      for (int r = 0; r < XR; ++r)
+        *reinterpret_cast<uint4*>(tiles + buf * TILE_BYTES + (tid + kThreads * r) * 16) = src[r];
+    };
+    load_sb(sbc, kb >> 8);
+    sbn = sbc;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // (a K range is a multiple of four steps)
+      fetch_x(xq[u], kb + u * BK);
+      load_w(wq[u], kb + u * BK);
+    }
+    store_x(0, xq[0]);
+    int k0 = kb;
+    for (; k0 + 4 * BK < ke; k0 += 4 * BK) {
+      load_sb(sbn, (k0 >> 8) + 1);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * BK;
+        __syncthreads();
+        store_x((u + 1) & 1, xq[(u + 1) & 3]);
+        fetch_x(xq[u], k + 4 * BK);
+        multiply(wq[u], u & 1, sbc, u);
+        load_w(wq[u], k + 4 * BK);
+      }
+      sbc = sbn;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // the last block: everything it needs is under way
+      __syncthreads();
+      if (u < 3) store_x((u + 1) & 1, xq[(u + 1) & 3]);
+      multiply(wq[u], u & 1, sbc, u);
+    }
+  }
   WStage w0, w1;
   SBlock sb0, sb1;  // current block of four K steps, next block
-  if (SB4) {
+  if (SB4 && !DEEP) {
     load_sb(sb0, kb >> 8);
     sb1 = sb0;
   }
-  load_x(0, kb);
-  load_w(w0, kb);
+  if (!DEEP) {
+    load_x(0, kb);
+    load_w(w0, kb);
+  }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile is in LDS
   __syncthreads();
   // At K step k: the x tile of k is in LDS buffer k&1 and the packed weights of k in w0.
   // The tile and the weights of k+1 are requested first, then tile k is multiplied; every
   // load of the step has landed before the one barrier that ends it.
   int buf = 0;
-  for (int k0 = kb; k0 < ke; k0 += BK) {
+  for (int k0 = kb; !DEEP && k0 < ke; k0 += BK) {
     const int ks = k0 >> 6;
     if (SB4 && (ks & 3) == 0) {  // a new block: its values arrived during the previous one
       sb0 = sb1;
@@ -500,6 +570,12 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 }
 
 constexpr int kQmmMaxSplit = 16;  // K ranges the reduce kernel adds
+#ifndef EXO_QMM_DEEP_MIN_K
+#define EXO_QMM_DEEP_MIN_K 768
+#endif
+// K range per workgroup from which the 128-row tile runs the four-stage pipeline (shorter
+// ranges never reach its steady state)
+constexpr int kDeepMinK = EXO_QMM_DEEP_MIN_K;
 
 // y = bf16(sum over the K ranges, in order) (+ residual): four outputs per thread
 __global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict__ part,
@@ -615,7 +691,9 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
   // 1023 rows, exactly 128 tall tiles: 93 -> 77 us), not beyond (192 tall tiles: 88 vs 97 us)
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (M <= 128 || small_grid || p.ksplit > 1) {  // (only the 128-row tile splits K)
-    if (sb4)
+    if (sb4 && p.kc >= kDeepMinK)
+      qmm_kernel<BITS, 2, false, true, false, false, true><<<g2, 256, 0, st>>>(p);
+    else if (sb4)
       qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, false, false><<<g2, 256, 0, st>>>(p);
@@ -638,10 +716,14 @@ void launch_grouped(const QmmParams& p, dim3 grid, hipStream_t st) {
   const bool sb4 = p.K % 256 == 0 &&
                    (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
   if (p.w2) {  // (gate, up) pair with the SwiGLU in the epilogue
-    if (sb4)
+    if (sb4 && p.K >= kDeepMinK)
+      qmm_kernel<BITS, 2, true, true, true, false, true><<<grid, 256, 0, st>>>(p);
+    else if (sb4)
       qmm_kernel<BITS, 2, true, true, true><<<grid, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, true, false, true><<<grid, 256, 0, st>>>(p);
+  } else if (sb4 && p.K >= kDeepMinK) {
+    qmm_kernel<BITS, 2, true, true, false, false, true><<<grid, 256, 0, st>>>(p);
   } else if (sb4) {
     qmm_kernel<BITS, 2, true, true><<<grid, 256, 0, st>>>(p);
   } else {
@@ -791,7 +873,9 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
                    (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (p.M <= 128 || small_grid) {
-    if (sb4)
+    if (sb4 && p.K >= kDeepMinK)
+      qmm_kernel<BITS, 2, false, true, true, false, true><<<g2, 256, 0, st>>>(p);
+    else if (sb4)
       qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, false, false, true><<<g2, 256, 0, st>>>(p);
