@@ -205,9 +205,11 @@ class ShardModel:
             if gemv:  # post-attention norm and SwiGLU fused into the gate/up GEMV pair
                 ops.qmv_swiglu(bf.h, L.gate, L.up, out=bf.act, norm_weight=L.post_norm,
                                eps=c.rms_norm_eps)
-            elif R > 128:  # one GEMM launch for both projections, SwiGLU in its epilogue
+            elif R >= 64:  # one GEMM launch for both projections, SwiGLU in its epilogue
                 ops.qmm_swiglu(bf.n, L.gate, L.up, out=bf.act)
-            else:  # short chunks: the split-K GEMM per projection is faster
+            else:  # up to 63 rows: the 256-column split-K GEMM per projection is faster
+                #   (8192x2048 at 126 rows: pair 27 us, two GEMMs + SwiGLU 44 us; at 32 rows 28 / 29
+                #   us; 14336x4096 at 32 rows 58 / 46 us, at 64 rows 57 / 59 us)
                 if bf.gate is None:
                     bf.gate = torch.empty_like(bf.act)
                     bf.up = torch.empty_like(bf.act)
