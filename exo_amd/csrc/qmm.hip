@@ -635,7 +635,7 @@ void plan_split(int M, int N, int K, bool have_ws, int* ksplit, int* kc) {
   const int tiles = exo_ceil_div(N, 128) * exo_ceil_div(M, 128);
   if (tiles >= kQmmSplitTiles) return;
   int ks = 1;
-  while (ks < 8 && tiles * ks < 256 && K / (ks * 2) >= 512) ks *= 2;
+  while (ks < 8 && tiles * ks < 256 && K / (ks * 2) >= 256) ks *= 2;
   if (ks == 1) return;
   int c = exo_ceil_div(K, ks);
   c = (c + 255) / 256 * 256;
