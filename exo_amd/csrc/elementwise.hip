@@ -2,6 +2,7 @@
 // SwiGLU, MoE routing/combination, greedy sampling reductions.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
+#include "route.h"
 
 namespace {
 
@@ -151,74 +152,18 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
 }
 
 // ------------------------------------------------------------------- MoE routing
-// One wave per row; E <= 256 (4 values per lane).  The k selections run on packed keys
-// (bf16 probability bits << 16 | 0xFFFF - expert): one unsigned max per selection finds
-// the largest probability and, among equals, the lowest expert id; the wave maximum is a
-// six-step DPP reduction whose result lands in lane 63.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
-  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false);
-  return o > v ? o : v;
-}
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-  v = dpp_max_u32<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
-  v = dpp_max_u32<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-  v = dpp_max_u32<0x141, 0xf>(v);  // row_half_mirror
-  v = dpp_max_u32<0x140, 0xf>(v);  // row_mirror: every lane holds its row-of-16 maximum
-  v = dpp_max_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v = dpp_max_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
-
+// One wave per row (route.h).
 __global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* __restrict__ logits,
                                                          int32_t* __restrict__ idx,
                                                          bf16_t* __restrict__ scores, int E,
                                                          int k, int renorm) {
   const int row = blockIdx.x, lane = threadIdx.x;
-  float v[4];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int e = lane + 64 * i;
-    v[i] = (e < E) ? bf2f(logits[(size_t)row * E + e]) : -INFINITY;
-    mx = fmaxf(mx, v[i]);
-  }
-  mx = wave_max(mx);
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    v[i] = (lane + 64 * i < E) ? expf(v[i] - mx) : 0.f;
-    sum += v[i];
-  }
-  sum = wave_sum(sum);
-  // probabilities rounded to bf16 (non-negative, so their bit patterns order like the
-  // values); key 0 marks "taken / absent"
-  uint32_t key[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int e = lane + 64 * i;
-    key[i] = (e < E) ? (((uint32_t)f2bf(v[i] / sum) << 16) | (uint32_t)(0xFFFF - e)) : 0u;
-  }
-  float sel[16];
-  float tot = 0.f;
-  for (int j = 0; j < k; ++j) {
-    uint32_t best = key[0];
-#pragma unroll
-    for (int i = 1; i < 4; ++i) best = key[i] > best ? key[i] : best;
-    best = wave_max_u32(best);
-    const int bi = 0xFFFF - (int)(best & 0xFFFFu);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (key[i] == best) key[i] = 0u;
-    const float bv = bf2f((bf16_t)(best >> 16));
-    sel[j] = bv;
-    tot += bv;
-    if (lane == 0) idx[(size_t)row * k + j] = bi;
-  }
-  if (lane == 0) {
-    const float totb = bf2f(f2bf(tot));
-    for (int j = 0; j < k; ++j)
-      scores[(size_t)row * k + j] = renorm ? f2bf(sel[j] / totb) : f2bf(sel[j]);
+  int my_id;
+  float my_p, tot;
+  route_topk_wave(logits + (size_t)row * E, E, k, lane, my_id, my_p, tot);
+  if (lane < k) {
+    idx[(size_t)row * k + lane] = my_id;
+    scores[(size_t)row * k + lane] = route_score(my_p, tot, renorm);
   }
 }
 

@@ -17,6 +17,7 @@
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 #include "qmv_internal.h"
+#include "route.h"
 
 namespace {
 
@@ -43,6 +44,13 @@ struct QmvParams {
   int E, topk, x_rows;
   // the same with ONE matrix: blockIdx.y = row of x and of y (topk = x_rows = 1, idx null)
   int each_row;
+  // gather mode that routes by itself: every wave repeats the softmax + top-k of its token
+  // over route[token, :E] (idx null) and takes the expert of its slot; the first workgroup
+  // of a token's first slot also writes the token's indices and scores out
+  const bf16_t* route;   // [T, E] router logits or null
+  int32_t* route_idx;    // [T*topk]
+  bf16_t* route_scores;  // [T*topk]
+  int route_renorm;
   // fused RMSNorm of the input rows: x <- bf16(x * rsqrt(mean(x^2) + eps) * norm_w)
   const bf16_t* norm_w;  // [K] or null
   float eps;
@@ -300,9 +308,26 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
   size_t ew = 0, eg = 0;
-  if (p.idx || p.each_row) {
+  if (p.idx || p.each_row || p.route) {
     const int pair = blockIdx.y;
-    if (p.idx) {
+    if (p.route) {  // wave 0 repeats the routing of the token, the others wait
+      __shared__ int s_expert;
+      const int t = pair / p.topk, slot = pair - t * p.topk;
+      if (wave == 0) {
+        int my_id;
+        float my_p, tot;
+        route_topk_wave(p.route + (size_t)t * p.E, p.E, p.topk, lane, my_id, my_p, tot);
+        if (blockIdx.x == 0 && slot == 0 && lane < p.topk) {
+          p.route_idx[(size_t)t * p.topk + lane] = my_id;
+          p.route_scores[(size_t)t * p.topk + lane] = route_score(my_p, tot, p.route_renorm);
+        }
+        if (lane == slot) s_expert = my_id;
+      }
+      __syncthreads();
+      const int e = __builtin_amdgcn_readfirstlane(s_expert);
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    } else if (p.idx) {
       int e = p.idx[pair];
       e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
       ew = (size_t)e * p.N * p.wpr;
@@ -504,27 +529,49 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
-  size_t ew = 0, eg = 0;
-  if (p.idx || p.each_row) {
-    const int pair = blockIdx.y;
-    if (p.idx) {
-      int e = p.idx[pair];
-      e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
-      ew = (size_t)e * p.N * p.wpr;
-      eg = (size_t)e * p.N * G;
-    }
+  const int pair = blockIdx.y;  // gather modes: (token, slot) of this workgroup
+  if (p.idx || p.each_row || p.route) {
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
     yout += (size_t)pair * p.N;
   }
   const char* wb[NMAT];
   const char* sb[NMAT];
   const char* bb[NMAT];
+  // Base pointers of this workgroup's matrices.  Gather modes: the expert of its pair.
+  // Routing mode: wave 0 repeats the routing of the token, the others wait at one barrier;
+  // called once the activation loads are on their way, so that their latency covers it.
+  __shared__ int s_expert;
+  auto select_matrices = [&]() {
+    size_t ew = 0, eg = 0;
+    if (p.route) {
+      const int t = pair / p.topk, slot = pair - t * p.topk;
+      if (wave == 0) {
+        int my_id;
+        float my_p, tot;
+        route_topk_wave(p.route + (size_t)t * p.E, p.E, p.topk, lane, my_id, my_p, tot);
+        if (blockIdx.x == 0 && slot == 0 && lane < p.topk) {
+          p.route_idx[(size_t)t * p.topk + lane] = my_id;
+          p.route_scores[(size_t)t * p.topk + lane] = route_score(my_p, tot, p.route_renorm);
+        }
+        if (lane == slot) s_expert = my_id;
+      }
+      __syncthreads();
+      const int e = __builtin_amdgcn_readfirstlane(s_expert);
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    } else if (p.idx) {
+      int e = p.idx[pair];
+      e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    }
 #pragma unroll
-  for (int a = 0; a < NMAT; ++a) {
-    wb[a] = reinterpret_cast<const char*>(p.w[a] + ew);
-    sb[a] = reinterpret_cast<const char*>(p.s[a] + eg);
-    bb[a] = reinterpret_cast<const char*>(p.b[a] + eg);
-  }
+    for (int a = 0; a < NMAT; ++a) {
+      wb[a] = reinterpret_cast<const char*>(p.w[a] + ew);
+      sb[a] = reinterpret_cast<const char*>(p.s[a] + eg);
+      bb[a] = reinterpret_cast<const char*>(p.b[a] + eg);
+    }
+  };
   struct Batch {
     uint4 w[NMAT][UB];
     // (scale, bias) words: a unit pair shares the word of its even unit (low half: even
@@ -665,7 +712,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // the weight loads still outstanding), then two weight batches, then the LDS staging.
   Batch buf[NBUF];
   if (XR) {
-    if (nrows <= 0) return;
+    if (nrows <= 0 && !p.route) return;  // (routing mode: every wave meets the barrier)
     uint4 raw[ITERS][4], nwv[ITERS][4];
 #pragma unroll
     for (int j = 0; j < ITERS; ++j)
@@ -675,6 +722,8 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
         raw[j][t] = load_word_x<BITS>(xin, wi);
         if (p.norm_w) nwv[j][t] = load_word_x<BITS>(p.norm_w, wi);
       }
+    select_matrices();
+    if (nrows <= 0) return;
     issue(buf[0], r0);
     if (p.norm_w) {
       float ss = 0.f;
@@ -709,6 +758,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   } else {
     XStage<BITS, MT, ITERS> xst;
     stage_x_load<BITS, MT, ITERS>(p, xin, xst);
+    select_matrices();
     if (nrows > 0) issue(buf[0], r0);
     __shared__ float s_red[4 * MT];
     stage_x_store<BITS, MT, ITERS>(p, xst, xs, sx, s_red);
@@ -1115,7 +1165,7 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   if (MT == 1 && NMAT == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.norm_w && !p.idx && !p.each_row &&
-      p.M == 1) {
+      !p.route && p.M == 1) {
     // measured against the row kernel: ahead at 14 units per row (8-bit, K = 14336: 17.0
     // vs 18.3 us for 4096 rows), level at 7 and 8, behind at 4
     if (pl.iters == 14) return launch_ksplit<BITS, 14>(p, st);
@@ -1151,6 +1201,11 @@ struct Gather {
   const int32_t* idx = nullptr;
   int pairs = 1, E = 0, topk = 1, x_rows = 1;
   bool each_row = false;  // no indices: `pairs` rows of x against the one matrix
+  // no indices either: the kernel routes from these logits and writes indices and scores
+  const bf16_t* route = nullptr;
+  int32_t* route_idx = nullptr;
+  bf16_t* route_scores = nullptr;
+  int route_renorm = 0;
 };
 
 template <int NMAT>
@@ -1163,7 +1218,7 @@ int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const*
   int m0 = 0;
   while (m0 < M) {
     int mt = (M - m0 >= 4) ? 4 : ((M - m0 >= 2) ? 2 : 1);
-    if (ga.idx || ga.each_row) mt = 1;
+    if (ga.idx || ga.each_row || ga.route) mt = 1;
     Plan pl;
     for (;;) {
       if (!make_plan(N, K, bits, mt, &pl)) {
@@ -1200,9 +1255,13 @@ int qmv_dispatch(const bf16_t* x, const uint32_t* const* w, const bf16_t* const*
     p.topk = ga.topk;
     p.x_rows = ga.x_rows;
     p.each_row = ga.each_row ? 1 : 0;
+    p.route = ga.route;
+    p.route_idx = ga.route_idx;
+    p.route_scores = ga.route_scores;
+    p.route_renorm = ga.route_renorm;
     p.norm_w = norm_w;
     p.eps = eps;
-    const int pairs = (ga.idx || ga.each_row) ? ga.pairs : 1;
+    const int pairs = (ga.idx || ga.each_row || ga.route) ? ga.pairs : 1;
     int rc;
     if (bits == 4) {
       rc = mt == 4   ? launch_one<4, 4, NMAT>(p, pl, pairs, st)
@@ -1460,6 +1519,40 @@ extern "C" int exo_gather_qmv_swiglu(const uint16_t* x, const uint32_t* wg, cons
                                      exo_stream_t stream) {
   return exo_norm_gather_qmv_swiglu(x, nullptr, 0.f, wg, sg, bg, wu, su, bu, idx, y, T, topk, E,
                                     N, K, bits, group_size, stream);
+}
+
+extern "C" int exo_norm_route_gather_qmv_swiglu(
+    const uint16_t* x, const uint16_t* norm_weight, float eps, const uint16_t* router_logits,
+    int renorm, int32_t* idx_out, uint16_t* scores_out, const uint32_t* wg, const uint16_t* sg,
+    const uint16_t* bg, const uint32_t* wu, const uint16_t* su, const uint16_t* bu, uint16_t* y,
+    int T, int topk, int E, int N, int K, int bits, int group_size, exo_stream_t stream) {
+  int rc = check_common("exo_norm_route_gather_qmv_swiglu", 1, N, K, bits, group_size);
+  if (rc) return rc;
+  rc = check_gather("exo_norm_route_gather_qmv_swiglu", T, topk, 1, E);
+  if (rc) return rc;
+  EXO_REQUIRE(x && router_logits && idx_out && scores_out && wg && sg && bg && wu && su && bu && y,
+              "exo_norm_route_gather_qmv_swiglu: null pointer");
+  EXO_REQUIRE(E <= 256 && topk <= 16 && topk <= E,
+              "exo_norm_route_gather_qmv_swiglu: need E<=256, topk<=min(16,E); got E=%d topk=%d", E,
+              topk);
+  if (T == 0) return EXO_OK;
+  const uint32_t* ws[2] = {wg, wu};
+  const bf16_t* ss[2] = {sg, su};
+  const bf16_t* bs[2] = {bg, bu};
+  Gather ga;
+  ga.pairs = T * topk;
+  ga.E = E;
+  ga.topk = topk;
+  ga.x_rows = 1;
+  ga.route = router_logits;
+  ga.route_idx = idx_out;
+  ga.route_scores = scores_out;
+  ga.route_renorm = renorm;
+  rc = qmv_dispatch<2>(x, ws, ss, bs, nullptr, y, 1, N, K, bits, (hipStream_t)stream,
+                       "exo_norm_route_gather_qmv_swiglu", ga, norm_weight, eps);
+  if (rc) return rc;
+  EXO_CHECK_LAUNCH("exo_norm_route_gather_qmv_swiglu");
+  return EXO_OK;
 }
 
 extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, const uint16_t* scales,

@@ -43,6 +43,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_gather_qmv_combine": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "exo_gather_qmv_swiglu": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "exo_norm_gather_qmv_swiglu": (_i, [_vp, _vp, _f] + [_vp] * 8 + [_i] * 7 + [_vp]),
+    "exo_norm_route_gather_qmv_swiglu": (_i, [_vp, _vp, _f, _vp, _i] + [_vp] * 9 + [_i] * 7 + [_vp]),
     "exo_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "exo_rope_kv_append": (_i, [_vp] * 8 + [_f] + [_i] * 6 + [_vp]),
     "exo_sdpa_decode_workspace": (_i64, [_i, _i, _i]),

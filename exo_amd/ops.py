@@ -466,6 +466,31 @@ def gather_qmv_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, idx, out=No
     return out
 
 
+def route_gather_qmv_swiglu(x, router_logits, k: int, renorm: bool, gate: QuantizedWeight,
+                            up: QuantizedWeight, out=None, norm_weight=None, eps: float = 0.0):
+    """router_topk + gather_qmv_swiglu in one launch (decode): x bf16 [T,K], router_logits
+    bf16 [T,E] -> (idx int32 [T,k], scores bf16 [T,k], out [T,k,N])."""
+    lib = native.load()
+    T, K = x.shape
+    E = gate.weight.shape[0]
+    if router_logits.shape != (T, E):
+        raise ValueError(f"router_logits {tuple(router_logits.shape)} != ({T}, {E})")
+    idx = torch.empty(T, k, dtype=torch.int32, device=x.device)
+    sc = torch.empty(T, k, dtype=torch.bfloat16, device=x.device)
+    if out is None:
+        out = torch.empty(T, k, gate.N, dtype=torch.bfloat16, device=x.device)
+    check(
+        lib.exo_norm_route_gather_qmv_swiglu(
+            _ptr(x), _ptr(norm_weight), eps, _ptr(router_logits), int(renorm), _ptr(idx), _ptr(sc),
+            _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
+            _ptr(up.scales), _ptr(up.biases), _ptr(out), T, k, E, gate.N, K, gate.bits,
+            gate.group_size, _stream(),
+        ),
+        "route_gather_qmv_swiglu",
+    )
+    return idx, sc, out
+
+
 # ------------------------------------------------------------------ small ops
 
 

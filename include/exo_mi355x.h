@@ -185,6 +185,20 @@ int exo_norm_gather_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, f
                                const int32_t* idx, uint16_t* y, int T, int topk, int E, int N,
                                int K, int bits, int group_size, exo_stream_t stream);
 
+/* K9+K3+K8 for decode: exo_router_topk and exo_norm_gather_qmv_swiglu in one launch.  Every
+ * wave repeats the routing of its token from router_logits bf16 [T,E] (same arithmetic as
+ * exo_router_topk: E <= 256, topk <= 16) and streams the expert of its slot; idx_out int32
+ * [T,topk] and scores_out bf16 [T,topk] are written for the down projection
+ * (exo_gather_qmv_combine).  (qwen3_moe's gate + SwitchGLU,
+ * .typings/mlx_lm/models/switch_layers.pyi:59-73) */
+int exo_norm_route_gather_qmv_swiglu(const uint16_t* x, const uint16_t* norm_weight, float eps,
+                                     const uint16_t* router_logits, int renorm,
+                                     int32_t* idx_out, uint16_t* scores_out, const uint32_t* wg,
+                                     const uint16_t* sg, const uint16_t* bg, const uint32_t* wu,
+                                     const uint16_t* su, const uint16_t* bu, uint16_t* y, int T,
+                                     int topk, int E, int N, int K, int bits, int group_size,
+                                     exo_stream_t stream);
+
 /* K5: mx.fast.rms_norm with the preceding residual add fused:
  *   h = residual ? bf16(x + residual) : x ;  h_out = h (may be null) ;
  *   n_out = bf16(h * rsqrt(mean(h^2)+eps) * weight).

@@ -304,6 +304,31 @@ def test_gather_qmv_swiglu(device, bits):
     assert_close(got, want, what="gather_qmv_swiglu")
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("E,N,K,T,topk,renorm,norm", [(128, 768, 2048, 1, 8, True, True), (128, 768, 2048, 4, 8, True, True),
+                                                      (60, 64, 2048, 3, 4, False, False), (256, 96, 512, 2, 16, True, True),
+                                                      (7, 200, 768, 5, 3, True, False)])
+def test_route_gather_qmv_swiglu_equals_topk_then_gather(device, bits, E, N, K, T, topk, renorm, norm):
+    """The expert gate/up launch that routes by itself: the indices and scores it writes are
+    those of exo_router_topk bit for bit, its output that of the gather launch given them
+    (row-streaming and generic kernel, with and without the fused norm); indices also against
+    the oracle."""
+    g = rand_quantized(N, K, bits, seed=70 + E, E=E)
+    u = rand_quantized(N, K, bits, seed=71 + E, E=E)
+    logits = rand_bf16((T, E), seed=72 + E, scale=2.0)
+    x = t_bf16(rand_bf16((T, K), seed=73), device)
+    nw = t_bf16(affine.bf16_round(rand_bf16((K,), seed=74) + 1.0), device) if norm else None
+    gq, uq, lt = t_qw(g, bits, device), t_qw(u, bits, device), t_bf16(logits, device)
+    idx0, sc0 = ops.router_topk(lt, topk, renorm)
+    want = ops.gather_qmv_swiglu(x, gq, uq, idx0, norm_weight=nw, eps=1e-5)
+    for _ in range(2):
+        idx, sc, got = ops.route_gather_qmv_swiglu(x, lt, topk, renorm, gq, uq, norm_weight=nw, eps=1e-5)
+        assert torch.equal(idx, idx0)
+        assert torch.equal(sc.view(torch.int16), sc0.view(torch.int16))
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    np.testing.assert_array_equal(idx0.cpu().numpy(), O.router_topk(logits, topk, renorm)[0])
+
+
 def test_bad_arguments_raise(device):
     trip = rand_quantized(64, 128, 4, seed=1)
     qw = t_qw(trip, 4, device)
