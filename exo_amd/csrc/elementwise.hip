@@ -78,37 +78,60 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
 }
 
 // ------------------------------------------------------ RoPE + KV append (+ head norm)
-// One workgroup per token; its four waves take the heads in turn, lane i < D/2 owns the
-// pair (i, i + D/2) of every head - so the angle's sine and cosine (a precise sincosf: the
-// angle reaches thousands of radians) are computed once per token and lane, not per head.
+// blockIdx.x = token, blockIdx.y = a run of 4 * kRopeHeadsPerWave heads; each wave takes
+// kRopeHeadsPerWave heads and requests all of them before it works on the first (a short
+// prompt is one latency chain per wave: 12 heads in turn took 7.9 us at 126 tokens).  Lane
+// i < D/2 owns the pair (i, i + D/2) of every head.  The angle's cosine and sine come from
+// the table ((cos, sin) per position and pair, as the decode step uses) when the position is
+// inside it, else from a precise sincosf (the angle reaches thousands of radians) of the
+// same product - the table holds exactly those values.
+constexpr int kRopeHeadsPerWave = 3;
 __global__ __launch_bounds__(256) void rope_kv_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kc,
     bf16_t* __restrict__ vc, const int32_t* __restrict__ pos, const float* __restrict__ inv_freq,
-    const bf16_t* __restrict__ qn, const bf16_t* __restrict__ kn, float eps, int T, int Hq,
-    int Hkv, int D, int S_max) {
+    const float2* __restrict__ tab, int tab_rows, const bf16_t* __restrict__ qn,
+    const bf16_t* __restrict__ kn, float eps, int T, int Hq, int Hkv, int D, int S_max) {
   const int tok = blockIdx.x;  // b*T + t
   const int b = tok / T, t = tok - b * T;
   const int i = threadIdx.x & 63, wave = threadIdx.x >> 6, half = D >> 1;
   const bool active = i < half;
   const int p = pos[b] + t;
+  const int nh = Hq + 2 * Hkv;  // heads [0,Hq) are q, [Hq,Hq+Hkv) k, then v
+  const int h0 = ((int)blockIdx.y * 4 + wave) * kRopeHeadsPerWave;
+  bf16_t lo[kRopeHeadsPerWave], hi[kRopeHeadsPerWave];
+#pragma unroll
+  for (int u = 0; u < kRopeHeadsPerWave; ++u) {
+    lo[u] = 0;
+    hi[u] = 0;
+    if (active && h0 + u < nh) {
+      const bf16_t* src = qkv + (size_t)tok * nh * D + (size_t)(h0 + u) * D;
+      lo[u] = src[i];
+      hi[u] = src[i + half];
+    }
+  }
   float sn = 0.f, cs = 1.f;
-  if (active) sincosf((float)p * inv_freq[i], &sn, &cs);
-  // heads [0,Hq) are q, [Hq,Hq+Hkv) k, then v
-  for (int head = wave; head < Hq + 2 * Hkv; head += 4) {
-    const bf16_t* src = qkv + (size_t)tok * (Hq + 2 * Hkv) * D + (size_t)head * D;
+  if (active) {
+    if (tab && p < tab_rows) {
+      const float2 v = tab[(size_t)p * half + i];
+      cs = v.x;
+      sn = v.y;
+    } else {
+      sincosf((float)p * inv_freq[i], &sn, &cs);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kRopeHeadsPerWave; ++u) {
+    const int head = h0 + u;
+    if (head >= nh) break;
     if (head >= Hq + Hkv) {  // v: copy into the cache
       if (active && p < S_max) {
         bf16_t* dst = vc + (((size_t)b * Hkv + (head - Hq - Hkv)) * S_max + p) * D;
-        dst[i] = src[i];
-        dst[i + half] = src[i + half];
+        dst[i] = lo[u];
+        dst[i + half] = hi[u];
       }
       continue;
     }
-    float x1 = 0.f, x2 = 0.f;
-    if (active) {
-      x1 = bf2f(src[i]);
-      x2 = bf2f(src[i + half]);
-    }
+    float x1 = bf2f(lo[u]), x2 = bf2f(hi[u]);
     const bool is_q = head < Hq;
     const bf16_t* nw = is_q ? qn : kn;
     if (nw) {  // per-head RMSNorm, rounded to bf16 like a separate rms_norm call
@@ -377,21 +400,34 @@ extern "C" int exo_add_rmsnorm(const uint16_t* x, const uint16_t* residual,
   return EXO_OK;
 }
 
-extern "C" int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
-                                  uint16_t* v_cache, const int32_t* pos, const float* inv_freq,
-                                  const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
-                                  int B, int T, int Hq, int Hkv, int D, int S_max,
-                                  exo_stream_t stream) {
+extern "C" int exo_rope_kv_append_tab(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
+                                      uint16_t* v_cache, const int32_t* pos,
+                                      const float* inv_freq, const float* rope_table,
+                                      int table_rows, const uint16_t* q_norm_w,
+                                      const uint16_t* k_norm_w, float eps, int B, int T, int Hq,
+                                      int Hkv, int D, int S_max, exo_stream_t stream) {
   EXO_REQUIRE(qkv && q_out && k_cache && v_cache && pos && inv_freq,
               "exo_rope_kv_append: null pointer");
   EXO_REQUIRE(B > 0 && T > 0 && Hq > 0 && Hkv > 0 && S_max > 0,
               "exo_rope_kv_append: non-positive size");
   EXO_REQUIRE(D == 64 || D == 128, "exo_rope_kv_append: head_dim %d not supported (64, 128)", D);
-  rope_kv_kernel<<<dim3(B * T), 256, 0, (hipStream_t)stream>>>(
-      qkv, q_out, k_cache, v_cache, pos, inv_freq, q_norm_w, k_norm_w, eps, T, Hq, Hkv, D,
-      S_max);
+  EXO_REQUIRE(!rope_table || table_rows > 0, "exo_rope_kv_append: table without rows");
+  EXO_REQUIRE((int64_t)B * T <= 0x7fffffff / 2, "exo_rope_kv_append: too many tokens");
+  const int runs = exo_ceil_div(Hq + 2 * Hkv, 4 * kRopeHeadsPerWave);
+  rope_kv_kernel<<<dim3(B * T, runs), 256, 0, (hipStream_t)stream>>>(
+      qkv, q_out, k_cache, v_cache, pos, inv_freq, reinterpret_cast<const float2*>(rope_table),
+      table_rows, q_norm_w, k_norm_w, eps, T, Hq, Hkv, D, S_max);
   EXO_CHECK_LAUNCH("exo_rope_kv_append");
   return EXO_OK;
+}
+
+extern "C" int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
+                                  uint16_t* v_cache, const int32_t* pos, const float* inv_freq,
+                                  const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
+                                  int B, int T, int Hq, int Hkv, int D, int S_max,
+                                  exo_stream_t stream) {
+  return exo_rope_kv_append_tab(qkv, q_out, k_cache, v_cache, pos, inv_freq, nullptr, 0, q_norm_w,
+                                k_norm_w, eps, B, T, Hq, Hkv, D, S_max, stream);
 }
 
 extern "C" int exo_swiglu(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n,

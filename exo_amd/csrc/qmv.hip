@@ -282,7 +282,8 @@ __device__ __forceinline__ void unpack_word_r(uint32_t w, uint32_t mask, uint32_
 }
 
 // NMAT == 2: the pair (gate, up) with the SwiGLU epilogue.
-template <int BITS, int MT, int NMAT>
+// ROUTE: the instantiation that can do the routing itself (p.route; MT == 1, the pair only)
+template <int BITS, int MT, int NMAT, bool ROUTE = false>
 __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   extern __shared__ uint4 smem[];
   uint4* xs = smem;
@@ -308,9 +309,9 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
   size_t ew = 0, eg = 0;
-  if (p.idx || p.each_row || p.route) {
+  if (p.idx || p.each_row || (ROUTE && p.route)) {
     const int pair = blockIdx.y;
-    if (p.route) {  // wave 0 repeats the routing of the token, the others wait
+    if (ROUTE && p.route) {  // wave 0 repeats the routing of the token, the others wait
       __shared__ int s_expert;
       const int t = pair / p.topk, slot = pair - t * p.topk;
       if (wave == 0) {
@@ -498,7 +499,7 @@ __global__ __launch_bounds__(kThreads) void qmv_kernel(const QmvParams p) {
 // (u * 64>>GSHIFT elements) linearly: no per-unit address arithmetic beyond a scalar
 // add.  ITERS is a template parameter: the per-row loop, the LDS offsets of x and the
 // point where a row ends are all static.
-template <int BITS, int MT, int NMAT, int ITERS>
+template <int BITS, int MT, int NMAT, int ITERS, bool ROUTE = false>
 __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   extern __shared__ uint4 smem[];
   uint4* xs = smem;
@@ -530,7 +531,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   const bf16_t* xin = p.x;
   bf16_t* yout = p.y;
   const int pair = blockIdx.y;  // gather modes: (token, slot) of this workgroup
-  if (p.idx || p.each_row || p.route) {
+  if (p.idx || p.each_row || (ROUTE && p.route)) {
     xin += (size_t)(p.x_rows == 1 ? pair / p.topk : pair) * p.K;
     yout += (size_t)pair * p.N;
   }
@@ -543,7 +544,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   __shared__ int s_expert;
   auto select_matrices = [&]() {
     size_t ew = 0, eg = 0;
-    if (p.route) {
+    if (ROUTE && p.route) {
       const int t = pair / p.topk, slot = pair - t * p.topk;
       if (wave == 0) {
         int my_id;
@@ -712,7 +713,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // the weight loads still outstanding), then two weight batches, then the LDS staging.
   Batch buf[NBUF];
   if (XR) {
-    if (nrows <= 0 && !p.route) return;  // (routing mode: every wave meets the barrier)
+    if (nrows <= 0 && !(ROUTE && p.route)) return;  // (routing mode: every wave meets the barrier)
     uint4 raw[ITERS][4], nwv[ITERS][4];
 #pragma unroll
     for (int j = 0; j < ITERS; ++j)
@@ -1097,8 +1098,12 @@ bool make_plan(int N, int K, int bits, int mt, Plan* pl) {
 
 template <int BITS, int MT, int NMAT, int ITERS>
 int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
-  auto kern = qmv_rows_kernel<BITS, MT, NMAT, ITERS>;
-  static bool attr_done = false;
+  constexpr bool CAN_ROUTE = MT == 1 && NMAT == 2;
+  const bool route = CAN_ROUTE && p.route;
+  auto kern = route ? qmv_rows_kernel<BITS, MT, NMAT, ITERS, CAN_ROUTE>
+                    : qmv_rows_kernel<BITS, MT, NMAT, ITERS, false>;
+  static bool attr_set[2] = {false, false};
+  bool& attr_done = attr_set[route ? 1 : 0];
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
@@ -1182,8 +1187,11 @@ int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
       default: break;
     }
   }
-  auto kern = qmv_kernel<BITS, MT, NMAT>;
-  static bool attr_done = false;
+  constexpr bool CAN_ROUTE = MT == 1 && NMAT == 2;
+  const bool route = CAN_ROUTE && p.route;
+  auto kern = route ? qmv_kernel<BITS, MT, NMAT, CAN_ROUTE> : qmv_kernel<BITS, MT, NMAT, false>;
+  static bool attr_set[2] = {false, false};
+  bool& attr_done = attr_set[route ? 1 : 0];
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);

@@ -274,7 +274,8 @@ class ShardModel:
                                 rope_tab=self._rope_table(cache.max_seq))
             else:
                 ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
-                                   L.q_norm, L.k_norm, c.rms_norm_eps)
+                                   L.q_norm, L.k_norm, c.rms_norm_eps,
+                                   rope_tab=self._rope_table(cache.max_seq))
                 ops.sdpa_prefill(bf.q, kc, vc, pos, bf.attn, self.scale, B, T, Hq, Hkv, D)
             ops.quantized_matmul(bf.attn, L.o, residual=bf.h, out=bf.h)
             if not mlp_gemv:

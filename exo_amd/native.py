@@ -46,6 +46,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_norm_route_gather_qmv_swiglu": (_i, [_vp, _vp, _f, _vp, _i] + [_vp] * 9 + [_i] * 7 + [_vp]),
     "exo_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "exo_rope_kv_append": (_i, [_vp] * 8 + [_f] + [_i] * 6 + [_vp]),
+    "exo_rope_kv_append_tab": (_i, [_vp] * 7 + [_i] + [_vp] * 2 + [_f] + [_i] * 6 + [_vp]),
     "exo_sdpa_decode_workspace": (_i64, [_i, _i, _i]),
     "exo_sdpa_decode": (_i, [_vp] * 6 + [_f] + [_i] * 5 + [_vp]),
     "exo_sdpa_decode_static": (_i, [_vp] * 5 + [_f] + [_i] * 5 + [_vp]),

@@ -518,14 +518,16 @@ def rms_norm(x, weight, eps: float, out=None):
 
 
 def rope_kv_append(qkv, q_out, k_cache, v_cache, pos, inv_freq, B, T, Hq, Hkv, D,
-                   q_norm_w=None, k_norm_w=None, eps: float = 0.0):
+                   q_norm_w=None, k_norm_w=None, eps: float = 0.0, rope_tab=None):
     """Split fused qkv [B*T,(Hq+2Hkv)*D]; (q/k head norm;) RoPE at pos[b]+t; q -> q_out
-    [B*T,Hq*D]; k,v -> caches [B,Hkv,S_max,D]."""
+    [B*T,Hq*D]; k,v -> caches [B,Hkv,S_max,D].  ``rope_tab`` (from rope_table): the angles'
+    cosines and sines are read from it for positions inside it."""
     lib = native.load()
     S_max = k_cache.shape[2]
     check(
-        lib.exo_rope_kv_append(
+        lib.exo_rope_kv_append_tab(
             _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq),
+            _ptr(rope_tab), 0 if rope_tab is None else rope_tab.shape[0],
             _ptr(q_norm_w), _ptr(k_norm_w), eps, B, T, Hq, Hkv, D, S_max, _stream(),
         ),
         "rope_kv_append",

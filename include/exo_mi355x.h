@@ -222,6 +222,15 @@ int exo_rope_kv_append(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
                        const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps, int B,
                        int T, int Hq, int Hkv, int D, int S_max, exo_stream_t stream);
 
+/* The same with the angles' (cos, sin) read from the table exo_rope_table wrote (float
+ * [table_rows, D/2, 2]) for positions inside it; positions beyond it, or rope_table == NULL,
+ * compute them from inv_freq - the same values either way. */
+int exo_rope_kv_append_tab(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cache,
+                           uint16_t* v_cache, const int32_t* pos, const float* inv_freq,
+                           const float* rope_table, int table_rows, const uint16_t* q_norm_w,
+                           const uint16_t* k_norm_w, float eps, int B, int T, int Hq, int Hkv,
+                           int D, int S_max, exo_stream_t stream);
+
 /* K7 decode: scaled_dot_product_attention for one new token per sequence over the
  * cache, grouped-query: q bf16 [B, Hq*D]; lens int32 [B] = pos[b]+1 valid keys;
  * out bf16 [B, Hq*D].  `workspace`: exo_sdpa_decode_workspace(B,Hq,D) bytes, zeroed ONCE

@@ -388,6 +388,17 @@ def test_rope_kv_append(device, D, Hq, Hkv, qk_norm):
         np.testing.assert_array_equal(n_f32(vc)[b, :, pos[b]:pos[b] + T], v[b].transpose(1, 0, 2))
     # nothing outside the appended window was written
     assert float(n_f32(kc)[0, :, :5].sum()) == 0.0 and float(n_f32(kc)[0, :, 8:].sum()) == 0.0
+    # with the angle table (long enough; too short for the second sequence): the same bits
+    inv_t = torch.from_numpy(inv).to(device)
+    for rows in (S_max, 12):
+        kc2, vc2, q2 = torch.zeros_like(kc), torch.zeros_like(vc), torch.empty_like(q_out)
+        ops.rope_kv_append(
+            t_bf16(qkv, device), q2, kc2, vc2, torch.from_numpy(pos).to(device), inv_t, B, T, Hq, Hkv, D,
+            t_bf16(qn, device) if qk_norm else None, t_bf16(kn, device) if qk_norm else None, 1e-6,
+            rope_tab=ops.rope_table(inv_t, rows, D),
+        )
+        for a, b_ in ((q2, q_out), (kc2, kc), (vc2, vc)):
+            assert torch.equal(a.view(torch.int16), b_.view(torch.int16))
 
 
 @pytest.mark.parametrize("D,Hq,Hkv", [(64, 32, 8), (128, 32, 8), (128, 32, 4), (128, 64, 4), (128, 4, 4)])

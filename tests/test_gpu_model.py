@@ -52,7 +52,11 @@ def ckpt(request, tmp_path_factory, device):
 def test_logits_match_oracle_in_exact_mode(ckpt, device):
     """The same prefill + single-token steps against the oracle's own arithmetic mode:
     un-rounded float32 weights for every matmul, whatever its row count (gemm_rows=None),
-    i.e. without telling the oracle where the matrix-core GEMM rounds its weights to bf16."""
+    i.e. without telling the oracle where the matrix-core GEMM rounds its weights to bf16.
+    Bound: relative RMS <= 2e-2 and at most 1 % of the elements past the elementwise bound,
+    as for the real-shape layers against this mode (the oracle differs from itself by 0.4 %
+    such elements when it rounds its weights; the 8-bit toy model, whose bf16 operand drops
+    the most bits, measures 0.43-0.51 % depending on how K is split, the others <= 0.1 %)."""
     cfg, gm = ckpt["cfg"], ckpt["model"]
     om = OM.ShardModel(ckpt["ocfg"], ckpt["ow"])
     prompt = rng(12).integers(0, cfg.vocab_size, size=40)
@@ -62,7 +66,7 @@ def test_logits_match_oracle_in_exact_mode(ckpt, device):
     if cfg.is_moe:
         tied = _check_tokens(n_f32(got), want, om, "prefill logits, exact oracle")
     else:
-        assert_close_stat(n_f32(got), want, what="prefill logits, exact oracle")
+        assert_close_stat(n_f32(got), want, max_outlier_frac=1e-2, what="prefill logits, exact oracle")
         tied = False
     for step in range(6):
         if tied:
@@ -74,7 +78,8 @@ def test_logits_match_oracle_in_exact_mode(ckpt, device):
         if cfg.is_moe:
             tied = _check_tokens(n_f32(got), want, om, f"decode step {step}, exact oracle")
         else:
-            assert_close_stat(n_f32(got), want, what=f"decode logits step {step}, exact oracle")
+            assert_close_stat(n_f32(got), want, max_outlier_frac=1e-2,
+                              what=f"decode logits step {step}, exact oracle")
 
 
 def test_prefill_and_decode_logits_match_oracle(ckpt, device):
