@@ -71,8 +71,8 @@ def measure_kernels(model, torch, reps: int = 20):
     y_h = torch.empty(1, H, **bf)
     y_i = torch.empty(1, I, **bf)
     y_v = torch.empty(1, c.vocab_size, **bf)
-    def kernel_name(nmat, K):  # template arguments <bits, rows of x, matrices, 1 KiB units per row>
-        return "qmv_rows_kernel<%d,1,%d,%d>" % (c.bits, nmat, K * c.bits // 8 // 1024)
+    def kernel_name(nmat, K):  # template arguments <bits, rows of x, matrices, 1 KiB units per row, self-routing>
+        return "qmv_rows_kernel<%d,1,%d,%d,false>" % (c.bits, nmat, K * c.bits // 8 // 1024)
 
     nw, eps = torch.ones(H, **bf), c.rms_norm_eps
     groups = {
