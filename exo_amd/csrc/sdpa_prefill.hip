@@ -8,12 +8,15 @@
 // The D-operand layout of the first product puts, in lane (query, half), registers that
 // are 8 consecutive keys per 16-key step once the K rows are fed in a permuted order;
 // they are rounded to bf16 and used as the B operand of the second product without any
-// data movement.  V is transposed on its way into LDS (2-byte stores), K goes in as is.
+// data movement.  V is transposed on its way into LDS (2-byte stores), K goes in as is.  (A
+// row-major V tile read back through ds_read_b64_tr_b16 was measured and is slower here:
+// 2046 tokens 100 -> 164 us.)
 //
 // Work split: a wave owns 32 query tokens of ONE query head; the four waves of a
 // workgroup take four consecutive (token tile, head) units of one kv head, so with GQA
 // (4, 8, 16 query heads per kv head) they share every K/V tile they stage.  Key tiles of
-// 64; the next tile's global loads are in flight while the current one is computed.
+// 64 in two LDS buffers: while a tile is computed, the next one goes from registers into the
+// other buffer and the one after that is on its way from memory; one barrier per tile.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 #include "sdpa_internal.h"
@@ -35,6 +38,11 @@ struct FaParams {
 };
 
 template <int D>
+constexpr int fa_lds_bytes() {
+  return 2 * (kBN * (D + kPadK) + D * (kBN + kPadK)) * 2;
+}
+
+template <int D>
 __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   constexpr int STEPS = D / 16;  // MFMA steps over d for S^T
   constexpr int DT = D / 32;     // 32-row tiles of O^T
@@ -42,15 +50,23 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   constexpr int VS = kBN + kPadK;  // LDS row stride of V^T (bf16)
   constexpr int VEC = D / 8;     // 16-byte vectors per K/V row
   constexpr int LOADS = kBN * VEC / 256;
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[kBN * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[D * VS];
+  constexpr int BUF = kBN * KS + D * VS;  // bf16 elements of one (K, V^T) tile pair
+  extern __shared__ __attribute__((aligned(16))) bf16_t fa_lds[];  // [2][BUF]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kq = lane >> 5;
   const int kvh = blockIdx.y, b = blockIdx.z;
-  // heavy (late) token tiles first
-  const int u0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 4;
+  // Heavy (late) token tiles first - but a launch of up to two workgroups per CU is one round
+  // with nothing left to balance it, and the dispatcher hands a CU its second workgroup 256
+  // positions after its first: every other run of 256 then takes the light tiles first, so
+  // that the two workgroups of a CU are a heavy and a light one (2046 tokens, 32 / 8 heads:
+  // 129 -> 109 us; with 2048 launches the same order lost 10 %).
+  const int row = (int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z;
+  const int rows_per_run = max(1, 256 / (int)gridDim.x);
+  const bool one_round = gridDim.x * gridDim.y * gridDim.z <= 512;  // (longer launches balance
+  const bool light_first = one_round && ((row / rows_per_run) & 1);  //  themselves, heavy first)
+  const int u0 = (light_first ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x) * 4;
   const int u = u0 + wave;
   const bool active = u < p.units;
   const int uc = active ? u : p.units - 1;
@@ -78,23 +94,25 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int vi = tid + i * 256;
-      const int key_k = min(kt * kBN + vi / VEC, p.S_max - 1);  // rows past the cache end: masked
-      kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)key_k * D + (vi % VEC) * 8);
+      const int key = min(kt * kBN + vi / VEC, p.S_max - 1);  // rows past the cache end: masked
+      kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)key * D + (vi % VEC) * 8);
       const int key_v = min(kt * kBN + (vi & (kBN - 1)), p.S_max - 1);
       vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)key_v * D + (vi / kBN) * 8);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int buf) {
+    bf16_t* kl = fa_lds + buf * BUF;
+    bf16_t* vl = kl + kBN * KS;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int vi = tid + i * 256;
-      *reinterpret_cast<uint4*>(&k_lds[(vi / VEC) * KS + (vi % VEC) * 8]) = kreg[i];
+      *reinterpret_cast<uint4*>(&kl[(vi / VEC) * KS + (vi % VEC) * 8]) = kreg[i];
       const int key = vi & (kBN - 1), c = vi / kBN;
       const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        vt_lds[(c * 8 + 2 * j) * VS + key] = (bf16_t)(w[j] & 0xFFFFu);
-        vt_lds[(c * 8 + 2 * j + 1) * VS + key] = (bf16_t)(w[j] >> 16);
+        vl[(c * 8 + 2 * j) * VS + key] = (bf16_t)(w[j] & 0xFFFFu);
+        vl[(c * 8 + 2 * j + 1) * VS + key] = (bf16_t)(w[j] >> 16);
       }
     }
   };
@@ -112,13 +130,19 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   float m_run = -INFINITY, l_run = 0.f;
 
   load_tile(0);
+  store_tile(0);
+  if (n_tiles > 1) load_tile(1);
   for (int kt = 0; kt < n_tiles; ++kt) {
-    __syncthreads();  // every wave is done reading the previous tile
-    store_tile();
+    // tile kt is complete in its buffer, and every wave is done reading the other buffer
     __syncthreads();
-    if (kt + 1 < n_tiles) load_tile(kt + 1);
+    if (kt + 1 < n_tiles) {
+      store_tile((kt + 1) & 1);
+      if (kt + 2 < n_tiles) load_tile(kt + 2);
+    }
     const int key0 = kt * kBN;
     if (key0 > last_w) continue;  // wave-uniform: nothing visible to this wave's rows
+    const bf16_t* k_lds = fa_lds + (kt & 1) * BUF;
+    const bf16_t* v_lds = k_lds + kBN * KS;
 
     // ---- S^T = K Q^T for the two 32-key sub-tiles
     floatx16 s[2];
@@ -181,7 +205,7 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
-      const bf16_t* vr = &vt_lds[(dt * 32 + n) * VS + kq * 8];
+      const bf16_t* vr = &v_lds[(dt * 32 + n) * VS + kq * 8];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -228,9 +252,20 @@ int exo_sdpa_prefill_mfma(const bf16_t* q, const bf16_t* k_cache, const bf16_t* 
   p.G = Hq / Hkv;
   p.units = ((T + kBM - 1) / kBM) * p.G;
   const dim3 grid((p.units + 3) / 4, Hkv, B);
+  static bool attr_done = false;  // 70 KiB of LDS for D = 128: above the default limit
+  if (!attr_done) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_prefill_kernel<128>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             fa_lds_bytes<128>());
+    if (e != hipSuccess) {
+      exo_set_error("exo_sdpa_prefill: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+      return EXO_ERR_HIP;
+    }
+    attr_done = true;
+  }
   if (D == 64)
-    fa_prefill_kernel<64><<<grid, 256, 0, stream>>>(p);
+    fa_prefill_kernel<64><<<grid, 256, fa_lds_bytes<64>(), stream>>>(p);
   else
-    fa_prefill_kernel<128><<<grid, 256, 0, stream>>>(p);
+    fa_prefill_kernel<128><<<grid, 256, fa_lds_bytes<128>(), stream>>>(p);
   return EXO_OK;
 }
