@@ -466,19 +466,22 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     buf ^= 1;
   }
 
-  if (WIDE || (!GROUPED && !PAIR && p.ksplit > 1)) {
+  if (WIDE || (!GROUPED && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
-    // small launch adds the ranges in a fixed order (qmm_reduce_kernel)
-    float* mine = p.part + (size_t)blockIdx.z * part_stride(p.M, p.N);
+    // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
+    // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
+    const size_t one = part_stride(p.M, p.N);
+    float* mine = p.part + (size_t)blockIdx.z * (PAIR ? 2 * one : one);
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int n = n0 + wn + j * 32 + frow;
+        const int n = PAIR ? n0 + wn + frow : n0 + wn + j * 32 + frow;
+        float* dst = mine + ((PAIR && j) ? one : 0);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + wm + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
-          if (m < m_end && n < p.N) mine[(size_t)m * p.N + n] = acc[i][j][r];
+          if (m < m_end && n < p.N) dst[(size_t)m * p.N + n] = acc[i][j][r];
         }
       }
     return;
@@ -618,6 +621,44 @@ __global__ __launch_bounds__(256) void qmm_reduce_kernel(const float* __restrict
       if (residual) t += bf2f(residual[e]);
       y[e] = f2bf(t);
     }
+  }
+}
+
+// Pair mode: sums of the gate and of the up partials, each rounded to bf16 as the projections
+// of two GEMMs would be, then SwiGLU.  `stride` floats between K ranges, `half` between the
+// gate and the up partials of one range.
+__global__ __launch_bounds__(256) void qmm_reduce_swiglu_kernel(const float* __restrict__ part,
+                                                                bf16_t* __restrict__ y,
+                                                                int64_t total, int64_t stride,
+                                                                int64_t half, int ksplit) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  const int cnt = (int)min((int64_t)4, total - i);
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+  if (cnt == 4) {  // (rows of partials start at multiples of four floats)
+    float4 gv[8], uv[8];
+#pragma unroll
+    for (int z = 0; z < 8; ++z)
+      if (z < ksplit) {
+        gv[z] = *reinterpret_cast<const float4*>(part + (size_t)z * stride + i);
+        uv[z] = *reinterpret_cast<const float4*>(part + (size_t)z * stride + half + i);
+      }
+#pragma unroll
+    for (int z = 0; z < 8; ++z)
+      if (z < ksplit) {
+        g[0] += gv[z].x; g[1] += gv[z].y; g[2] += gv[z].z; g[3] += gv[z].w;
+        u[0] += uv[z].x; u[1] += uv[z].y; u[2] += uv[z].z; u[3] += uv[z].w;
+      }
+  } else {
+    for (int e = 0; e < cnt; ++e)
+      for (int z = 0; z < ksplit; ++z) {
+        g[e] += part[(size_t)z * stride + i + e];
+        u[e] += part[(size_t)z * stride + half + i + e];
+      }
+  }
+  for (int e = 0; e < cnt; ++e) {
+    const float gb = bf2f(f2bf(g[e])), ub = bf2f(f2bf(u[e]));
+    y[i + e] = f2bf(gb / (1.f + __expf(-gb)) * ub);
   }
 }
 
@@ -866,19 +907,51 @@ extern "C" int exo_gather_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate,
                          x_rows, E, N, K, bits, group_size, stream);
 }
 
+// K ranges of a pair launch of up to 128 rows whose 128 x 64 output tiles (of the pair) leave
+// half of the chip or more idle - the MLP of a small model under a short prompt (8192 x 2048
+// pair at 126 rows: 128 tiles): ranges of four K steps or more until the launch has up to
+// one workgroup per CU; a second launch adds the ranges and applies the SwiGLU.
+int pair_max_split(int M, int N) {
+  if (M > 128) return 1;
+  const int64_t tiles = (int64_t)exo_ceil_div(N, 64) * exo_ceil_div(M, 128);
+  int ks = 1;
+  while (ks < 8 && tiles * ks * 2 <= 256) ks *= 2;
+  return ks;
+}
+
+void plan_pair_split(const QmmParams& p, bool have_ws, int* ksplit, int* kc) {
+  *ksplit = 1;
+  *kc = p.K;
+  if (!have_ws || p.K % 256 != 0) return;
+  const int cap = pair_max_split(p.M, p.N);
+  int ks = 1;
+  while (ks < cap && p.K / (ks * 2) >= 256) ks *= 2;
+  if (ks == 1) return;
+  int c = exo_ceil_div(p.K, ks);
+  c = (c + 255) / 256 * 256;
+  *kc = c;
+  *ksplit = exo_ceil_div(p.K, c);
+}
+
 template <int BITS>
 void launch_pair(const QmmParams& p, hipStream_t st) {
-  const dim3 g2(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 128)), g4(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 256));
+  const dim3 g2(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 128), p.ksplit),
+      g4(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 256));
   const bool sb4 = p.K % 256 == 0 &&
                    (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (p.M <= 128 || small_grid) {
-    if (sb4 && p.K >= kDeepMinK)
+    if (sb4 && p.kc >= kDeepMinK)
       qmm_kernel<BITS, 2, false, true, true, false, true><<<g2, 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, false, false, true><<<g2, 256, 0, st>>>(p);
+    if (p.ksplit > 1) {
+      const int64_t total = (int64_t)p.M * p.N, one = (int64_t)part_stride(p.M, p.N);
+      qmm_reduce_swiglu_kernel<<<dim3(exo_ceil_div(exo_ceil_div(total, 4), 256)), 256, 0, st>>>(
+          p.part, p.y, total, 2 * one, one, p.ksplit);
+    }
   } else {
     if (sb4)
       qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
@@ -887,10 +960,18 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
   }
 }
 
-extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
-                              const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
-                              const uint16_t* b_up, uint16_t* y, int M, int N, int K, int bits,
-                              int group_size, exo_stream_t stream) {
+extern "C" int64_t exo_qmm_swiglu_workspace(int M, int N) {
+  if (M <= 0 || N <= 0) return 0;
+  const int ks = pair_max_split(M, N);
+  return ks > 1 ? (int64_t)ks * 2 * (int64_t)part_stride(M, N) * 4 : 0;
+}
+
+extern "C" int exo_qmm_swiglu_ws(const uint16_t* x, const uint32_t* w_gate,
+                                 const uint16_t* s_gate, const uint16_t* b_gate,
+                                 const uint32_t* w_up, const uint16_t* s_up,
+                                 const uint16_t* b_up, uint16_t* y, void* workspace,
+                                 int64_t workspace_bytes, int M, int N, int K, int bits,
+                                 int group_size, exo_stream_t stream) {
   EXO_REQUIRE(bits == 4 || bits == 8, "exo_qmm_swiglu: bits must be 4 or 8, got %d", bits);
   EXO_REQUIRE(group_size == 64, "exo_qmm_swiglu: group_size must be 64, got %d", group_size);
   EXO_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 64 == 0, "exo_qmm_swiglu: bad shape M=%d N=%d K=%d",
@@ -901,23 +982,37 @@ extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const u
   EXO_REQUIRE(exo_ceil_div(M, 128) <= 65535, "exo_qmm_swiglu: M=%d too large", M);
   EXO_REQUIRE((int64_t)M * K < (1ll << 31),
               "exo_qmm_swiglu: M*K=%lld exceeds 32-bit byte offsets", (long long)M * K);
+  if (exo_qmm_swiglu_workspace(M, N) == 0) workspace = nullptr;
+  EXO_REQUIRE(!workspace || (workspace_bytes >= exo_qmm_swiglu_workspace(M, N) &&
+                             ((uintptr_t)workspace & 255) == 0),
+              "exo_qmm_swiglu_ws: workspace of %lld bytes, need %lld (256-byte aligned)",
+              (long long)workspace_bytes, (long long)exo_qmm_swiglu_workspace(M, N));
   QmmParams p{x, w_gate, s_gate, b_gate, nullptr, y, M, N, K};
   p.sorted = nullptr;
   p.tiles = nullptr;
   p.x_div = 1;
   p.w_stride = p.s_stride = 0;
-  p.ksplit = 1;
-  p.kc = K;
-  p.part = nullptr;
   p.w2 = w_up;
   p.s2 = s_up;
   p.b2 = b_up;
+  const bool sb4 = K % 256 == 0 &&
+                   (((uintptr_t)s_gate | (uintptr_t)b_gate | (uintptr_t)s_up | (uintptr_t)b_up) & 7) == 0;
+  plan_pair_split(p, workspace != nullptr && sb4, &p.ksplit, &p.kc);
+  p.part = reinterpret_cast<float*>(workspace);
   if (bits == 4)
     launch_pair<4>(p, (hipStream_t)stream);
   else
     launch_pair<8>(p, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_qmm_swiglu");
   return EXO_OK;
+}
+
+extern "C" int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
+                              const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
+                              const uint16_t* b_up, uint16_t* y, int M, int N, int K, int bits,
+                              int group_size, exo_stream_t stream) {
+  return exo_qmm_swiglu_ws(x, w_gate, s_gate, b_gate, w_up, s_up, b_up, y, nullptr, 0, M, N, K,
+                           bits, group_size, stream);
 }
 
 extern "C" int64_t exo_qmm_workspace(int M, int N) {

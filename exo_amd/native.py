@@ -39,6 +39,8 @@ SIGNATURES: dict[str, tuple] = {
     "exo_qmm_workspace": (_i64, [_i, _i]),
     "exo_qmm_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "exo_qmm_swiglu": (_i, [_vp] * 8 + [_i, _i, _i, _i, _i, _vp]),
+    "exo_qmm_swiglu_workspace": (_i64, [_i, _i]),
+    "exo_qmm_swiglu_ws": (_i, [_vp] * 9 + [_i64, _i, _i, _i, _i, _i, _vp]),
     "exo_gather_qmv": (_i, [_vp] * 6 + [_i] * 8 + [_vp]),
     "exo_gather_qmv_combine": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "exo_gather_qmv_swiglu": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),

@@ -176,11 +176,12 @@ def qmv_workspace(N: int, device) -> torch.Tensor:
 _QMM_WS: dict[int, list[torch.Tensor]] = {}
 
 
-def qmm_workspace(M: int, N: int, device) -> torch.Tensor | None:
-    """Split-K workspace of the GEMM for launches of few output tiles (None for the others),
-    one per device, grown on demand; a replaced buffer stays alive (a captured graph may still
-    point at it)."""
-    need = native.load().exo_qmm_workspace(M, N)
+def qmm_workspace(M: int, N: int, device, pair: bool = False) -> torch.Tensor | None:
+    """Split-K workspace of the GEMM (``pair``: of the gate/up pair GEMM) for launches of few
+    output tiles (None for the others), one per device, grown on demand; a replaced buffer
+    stays alive (a captured graph may still point at it)."""
+    lib = native.load()
+    need = lib.exo_qmm_swiglu_workspace(M, N) if pair else lib.exo_qmm_workspace(M, N)
     if need == 0:
         return None
     key = torch.device(device).index or 0
@@ -262,19 +263,23 @@ def quantized_matmul(
     return out
 
 
-def qmm_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None) -> torch.Tensor:
-    """silu(x @ gate^T) * (x @ up^T) on the matrix cores, one launch (any M)."""
+def qmm_swiglu(x, gate: QuantizedWeight, up: QuantizedWeight, out=None,
+               split_k: bool = True) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) on the matrix cores (any M): one launch, or a K-split
+    launch plus a reduce + SwiGLU launch where few output tiles would leave the chip idle
+    (``split_k=False``: never)."""
     lib = native.load()
     M, K = x.shape
     if K != gate.K or gate.K != up.K or gate.N != up.N or gate.bits != up.bits:
         raise ValueError("qmm_swiglu: gate and up must have the same shape and bits as x's K")
     if out is None:
         out = torch.empty(M, gate.N, dtype=torch.bfloat16, device=x.device)
+    ws = qmm_workspace(M, gate.N, x.device, pair=True) if split_k else None
     check(
-        lib.exo_qmm_swiglu(
+        lib.exo_qmm_swiglu_ws(
             _ptr(x), _ptr(gate.weight), _ptr(gate.scales), _ptr(gate.biases), _ptr(up.weight),
-            _ptr(up.scales), _ptr(up.biases), _ptr(out), M, gate.N, K, gate.bits,
-            gate.group_size, _stream(),
+            _ptr(up.scales), _ptr(up.biases), _ptr(out), _ptr(ws), 0 if ws is None else ws.numel(),
+            M, gate.N, K, gate.bits, gate.group_size, _stream(),
         ),
         "qmm_swiglu",
     )

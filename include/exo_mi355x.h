@@ -131,6 +131,19 @@ int exo_qmm_swiglu(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_
                    const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
                    const uint16_t* b_up, uint16_t* y, int M, int N, int K, int bits,
                    int group_size, exo_stream_t stream);
+/* exo_qmm_swiglu with a workspace, for inputs of up to 128 rows whose output tiles leave
+ * half of the chip or more idle (the MLP of a small model under a short prompt): K is split
+ * over up to 8 workgroups per tile, the float32 partials of both projections go to
+ * `workspace` and a second small launch adds them in a fixed order, rounds each projection to
+ * bf16 and applies the SwiGLU.  exo_qmm_swiglu_workspace(M, N) bytes (0: this shape never
+ * splits), 256-byte aligned, no initialisation needed; launches that share it must be ordered
+ * on one stream.  workspace == NULL behaves like exo_qmm_swiglu. */
+int64_t exo_qmm_swiglu_workspace(int M, int N);
+int exo_qmm_swiglu_ws(const uint16_t* x, const uint32_t* w_gate, const uint16_t* s_gate,
+                      const uint16_t* b_gate, const uint32_t* w_up, const uint16_t* s_up,
+                      const uint16_t* b_up, uint16_t* y, void* workspace,
+                      int64_t workspace_bytes, int M, int N, int K, int bits, int group_size,
+                      exo_stream_t stream);
 
 /* K3 for prefill-sized T: the same operator as exo_gather_qmv on the matrix cores.  The
  * (token, slot) pairs are first sorted by expert (exo_moe_group, once per routing

@@ -188,6 +188,27 @@ def test_qmm_swiglu_pair(device, bits, M, N, K):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(126, 8192, 2048), (40, 256, 1024), (100, 100, 768), (128, 4100, 4096), (17, 64, 512)])
+def test_qmm_swiglu_pair_split_k(device, bits, M, N, K):
+    """The pair GEMM of a short input with K split over workgroups (partials of both
+    projections, then one reduce + SwiGLU launch): against the oracle, and against the unsplit
+    launch (same rounding points, the float32 sums in another order), twice in a row on the
+    shared workspace."""
+    g = rand_quantized(N, K, bits, seed=N + 21)
+    u = rand_quantized(N, K, bits, seed=N + 22)
+    x = rand_bf16((M, K), seed=M + K + 1)
+    gq, uq, xt = t_qw(g, bits, device), t_qw(u, bits, device), t_bf16(x, device)
+    assert native.load().exo_qmm_swiglu_workspace(M, N) > 0
+    one = ops.qmm_swiglu(xt, gq, uq, split_k=False)
+    want = O.swiglu(affine.qmm(x, *g, 64, bits), affine.qmm(x, *u, 64, bits))
+    for _ in range(2):
+        got = ops.qmm_swiglu(xt, gq, uq)
+        assert_close_stat(n_f32(got), want, max_outlier_frac=1e-5, what="qmm_swiglu split-K")
+        assert_close_stat(n_f32(got), n_f32(one), max_outlier_frac=1e-4, what="split-K vs one launch")
+        ops.qmm(xt, gq)  # another user of the workspace pool in between
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("M,N,K", [(128, 256, 512), (33, 130, 192), (257, 128, 1024), (17, 64, 64)])
 def test_qmm_mfma(device, bits, M, N, K):
     trip = rand_quantized(N, K, bits, seed=M + N)
