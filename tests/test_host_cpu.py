@@ -7,6 +7,8 @@ import re
 from pathlib import Path
 
 import numpy as np
+import ctypes as C
+
 import pytest
 import torch
 
@@ -55,6 +57,24 @@ def test_argument_errors_without_gpu():
     assert lib.exo_sdpa_decode_static(None, None, None, None, None, 1.0, 9, 32, 8, 128, 64, None) == -1
     assert b"exceed the static scratch" in lib.exo_last_error()
     assert lib.exo_sdpa_decode_workspace(2, 32, 128) == (2 * 32 * 16 * 130 + 2 * 32) * 4
+    # the expert launch that routes by itself: the limits of exo_router_topk
+    one = C.c_void_p(1)  # any non-null pointer: rejected before it is ever used
+    rc = lib.exo_norm_route_gather_qmv_swiglu(one, None, 0.0, one, 1, one, one, one, one, one, one, one, one,
+                                              one, 1, 8, 300, 64, 2048, 4, 64, None)
+    assert rc == -1 and b"E<=256" in lib.exo_last_error()
+    # RoPE with a table but no rows; head_dim outside {64, 128}
+    assert lib.exo_rope_kv_append_tab(one, one, one, one, one, one, one, 0, None, None, 0.0, 1, 1, 8, 2, 128,
+                                      16, None) == -1
+    assert b"table without rows" in lib.exo_last_error()
+    assert lib.exo_rope_kv_append_tab(one, one, one, one, one, one, None, 0, None, None, 0.0, 1, 1, 8, 2, 96,
+                                      16, None) == -1
+    # pair GEMM: the K-split workspace is sized per shape, 0 where the launch never splits
+    assert lib.exo_qmm_swiglu_workspace(126, 8192) == 2 * 2 * 126 * 8192 * 4
+    assert lib.exo_qmm_swiglu_workspace(126, 4096) == 4 * 2 * 126 * 4096 * 4  # 64 tiles: four ranges
+    assert lib.exo_qmm_swiglu_workspace(129, 8192) == 0 and lib.exo_qmm_swiglu_workspace(126, 14336) == 0
+    rc = lib.exo_qmm_swiglu_ws(one, one, one, one, one, one, one, one, C.c_void_p(256), 16, 126, 8192, 2048,
+                               4, 64, None)
+    assert rc == -1 and b"workspace of 16 bytes" in lib.exo_last_error()
     with pytest.raises(ValueError):
         native.check(-1, "x")
 
