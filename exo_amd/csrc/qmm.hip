@@ -164,9 +164,11 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // PAIR: the workgroup's 128 weight rows are 64 rows of the gate matrix and the same 64 rows
 // of the up matrix - a wave's two column tiles are (gate, up) of the same 32 output columns,
 // so the SwiGLU happens in the epilogue and neither projection is written to memory.
-// WIDE (inputs of up to 64 rows): the four waves sit side by side - the workgroup tile is
-// (32*MI) x 256, every wave owns 64 weight rows of its own, so nothing is dequantised twice;
-// blockIdx.z always owns a K range and the tile leaves as a float32 partial.
+// WIDE: the four waves sit side by side - the workgroup tile is (32*MI) x 256 weight rows,
+// every wave owns 64 of them, so nothing is dequantised twice.  Plain GEMM (inputs of up to
+// 64 rows): blockIdx.z always owns a K range and the tile leaves as a float32 partial.
+// Grouped GEMM (MI = 4: the expert's 128-row tile against 256 weight rows, the wave tile of
+// the 256-row kernel): whole K, the usual epilogue.
 // DEEP (128-row tiles with SB4): four K steps of weights and three of activations in flight
 // instead of one.  A 128-row tile holds half the arithmetic per K step of the 256-row one, so
 // with one step in flight a workgroup spends most of a step waiting for the next one's loads,
@@ -176,15 +178,17 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false,
           bool WIDE = false, bool DEEP = false>
 __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
-  static_assert(!WIDE || (!GROUPED && !PAIR), "the wide tile is for the plain GEMM");
+  static_assert(!WIDE || GROUPED || !PAIR, "the wide pair tile is for the grouped GEMM");
   static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
   constexpr int kThreads = 256;
   constexpr int BM = WIDE ? 32 * MI : 64 * MI;
-  constexpr int BN = PAIR ? 64 : WIDE ? 256 : 128;  // output columns per workgroup
-  constexpr int WN = PAIR ? 32 : 64;                // output columns per wave
+  constexpr int WN = PAIR ? 32 : 64;              // output columns per wave
+  constexpr int BN = WIDE ? 4 * WN : 2 * WN;      // output columns per workgroup
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   constexpr int SLOTS = 2;  // activation tiles in LDS
-  __shared__ __attribute__((aligned(16))) bf16_t xs[SLOTS][BM * LDS_STRIDE];
+  // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
+  constexpr int XS_ROWS = (WIDE && GROUPED && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[SLOTS][XS_ROWS * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -466,7 +470,7 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     buf ^= 1;
   }
 
-  if (WIDE || (!GROUPED && p.ksplit > 1)) {
+  if ((WIDE && !GROUPED) || (!GROUPED && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
     // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
@@ -573,6 +577,10 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
 }
 
 constexpr int kQmmMaxSplit = 16;  // K ranges the reduce kernel adds
+#ifndef EXO_QMM_GROUPED_WIDE
+#define EXO_QMM_GROUPED_WIDE 1
+#endif
+constexpr bool kGroupedWide = EXO_QMM_GROUPED_WIDE != 0;
 #ifndef EXO_QMM_DEEP_MIN_K
 #define EXO_QMM_DEEP_MIN_K 768
 #endif
@@ -753,10 +761,23 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
 }
 
 template <int BITS>
-void launch_grouped(const QmmParams& p, dim3 grid, hipStream_t st) {
+void launch_grouped(const QmmParams& p, int row_tiles, hipStream_t st) {
   const bool sb4 = p.K % 256 == 0 &&
                    (((uintptr_t)p.s | (uintptr_t)p.b | (uintptr_t)p.s2 | (uintptr_t)p.b2) & 7) == 0;
-  if (p.w2) {  // (gate, up) pair with the SwiGLU in the epilogue
+  const bool pair = p.w2 != nullptr;  // (gate, up) with the SwiGLU in the epilogue
+  // Four waves side by side on 256 weight rows per workgroup and K step instead of 2 x 2 on
+  // 128: the expert matrices are streamed once per 128-row tile whatever the tile's width, and
+  // a wave of the 2 x 2 layout dequantises the same 64 weight rows as its neighbour.
+  if (sb4 && kGroupedWide) {
+    const dim3 grid(exo_ceil_div(p.N, pair ? 128 : 256), row_tiles);
+    if (pair)
+      qmm_kernel<BITS, 4, true, true, true, true><<<grid, 256, 0, st>>>(p);
+    else
+      qmm_kernel<BITS, 4, true, true, false, true><<<grid, 256, 0, st>>>(p);
+    return;
+  }
+  const dim3 grid(exo_ceil_div(p.N, pair ? 64 : 128), row_tiles);
+  if (pair) {
     if (sb4 && p.K >= kDeepMinK)
       qmm_kernel<BITS, 2, true, true, true, false, true><<<grid, 256, 0, st>>>(p);
     else if (sb4)
@@ -879,11 +900,10 @@ static int gather_qmm_impl(const uint16_t* x, const uint32_t* w, const uint16_t*
   p.w2 = w2;
   p.s2 = s2;
   p.b2 = b2;
-  const dim3 grid(exo_ceil_div(N, w2 ? 64 : 128), max_tiles);
   if (bits == 4)
-    launch_grouped<4>(p, grid, (hipStream_t)stream);
+    launch_grouped<4>(p, max_tiles, (hipStream_t)stream);
   else
-    launch_grouped<8>(p, grid, (hipStream_t)stream);
+    launch_grouped<8>(p, max_tiles, (hipStream_t)stream);
   EXO_CHECK_LAUNCH("exo_gather_qmm");
   return EXO_OK;
 }
