@@ -797,7 +797,7 @@ constexpr int kGroupBM = 128;  // rows per tile of the grouped GEMM
 constexpr int kGroupMaxE = 256;
 
 // Sort the (token, slot) pairs by expert and cut every expert's run into tiles of
-// kGroupBM rows.  One workgroup: counts in LDS, a serial scan over the experts, a second
+// kGroupBM rows.  One workgroup: counts in LDS, a wave's scan over the experts, a second
 // pass that scatters the pair indices.  The order inside an expert's run depends on
 // atomic arrival order; every output row is computed independently of its tile position,
 // so results do not.
@@ -814,16 +814,41 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
     if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
   }
   __syncthreads();
-  if (tid == 0) {
-    int o = 0, t = 0;
-    for (int e = 0; e < E; ++e) {
-      off[e] = o;
-      cur[e] = o;
-      tile0[e] = t;
-      o += cnt[e];
-      t += (cnt[e] + kGroupBM - 1) / kGroupBM;
+  if (tid < 64) {
+    // exclusive scans of the counts and of the tile counts over the experts by one wave:
+    // lane l owns experts [4l, 4l+4) (E <= 256); a scan over one thread's loop of dependent
+    // LDS accesses took 5 of this launch's 10.8 us at 128 experts
+    int c[4], o = 0, t = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 4 * tid + j;
+      c[j] = e < E ? cnt[e] : 0;
+      o += c[j];
+      t += (c[j] + kGroupBM - 1) / kGroupBM;
     }
-    tile0[E] = t;
+    int po = o, pt = t;  // inclusive prefix over the lanes
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int uo = __shfl_up(po, d, 64), ut = __shfl_up(pt, d, 64);
+      if (tid >= d) {
+        po += uo;
+        pt += ut;
+      }
+    }
+    o = po - o;  // exclusive
+    t = pt - t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 4 * tid + j;
+      if (e < E) {
+        off[e] = o;
+        cur[e] = o;
+        tile0[e] = t;
+      }
+      o += c[j];
+      t += (c[j] + kGroupBM - 1) / kGroupBM;
+    }
+    if (tid == 63) tile0[E] = pt;
   }
   __syncthreads();
   for (int i = tid; i < P; i += 1024) {
