@@ -175,12 +175,19 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // and the whole launch moves (bytes in flight) / (memory latency): 8 KB per workgroup and
 // step, 512 workgroups, 2 us = 2 TB/s, which is what the grouped expert GEMMs of a MoE prompt
 // ran at.
+// KH (the 256-row tile of the plain GEMM): eight waves, two teams of four that each run the
+// kernel's loop over one half of K on tiles of their own; at the end the second team's
+// accumulators pass through LDS and are added to the first's, which writes the tile out.  A
+// launch of one such tile per CU has two waves per SIMD where four-wave workgroups would leave
+// one, without partial tiles in memory.
 template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false,
-          bool WIDE = false, bool DEEP = false>
-__global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
+          bool WIDE = false, bool DEEP = false, bool KH = false>
+__global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const QmmParams p) {
   static_assert(!WIDE || GROUPED || !PAIR, "the wide pair tile is for the grouped GEMM");
   static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
-  constexpr int kThreads = 256;
+  static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !PAIR && !WIDE && !DEEP),
+                "two K halves per workgroup: the plain 256-row tile only");
+  constexpr int kThreads = 256;  // of a team
   constexpr int BM = WIDE ? 32 * MI : 64 * MI;
   constexpr int WN = PAIR ? 32 : 64;              // output columns per wave
   constexpr int BN = WIDE ? 4 * WN : 2 * WN;      // output columns per workgroup
@@ -188,9 +195,10 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   constexpr int SLOTS = 2;  // activation tiles in LDS
   // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
   constexpr int XS_ROWS = (WIDE && GROUPED && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[SLOTS][XS_ROWS * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[KH ? 2 * SLOTS : SLOTS][XS_ROWS * LDS_STRIDE];
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x & (kThreads - 1), lane = tid & 63;  // within the team
+  const int team = KH ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * BN;
   const int wm = WIDE ? 0 : (wave >> 1) * (32 * MI), wn = WIDE ? wave * WN : (wave & 1) * WN;
@@ -264,8 +272,8 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // the activation tile goes from global memory straight into LDS (no registers, no LDS
   // store instructions): wave instruction r writes chunks [wave*64 + 256*r, +64) in lane
   // order.  Completion is counted by vmcnt.
-  char* const tiles = reinterpret_cast<char*>(&xs[0][0]);
   constexpr int TILE_BYTES = BM * 128;
+  char* const tiles = reinterpret_cast<char*>(&xs[0][0]) + team * (SLOTS * TILE_BYTES);
   auto load_x = [&](int buf, int k0) {
 #pragma unroll
     for (int r = 0; r < XR; ++r)
@@ -383,8 +391,8 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
   // the other LDS buffer and its registers are refilled two steps ahead, the current tile
   // is multiplied, the freed weight stage is refilled two steps ahead; one barrier.
   // this workgroup's K range (all of K unless split; a multiple of four K steps)
-  const int kb = GROUPED ? 0 : (int)blockIdx.z * p.kc;
-  const int ke = GROUPED ? p.K : min(p.K, kb + p.kc);
+  const int kb = KH ? team * (p.K >> 1) : GROUPED ? 0 : (int)blockIdx.z * p.kc;
+  const int ke = KH ? kb + (p.K >> 1) : GROUPED ? p.K : min(p.K, kb + p.kc);
   if (DEEP) {
     // Four register stages each of weights and of activation chunks, requested four steps
     // ahead; the activations pass through registers into the two LDS tiles one step ahead
@@ -491,12 +499,42 @@ __global__ __launch_bounds__(256, 2) void qmm_kernel(const QmmParams p) {
     return;
   }
 
+  if (KH) {
+    // the second team's sums: through LDS (lane-contiguous floats per accumulator register),
+    // added to the first team's, which goes on alone
+    float* ex = reinterpret_cast<float*>(&xs[0][0]);
+    __syncthreads();  // both teams have finished reading their activation tiles
+    if (team == 1) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            ex[(((wave * MI + i) * 2 + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+    }
+    __syncthreads();
+    if (team == 0) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[i][j][r] += ex[(((wave * MI + i) * 2 + j) * 16 + r) * 64 + lane];
+          asm volatile("" ::: "memory");  // one accumulator's reads at a time: no extra registers
+        }
+    }
+    __syncthreads();  // the sums have been read: the staging below overwrites this memory
+    if (team == 1) return;  // (no workgroup barrier after this point)
+  }
+
   // Epilogue through LDS.  D[i][j] holds column lane%32 (W row n) and rows
   // 8*(r/4) + 4*(lane/32) + r%4 (token m): a wave first writes its (32*MI) x 64 tile as bf16
   // into its own slice of the (now idle) activation buffers - 2-byte LDS stores at constant
   // offsets from one base, so no address lives in registers next to the accumulators -
   // and then copies whole rows out with 16-byte stores (residual added on the way).
-  __syncthreads();  // every wave has finished reading the last activation tile
+  if (!KH) __syncthreads();  // every wave has finished reading the last activation tile
   constexpr int TS = 64 + 8;  // row stride of the staging tile (bf16)
   bf16_t* stage = &xs[0][0] + (size_t)wave * (32 * MI) * TS;
   if (PAIR) {
@@ -753,7 +791,14 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
           p.part, p.residual, p.y, total, (int64_t)part_stride(M, N), p.ksplit, vec_ok);
     }
   } else {
-    if (sb4)
+    // up to one tall tile per CU: eight waves per tile, K in two halves (four-wave workgroups
+    // leave one wave per SIMD there).  4096x4096 under 2046 rows, 256 tiles: 95.0 -> 89.7 us,
+    // 4096x14336: 279 -> 266 us, 6144x4096 under 1022 rows, 192 tiles: 82.0 -> 77.5 us; more
+    // tiles than CUs lose (384: 127 -> 144 us, 512: 155 -> 171 us)
+    const int64_t tall = (int64_t)g4.x * g4.y;
+    if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
+      qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
+    else if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 4, false, false><<<g4, 256, 0, st>>>(p);
