@@ -185,8 +185,8 @@ template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = 
 __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const QmmParams p) {
   static_assert(!WIDE || GROUPED || !PAIR, "the wide pair tile is for the grouped GEMM");
   static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
-  static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !PAIR && !WIDE && !DEEP),
-                "two K halves per workgroup: the plain 256-row tile only");
+  static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !WIDE && !DEEP),
+                "two K halves per workgroup: the 256-row tile of the plain and the pair GEMM");
   constexpr int kThreads = 256;  // of a team
   constexpr int BM = WIDE ? 32 * MI : 64 * MI;
   constexpr int WN = PAIR ? 32 : 64;              // output columns per wave
@@ -1043,7 +1043,10 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
           p.part, p.y, total, 2 * one, one, p.ksplit);
     }
   } else {
-    if (sb4)
+    // (up to one tall tile per CU: eight waves per tile, as in launch_qmm)
+    if (sb4 && (int64_t)g4.x * g4.y <= 256 && p.K % 512 == 0 && p.K >= 1024)
+      qmm_kernel<BITS, 4, false, true, true, false, false, true><<<g4, 512, 0, st>>>(p);
+    else if (sb4)
       qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 4, false, false, true><<<g4, 256, 0, st>>>(p);
