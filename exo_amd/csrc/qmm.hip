@@ -222,6 +222,10 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // weight rows of this lane: column tile j -> row n0 + wn + 32*j + lane%32, half lane/32.
   // Addresses are a workgroup-uniform base plus a 32-bit lane offset (the tile spans at
   // most 128 rows), so the loop carries no 64-bit address arithmetic.
+  // a wave whose rows all lie past the end of the input (the lower half of a last, short row
+  // tile) requests no weights and multiplies nothing: it only helps to load the activation
+  // tiles and keeps the barriers, and leaves the CU's vector and matrix pipes to the others
+  const bool idle = m0 + wm >= m_end;
   const int frow = lane & 31, kq = lane >> 5;
   const uint32_t* wbase = p.w + w_off + (size_t)n0 * wpr;
   const bf16_t* sbase = p.s + s_off + (size_t)n0 * G;
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
 #pragma unroll
     for (int u = 0; u < 4; ++u) {  // (a K range is a multiple of four steps)
       fetch_x(xq[u], kb + u * BK);
-      load_w(wq[u], kb + u * BK);
+      if (!idle) load_w(wq[u], kb + u * BK);
     }
     store_x(0, xq[0]);
     int k0 = kb;
@@ -433,8 +437,10 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
         __syncthreads();
         store_x((u + 1) & 1, xq[(u + 1) & 3]);
         fetch_x(xq[u], k + 4 * BK);
-        multiply(wq[u], u & 1, sbc, u);
-        load_w(wq[u], k + 4 * BK);
+        if (!idle) {
+          multiply(wq[u], u & 1, sbc, u);
+          load_w(wq[u], k + 4 * BK);
+        }
       }
       sbc = sbn;
     }
@@ -442,7 +448,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     for (int u = 0; u < 4; ++u) {  // the last block: everything it needs is under way
       __syncthreads();
       if (u < 3) store_x((u + 1) & 1, xq[(u + 1) & 3]);
-      multiply(wq[u], u & 1, sbc, u);
+      if (!idle) multiply(wq[u], u & 1, sbc, u);
     }
   }
   WStage w0, w1;
@@ -453,7 +459,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   }
   if (!DEEP) {
     load_x(0, kb);
-    load_w(w0, kb);
+    if (!idle) load_w(w0, kb);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tile is in LDS
   __syncthreads();
@@ -469,9 +475,9 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     }
     if (k0 + BK < ke) {
       load_x(buf ^ 1, k0 + BK);
-      load_w(w1, k0 + BK);
+      if (!idle) load_w(w1, k0 + BK);
     }
-    multiply(w0, buf, sb0, ks & 3);
+    if (!idle) multiply(w0, buf, sb0, ks & 3);
     w0 = w1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
