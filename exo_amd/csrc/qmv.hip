@@ -1020,7 +1020,10 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
       }
     }
   }
-  __syncthreads();
+  // xs and sx of a slot belong to its wave alone: its own LDS writes are complete before its
+  // reads, no workgroup barrier
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
 
   uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
   asm volatile("" : "+s"(kmask));
