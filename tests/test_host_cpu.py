@@ -79,6 +79,20 @@ def test_argument_errors_without_gpu():
         native.check(-1, "x")
 
 
+def test_bench_reads_the_committed_counter_summary():
+    """roofline.traffic of the bench line comes from the committed rocprofv3 --pmc summary:
+    the launch names bench.py asks for must be the ones that file lists."""
+    import importlib.util
+    import pathlib
+    root = pathlib.Path(__file__).resolve().parents[1]
+    spec = importlib.util.spec_from_file_location("bench_module", root / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    traffic, src = bench.pmc_traffic("norm_gate_up_swiglu")
+    assert traffic is not None and 0.95 < traffic / 66105344 < 1.10, (traffic, src)
+    assert "commit" in src
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(native, "_lib", None)
     monkeypatch.setattr(native, "LIB_PATH", tmp_path / "nope.so")
