@@ -205,6 +205,8 @@ def _causal_ref(q, k, v, pos, T, heads, Hq, Hkv, D):
     (64, 4, 4094, 0, 4224),      # Qwen3-235B-A22B prompt chunk
     (32, 8, 2048, 1500, 8192),   # a later chunk of a long prompt in the engine's default cache
     (32, 8, 4096, 4096, 8192),   # a full-size chunk ending exactly at the end of the cache
+    (32, 4, 1024, 39936, 40960),   # the last chunk of a prompt that fills Qwen3's 40960 positions
+    (32, 8, 1024, 130048, 131072), # the same at Llama-3.1's 131072 positions
 ])
 def test_prefill_attention_at_config_lengths(device, Hq, Hkv, T, pos, S_max):
     """The matrix-core flash kernel over thousands of keys (many key tiles, the causal edge
@@ -267,6 +269,9 @@ def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed):
     (4, 32, 8, [8191, 2050, 4097, 3], 8192),
     (8, 32, 8, [8192, 8191, 2050, 2049, 4097, 4096, 65, 64], 8192),
     (2, 64, 4, [4224, 4097], 4224),                                   # Qwen3-235B shard heads
+    (2, 32, 4, [40960, 32769], 40960),                                # Qwen3's longest context
+    (1, 32, 8, [131072], 131072),                                     # Llama-3.1's longest context
+    (4, 32, 8, [131072, 65537, 2050, 1], 131072),                     # 2 GiB of keys: byte offsets past 2^31
 ])
 def test_fused_decode_attention_at_config_lengths(device, B, Hq, Hkv, lens, S_max):
     _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0])
