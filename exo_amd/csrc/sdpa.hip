@@ -24,8 +24,11 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kMaxSplits = 16;
-// More splits than 16 were slower for every head layout measured (4 and 8 kv heads): the
-// merge by the last workgroup grows with the split count.
+// More splits than 16 were slower for every head layout measured (4 and 8 kv heads) at a few
+// thousand keys: the merge by the last workgroup grows with the split count.  Contexts the
+// host declares long (exo_attn_decode_hint) take up to kMaxSplitsLong (64 lost to 32 at
+// every length up to 130000 keys).
+constexpr int kMaxSplitsLong = 32;
 constexpr int kBlk = 4;  // keys per lane group per step
 
 struct SdpaParams {
@@ -82,6 +85,43 @@ __device__ __forceinline__ void st_dev(float* p, float v) {
 }
 __device__ __forceinline__ float ld_dev(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The last workgroup's merge of the key splits of one output element: partials
+// [splits][D + 2] (D sums, then the split's maximum and its sum of weights), taken sixteen
+// splits at a time - all loads of a batch are issued before any is used (they miss every
+// cache) - and folded into a running (maximum, sum, weighted sum).
+template <int D>
+__device__ __forceinline__ float merge_splits(const float* src, int splits, int e) {
+  constexpr int MS = 16;
+  float mw = -INFINITY, acc = 0.f, lsum = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += MS) {
+    float pm[MS], pl[MS], po[MS];
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp) {
+      const int spc = min(s0 + sp, splits - 1);
+      pm[sp] = ld_dev(src + (size_t)spc * (D + 2) + D);
+      pl[sp] = ld_dev(src + (size_t)spc * (D + 2) + D + 1);
+      po[sp] = ld_dev(src + (size_t)spc * (D + 2) + e);
+    }
+    float mc = mw;
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp)
+      if (s0 + sp < splits) mc = fmaxf(mc, pm[sp]);
+    if (s0 > 0) {  // earlier batches move to the new maximum
+      const float r = (mw == -INFINITY) ? 0.f : __expf(mw - mc);
+      acc *= r;
+      lsum *= r;
+    }
+#pragma unroll
+    for (int sp = 0; sp < MS; ++sp) {
+      const float sc = (s0 + sp >= splits || pm[sp] == -INFINITY) ? 0.f : __expf(pm[sp] - mc);
+      acc += po[sp] * sc;
+      lsum += pl[sp] * sc;
+    }
+    mw = mc;
+  }
+  return acc / lsum;
 }
 
 // One head slice (8 elements of this lane, the head spread over LPK lanes) taken from a
@@ -379,28 +419,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_kernel(const SdpaParams p) {
     const int g = idx / D, e = idx % D;
     const int h = h0 + g;
     const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
-    // all loads of all splits are issued before any is used (they miss every cache)
-    constexpr int MS = kMaxSplits;
-    float pm[MS], pl[MS], po[MS];
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp) {
-      const int spc = min(sp, p.splits - 1);
-      pm[sp] = ld_dev(src + (size_t)spc * (D + 2) + D);
-      pl[sp] = ld_dev(src + (size_t)spc * (D + 2) + D + 1);
-      po[sp] = ld_dev(src + (size_t)spc * (D + 2) + e);
-    }
-    float mw = -INFINITY;
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp)
-      if (sp < p.splits) mw = fmaxf(mw, pm[sp]);
-    float acc = 0.f, lsum = 0.f;
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp) {
-      const float sc = (sp >= p.splits || pm[sp] == -INFINITY) ? 0.f : __expf(pm[sp] - mw);
-      acc += po[sp] * sc;
-      lsum += pl[sp] * sc;
-    }
-    p.out[qrow + (size_t)h * D + e] = f2bf(acc / lsum);
+    p.out[qrow + (size_t)h * D + e] = f2bf(merge_splits<D>(src, p.splits, e));
   }
 }
 
@@ -698,27 +717,7 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
     const int g = idx / D, e = idx % D;
     const int h = h0 + g;
     const float* src = p.ws + (size_t)(b * p.Hq + h) * p.splits * (D + 2);
-    constexpr int MS = kMaxSplits;
-    float pm[MS], pl[MS], po[MS];
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp) {
-      const int spc = min(sp, p.splits - 1);
-      pm[sp] = ld_dev(src + (size_t)spc * (D + 2) + D);
-      pl[sp] = ld_dev(src + (size_t)spc * (D + 2) + D + 1);
-      po[sp] = ld_dev(src + (size_t)spc * (D + 2) + e);
-    }
-    float mw = -INFINITY;
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp)
-      if (sp < p.splits) mw = fmaxf(mw, pm[sp]);
-    float acc = 0.f, lsum = 0.f;
-#pragma unroll
-    for (int sp = 0; sp < MS; ++sp) {
-      const float scw = (sp >= p.splits || pm[sp] == -INFINITY) ? 0.f : __expf(pm[sp] - mw);
-      acc += po[sp] * scw;
-      lsum += pl[sp] * scw;
-    }
-    p.out[qrow + (size_t)h * D + e] = f2bf(acc / lsum);
+    p.out[qrow + (size_t)h * D + e] = f2bf(merge_splits<D>(src, p.splits, e));
   }
 }
 
@@ -779,15 +778,21 @@ int check(const char* name, int B, int T, int Hq, int Hkv, int D, int S_max) {
   return EXO_OK;
 }
 
-// partials for kMaxSplits splits, then one int counter per (sequence, kv head)
-int64_t ws_partial_floats(int B, int Hq, int D) {
-  return (int64_t)B * Hq * kMaxSplits * (D + 2);
+// Workspace: one int counter per (sequence, query head) first, then the partials of
+// (query heads x splits): kMaxSplits splits for any launch; a long-context launch has up to
+// kMaxSplitsLong splits but at most 256 workgroups of at most 16 heads each.
+constexpr int64_t kLongHeadSplits = 256 * 16;
+int64_t ws_counter_floats(int B, int Hq) { return ((int64_t)B * Hq + 63) / 64 * 64; }
+int64_t ws_head_splits(int B, int Hq) {
+  const int64_t heads = (int64_t)B * Hq;
+  const int64_t lng = heads * kMaxSplitsLong < kLongHeadSplits ? heads * kMaxSplitsLong : kLongHeadSplits;
+  return heads * kMaxSplits > lng ? heads * kMaxSplits : lng;
 }
 
 }  // namespace
 
 extern "C" int64_t exo_sdpa_decode_workspace(int B, int Hq, int D) {
-  return (ws_partial_floats(B, Hq, D) + (int64_t)B * Hq) * (int64_t)sizeof(float);
+  return (ws_counter_floats(B, Hq) + ws_head_splits(B, Hq) * (D + 2)) * (int64_t)sizeof(float);
 }
 
 extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
@@ -798,8 +803,8 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
   if (rc) return rc;
   EXO_REQUIRE(q && k_cache && v_cache && pos && out && workspace,
               "exo_sdpa_decode: null pointer");
-  SdpaParams p{q, k_cache, v_cache, pos, out, workspace,
-               reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
+  SdpaParams p{q, k_cache, v_cache, pos, out, workspace + ws_counter_floats(B, Hq),
+               reinterpret_cast<int*>(workspace), scale, B, 1, Hq,
                Hkv, S_max, pick_splits(B, Hq, Hkv, S_max), nullptr, nullptr, nullptr, nullptr, nullptr,
                0.f};
   rc = (D == 64) ? launch_sdpa<64, 1>(p, (hipStream_t)stream)
@@ -816,8 +821,8 @@ extern "C" int exo_sdpa_decode(const uint16_t* q, const uint16_t* k_cache,
 // host-side handle; its device address is looked up once per device and kept.
 constexpr int kStaticMaxHeads = EXO_SDPA_DECODE_STATIC_MAX_HEADS;  // B * Hq of one call
 constexpr int kStaticMaxD = 128;
-constexpr int64_t kStaticFloats =
-    (int64_t)kStaticMaxHeads * kMaxSplits * (kStaticMaxD + 2) + kStaticMaxHeads;
+constexpr int64_t kStaticFloats =  // the counters, then kMaxSplits partials per head
+    (kStaticMaxHeads + 63) / 64 * 64 + (int64_t)kStaticMaxHeads * kMaxSplits * (kStaticMaxD + 2);
 static __device__ __align__(256) float scratch[kStaticFloats];
 
 constexpr int kMaxDevices = 64;
@@ -867,11 +872,11 @@ extern "C" int exo_sdpa_decode_static(const uint16_t* q, const uint16_t* k_cache
   float* ws = nullptr;
   rc = scratch_address(&ws);
   if (rc) return rc;
-  // The counters of this call's layout sit right behind its partials, where an earlier
-  // call of another shape may have left partial sums: they are cleared by a small kernel
+  // The counters of this call's layout reach as far as its head count, where an earlier
+  // call with fewer heads may have left partial sums: they are cleared by a small kernel
   // (no memset node, so the call can be captured into a graph).
   const int n_cnt = B * Hq;
-  int* cnt = reinterpret_cast<int*>(ws + ws_partial_floats(B, Hq, D));
+  int* cnt = reinterpret_cast<int*>(ws);
   zero_ints_kernel<<<dim3(exo_ceil_div(n_cnt, 256)), 256, 0, (hipStream_t)stream>>>(cnt, n_cnt);
   return exo_sdpa_decode(q, k_cache, v_cache, pos, out, ws, scale, B, Hq, Hkv, D, S_max, stream);
 }
@@ -897,17 +902,36 @@ extern "C" int exo_rope_table(const float* inv_freq, float* table, int S_max, in
   return EXO_OK;
 }
 
-extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
-                               const int32_t* pos, const float* inv_freq, const float* rope_table,
-                               const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
-                               uint16_t* out, float* workspace, float scale, int B, int Hq,
-                               int Hkv, int D, int S_max, exo_stream_t stream) {
+// Contexts the host declares long (keys_hint) take the matrix-core kernel whatever the head
+// count.  One sequence of 32 query heads, us per launch, scalar kernel with 8 splits | the
+// matrix-core kernel with 16 | 32 | 64 splits per kv head:
+//   8 kv heads:   2050 keys 9.3 | 10.6;  8000 keys 17.0 | 15.5 | 17.0 | 23.9;  16000 keys
+//                 . | 24.1 | 22.3 | 28.4;  32000 keys 51.1 | 37.3 | 35.8 | 37.6;  130000 keys
+//                 178 | 110 | 107 | 111
+//   4 kv heads:   2050 keys 9.3 | 12.6;  8000 keys 15.4 | 16.2 | 18.7 | 27.5;  32000 keys
+//                 49.2 | 37.0 | 31.1 | 34.7;  130000 keys 172 | 104 | 69 | 72
+//   64 query / 4 kv heads: 8000 keys 24.2 | 21.9 | 28.0 | 44.5;  32000 keys 88.6 | 44.5 |
+//                 41.5 | 51.8;  130000 keys 328 | 115 | 81 | 88
+// (a wave has one tile of 32 keys, 16 KB of K and V, in flight: over tens of thousands of keys
+// more workgroups keep the memory busier, until the last workgroup's merge of the splits
+// costs more than that returns).  Hence: from kAttnLongKeys keys the matrix-core kernel with
+// up to 16 splits, from kAttnVeryLongKeys with up to 32.
+constexpr int kAttnLongKeys = EXO_ATTN_LONG_KEYS;
+constexpr int kAttnVeryLongKeys = EXO_ATTN_VERY_LONG_KEYS;
+
+extern "C" int exo_attn_decode_hint(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
+                                    const int32_t* pos, const float* inv_freq,
+                                    const float* rope_table, const uint16_t* q_norm_w,
+                                    const uint16_t* k_norm_w, float eps, uint16_t* out,
+                                    float* workspace, float scale, int B, int Hq, int Hkv, int D,
+                                    int S_max, int keys_hint, exo_stream_t stream) {
   int rc = check("exo_attn_decode", B, 1, Hq, Hkv, D, S_max);
   if (rc) return rc;
   EXO_REQUIRE(qkv && k_cache && v_cache && pos && inv_freq && out && workspace,
               "exo_attn_decode: null pointer");
-  SdpaParams p{nullptr, k_cache, v_cache, pos, out, workspace,
-               reinterpret_cast<int*>(workspace + ws_partial_floats(B, Hq, D)), scale, B, 1, Hq,
+  EXO_REQUIRE(keys_hint >= 0, "exo_attn_decode: keys_hint=%d is negative", keys_hint);
+  SdpaParams p{nullptr, k_cache, v_cache, pos, out, workspace + ws_counter_floats(B, Hq),
+               reinterpret_cast<int*>(workspace), scale, B, 1, Hq,
                Hkv, S_max, pick_splits(B, Hq, Hkv, S_max), qkv, inv_freq,
                reinterpret_cast<const float2*>(rope_table), q_norm_w, k_norm_w, eps};
   // 128 or more query heads per step (4+ sequences of 32 heads): the scalar kernel is bound
@@ -919,9 +943,12 @@ extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t*
   // the matrix-core kernel's workgroups; 32 / 4 heads: 4 sequences level, 8 sequences
   // 22.7 -> 18.4 us; 64 / 4 heads: 4 sequences 21.1 -> 19.2, 8 sequences 34.2 -> 23.5 us)
   const int G = Hq / Hkv;
-  if (D == 128 && (G == 4 || G == 8 || G == 16) && B * Hq >= 128 && B * Hkv >= 16) {
+  const bool long_ctx = keys_hint >= kAttnLongKeys && S_max >= kAttnLongKeys;
+  if (D == 128 && (G == 4 || G == 8 || G == 16) &&
+      ((B * Hq >= 128 && B * Hkv >= 16) || long_ctx)) {
+    const int max_sp = keys_hint >= kAttnVeryLongKeys && S_max >= kAttnVeryLongKeys ? kMaxSplitsLong : kMaxSplits;
     int sp = 256 / (B * Hkv);
-    sp = sp > kMaxSplits ? kMaxSplits : (sp < 1 ? 1 : sp);
+    sp = sp > max_sp ? max_sp : (sp < 1 ? 1 : sp);
     if (sp > S_max / 128) sp = S_max / 128 > 0 ? S_max / 128 : 1;
     p.splits = sp;
     p.hgroups = 1;
@@ -940,6 +967,15 @@ extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t*
   if (rc) return rc;
   EXO_CHECK_LAUNCH("exo_attn_decode");
   return EXO_OK;
+}
+
+extern "C" int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
+                               const int32_t* pos, const float* inv_freq, const float* rope_table,
+                               const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
+                               uint16_t* out, float* workspace, float scale, int B, int Hq,
+                               int Hkv, int D, int S_max, exo_stream_t stream) {
+  return exo_attn_decode_hint(qkv, k_cache, v_cache, pos, inv_freq, rope_table, q_norm_w, k_norm_w,
+                              eps, out, workspace, scale, B, Hq, Hkv, D, S_max, 0, stream);
 }
 
 extern "C" int exo_sdpa_prefill(const uint16_t* q, const uint16_t* k_cache,

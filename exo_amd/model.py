@@ -246,6 +246,15 @@ class ShardModel:
         ops.gather_qmv_combine(bf.act, L.down, idx, sc, residual=bf.h, out=bf.h,
                                scratch=bf.expert_out, check_indices=False)
 
+    @staticmethod
+    def _keys_hint(cache: ShardKVCache, rsl: slice) -> int:
+        """The context regime of a decode step from the host's count of the longest sequence
+        (0 or the threshold reached): the attention launch is laid out per regime, and a
+        captured step stays valid inside one."""
+        n = max(cache.offsets[rsl]) + 1
+        return (ops.ATTN_VERY_LONG_KEYS if n >= ops.ATTN_VERY_LONG_KEYS else
+                ops.ATTN_LONG_KEYS if n >= ops.ATTN_LONG_KEYS else 0)
+
     def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
              rows: slice | None = None):
         """Launch the shard forward for B sequences x T tokens on the current stream.
@@ -256,6 +265,7 @@ class ShardModel:
         Hq, Hkv, D = c.num_attention_heads, c.num_key_value_heads, c.head_dim
         rsl = rows if rows is not None else slice(0, B)
         pos = cache.pos[rsl]
+        keys_hint = self._keys_hint(cache, rsl)
         if self.is_first:
             ops.embed(bf.tokens, self.embed_tokens, out=bf.h)
         gemv = R <= self.gemv_rows                                       # qkv, o, lm_head
@@ -271,7 +281,7 @@ class ShardModel:
             if T == 1:  # rope + append + attention in one launch
                 ops.attn_decode(bf.qkv, kc, vc, pos, self.inv_freq, bf.attn, bf.sdpa_ws, self.scale,
                                 B, Hq, Hkv, D, L.q_norm, L.k_norm, c.rms_norm_eps,
-                                rope_tab=self._rope_table(cache.max_seq))
+                                rope_tab=self._rope_table(cache.max_seq), keys_hint=keys_hint)
             else:
                 ops.rope_kv_append(bf.qkv, bf.q, kc, vc, pos, self.inv_freq, B, T, Hq, Hkv, D,
                                    L.q_norm, L.k_norm, c.rms_norm_eps,
@@ -363,7 +373,7 @@ class ShardModel:
         if not use_graph:
             body()
         else:
-            key = (B, feedback, sampler is not None, mode, row0)
+            key = (B, feedback, sampler is not None, mode, row0, self._keys_hint(cache, rsl))
             hit = self._graphs.get(key)
             if hit is None or hit[1] is not cache or hit[2] is not sampler:
                 # warm up outside capture (lazy module loads, attribute settings), then

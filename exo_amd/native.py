@@ -53,6 +53,7 @@ SIGNATURES: dict[str, tuple] = {
     "exo_sdpa_decode": (_i, [_vp] * 6 + [_f] + [_i] * 5 + [_vp]),
     "exo_sdpa_decode_static": (_i, [_vp] * 5 + [_f] + [_i] * 5 + [_vp]),
     "exo_attn_decode": (_i, [_vp] * 8 + [_f, _vp, _vp, _f] + [_i] * 5 + [_vp]),
+    "exo_attn_decode_hint": (_i, [_vp] * 8 + [_f, _vp, _vp, _f] + [_i] * 6 + [_vp]),
     "exo_rope_table": (_i, [_vp, _vp, _i, _i, _vp]),
     "exo_sdpa_prefill": (_i, [_vp] * 5 + [_f] + [_i] * 6 + [_vp]),
     "exo_kv_export_nhd": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -563,18 +563,25 @@ def rope_table(inv_freq: torch.Tensor, S_max: int, D: int) -> torch.Tensor:
     return tab
 
 
+ATTN_LONG_KEYS = 6144        # EXO_ATTN_LONG_KEYS of the C header
+ATTN_VERY_LONG_KEYS = 12288  # EXO_ATTN_VERY_LONG_KEYS
+
+
 def attn_decode(qkv, k_cache, v_cache, pos, inv_freq, out, workspace, scale, B, Hq, Hkv, D,
-                q_norm_w=None, k_norm_w=None, eps: float = 0.0, rope_tab=None):
-    """rope (+ head norm) + cache append + attention for one new token per sequence."""
+                q_norm_w=None, k_norm_w=None, eps: float = 0.0, rope_tab=None, keys_hint: int = 0):
+    """rope (+ head norm) + cache append + attention for one new token per sequence.
+    ``keys_hint``: keys the longest sequence holds as far as the host knows (0: unknown); from
+    ATTN_LONG_KEYS and again from ATTN_VERY_LONG_KEYS on the launch is laid out for longer
+    contexts."""
     lib = native.load()
     if rope_tab is not None and rope_tab.shape[0] < k_cache.shape[2]:
         raise ValueError("rope table shorter than the cache")
     check(
-        lib.exo_attn_decode(
+        lib.exo_attn_decode_hint(
             _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), _ptr(rope_tab),
             _ptr(q_norm_w),
             _ptr(k_norm_w), eps, _ptr(out), _ptr(workspace), scale, B, Hq, Hkv, D,
-            k_cache.shape[2], _stream(),
+            k_cache.shape[2], int(keys_hint), _stream(),
         ),
         "attn_decode",
     )

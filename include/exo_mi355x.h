@@ -247,7 +247,7 @@ int exo_rope_kv_append_tab(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_cac
 /* K7 decode: scaled_dot_product_attention for one new token per sequence over the
  * cache, grouped-query: q bf16 [B, Hq*D]; lens int32 [B] = pos[b]+1 valid keys;
  * out bf16 [B, Hq*D].  `workspace`: exo_sdpa_decode_workspace(B,Hq,D) bytes, zeroed ONCE
- * by the caller before its first use (it ends with arrival counters that every launch
+ * by the caller before its first use (it starts with arrival counters that every launch
  * leaves at zero); launches that share a workspace must not overlap.
  * (.typings/mlx_lm/models/base.pyi:39-47) */
 int64_t exo_sdpa_decode_workspace(int B, int Hq, int D);
@@ -282,6 +282,22 @@ int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
                     const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps, uint16_t* out,
                     float* workspace, float scale, int B, int Hq, int Hkv, int D, int S_max,
                     exo_stream_t stream);
+
+/* exo_attn_decode with the host's knowledge of the context: keys_hint = the number of keys
+ * the longest sequence of this step holds, as far as the host knows (0: unknown, which is
+ * exo_attn_decode).  From EXO_ATTN_LONG_KEYS keys on (in a cache at least that long) the
+ * launch is laid out for long contexts: the matrix-core kernel whatever the head count; from
+ * EXO_ATTN_VERY_LONG_KEYS on with the keys of a kv head over up to 32 workgroups instead of
+ * 16.  The hint only selects the layout - any value gives a correct result for any pos[] -
+ * so a captured launch stays valid while the context grows; the layouts round differently
+ * (within the tolerance of the attention tests). */
+#define EXO_ATTN_LONG_KEYS 6144
+#define EXO_ATTN_VERY_LONG_KEYS 12288
+int exo_attn_decode_hint(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
+                         const int32_t* pos, const float* inv_freq, const float* rope_table,
+                         const uint16_t* q_norm_w, const uint16_t* k_norm_w, float eps,
+                         uint16_t* out, float* workspace, float scale, int B, int Hq, int Hkv,
+                         int D, int S_max, int keys_hint, exo_stream_t stream);
 
 /* (cos, sin) of position*inv_freq[i] for every position < S_max: float [S_max, D/2, 2],
  * the same sincosf values the RoPE kernels compute inline.  Passing it to

@@ -227,7 +227,7 @@ def test_prefill_attention_at_config_lengths(device, Hq, Hkv, T, pos, S_max):
     assert_close(n_f32(got), n_f32(ref), what=f"prefill sdpa T={T} pos={pos} {Hq}/{Hkv}")
 
 
-def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed):
+def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed, keys_hint=0):
     """exo_attn_decode (rope + append + attention) for B sequences at the given lengths,
     against: rope by the oracle, float32 library attention over the cache."""
     from oracle import ops as O
@@ -245,7 +245,8 @@ def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed):
     ws = ops.sdpa_decode_workspace(B, Hq, D, device)
     tab = ops.rope_table(inv_t, S_max, D)
     for _ in range(2):  # twice: the arrival counters must be back at zero
-        ops.attn_decode(qkv, kc, vc, pos, inv_t, out, ws, D ** -0.5, B, Hq, Hkv, D, rope_tab=tab)
+        ops.attn_decode(qkv, kc, vc, pos, inv_t, out, ws, D ** -0.5, B, Hq, Hkv, D, rope_tab=tab,
+                        keys_hint=keys_hint)
     x = n_f32(qkv).reshape(B, 1, Hq + 2 * Hkv, D)
     for b in range(B):
         p = lens[b] - 1
@@ -275,6 +276,47 @@ def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed):
 ])
 def test_fused_decode_attention_at_config_lengths(device, B, Hq, Hkv, lens, S_max):
     _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0])
+
+
+@pytest.mark.parametrize("hint", [ops.ATTN_LONG_KEYS, ops.ATTN_VERY_LONG_KEYS])
+@pytest.mark.parametrize("B,Hq,Hkv,lens,S_max", [
+    (1, 32, 8, [6144], 8192),                          # the first step of the long layout
+    (1, 32, 8, [1], 16384),                            # a hint may be wrong: one key
+    (2, 32, 4, [12288, 130], 16384),                   # splits of 128 keys, most empty for row 1
+    (1, 64, 4, [16383], 16384),                        # 16 query heads per kv head
+    (2, 32, 4, [40960, 32769], 40960),
+    (1, 32, 8, [131072], 131072),
+    (4, 32, 8, [131072, 65537, 2050, 1], 131072),      # the layout the head count takes anyway
+    (1, 16, 8, [9000], 16384),                         # 2 heads per kv head: stays on the scalar kernel
+])
+def test_fused_decode_attention_long_context_layout(device, B, Hq, Hkv, lens, S_max, hint):
+    """exo_attn_decode_hint with the hint at the two long-context thresholds: the matrix-core
+    kernel for any head count, up to 16 or 32 key splits merged by the last workgroup; run
+    twice on one workspace (the arrival counters return to zero)."""
+    _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0] + 7, keys_hint=hint)
+
+
+def test_attention_layouts_share_a_workspace(device):
+    """One workspace, zeroed once, taken in turn by the three layouts (their counters sit at
+    the same place, the partials of one never reach the counters)."""
+    from oracle import ops as O
+    B, Hq, Hkv, D, S_max, n = 1, 32, 8, 128, 16384, 13000
+    g = torch.Generator(device=device).manual_seed(11)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, device=device, generator=g).bfloat16()
+    kc = torch.randn(B, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    vc = torch.randn(B, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    pos = torch.tensor([n - 1], dtype=torch.int32, device=device)
+    inv_t = torch.from_numpy(O.rope_inv_freq(D, 1e6, None)).to(device)
+    ws = ops.sdpa_decode_workspace(B, Hq, D, device)
+    outs = []
+    hints = (0, ops.ATTN_LONG_KEYS, ops.ATTN_VERY_LONG_KEYS)
+    for hint in hints + hints:
+        out = torch.empty(B, Hq * D, dtype=torch.bfloat16, device=device)
+        ops.attn_decode(qkv, kc, vc, pos, inv_t, out, ws, D ** -0.5, B, Hq, Hkv, D, keys_hint=hint)
+        outs.append(out)
+    assert all(torch.equal(outs[i], outs[i + 3]) for i in range(3))
+    assert_close(n_f32(outs[1]), n_f32(outs[0]), what="long against short layout")
+    assert_close(n_f32(outs[2]), n_f32(outs[0]), what="very long against short layout")
 
 
 # ------------------------------------------------------------------ batched decode blocks

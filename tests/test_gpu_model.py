@@ -240,6 +240,35 @@ def test_decode_step_first_replay_matches_call(ckpt, device):
     assert got_toks == want_toks
 
 
+def test_decode_step_recaptures_when_the_context_regime_changes(ckpt, device):
+    """The attention launch of a decode step is laid out per context regime (the host's count
+    of the longest sequence against ATTN_LONG_KEYS): graph replays across the threshold give
+    the tokens of eager steps, and the step is captured once per regime."""
+    from exo_amd import ops
+    cfg, gm = ckpt["cfg"], ckpt["model"]
+    start = ops.ATTN_LONG_KEYS - 4
+    ce, cg = gm.make_cache(1, ops.ATTN_LONG_KEYS + 64), gm.make_cache(1, ops.ATTN_LONG_KEYS + 64)
+    g = torch.Generator(device=device).manual_seed(5)
+    for li in range(len(ce.k)):
+        for t in (ce.k[li], ce.v[li]):
+            t[:, :, :start] = (0.5 * torch.randn(t[:, :, :start].shape, device=device, generator=g)).bfloat16()
+        cg.k[li].copy_(ce.k[li])
+        cg.v[li].copy_(ce.v[li])
+    for c in (ce, cg):
+        c.offsets[0] = start
+        c.sync_pos()
+    bufs = gm._buffers(1, 1)
+    first = int(rng(21).integers(0, cfg.vocab_size))
+    bufs.tokens[0] = first
+    want = [int(gm.decode_step(ce, 1, use_graph=False, feedback=True).next_token[0]) for _ in range(8)]
+    bufs.tokens[0] = first
+    got = [int(gm.decode_step(cg, 1, feedback=True).next_token[0]) for _ in range(8)]
+    assert got == want
+    assert cg.offsets[0] == start + 8 and cg.pos.tolist() == [start + 8]
+    for hint in (0, ops.ATTN_LONG_KEYS):  # one capture per regime, both on this cache
+        assert gm._graphs[(1, True, False, 0, 0, hint)][1] is cg
+
+
 def test_batch_generator_b2_equals_b1(ckpt, device):
     """Port of the reference's B=2 vs B=1 criterion
     (src/exo/worker/engines/mlx/tests/test_batch_generate.py:164-268): same greedy

@@ -56,9 +56,17 @@ def test_argument_errors_without_gpu():
     # the no-allocation decode attention rejects sizes beyond its static scratch
     assert lib.exo_sdpa_decode_static(None, None, None, None, None, 1.0, 9, 32, 8, 128, 64, None) == -1
     assert b"exceed the static scratch" in lib.exo_last_error()
-    assert lib.exo_sdpa_decode_workspace(2, 32, 128) == (2 * 32 * 16 * 130 + 2 * 32) * 4
-    # the expert launch that routes by itself: the limits of exo_router_topk
+    # decode attention workspace: a counter per query head (whole 256-byte lines), then the
+    # partials of 16 key splits per head, or of the long-context layout's up to 32 splits on
+    # at most 256 workgroups where that is more
+    assert lib.exo_sdpa_decode_workspace(2, 32, 128) == (64 + 64 * 32 * 130) * 4
+    assert lib.exo_sdpa_decode_workspace(8, 32, 128) == (256 + 256 * 16 * 130) * 4
+    assert lib.exo_sdpa_decode_workspace(64, 32, 128) == (2048 + 2048 * 16 * 130) * 4
     one = C.c_void_p(1)  # any non-null pointer: rejected before it is ever used
+    assert lib.exo_attn_decode_hint(one, one, one, one, one, None, None, None, 0.0, one, one, 1.0, 1, 32, 8,
+                                    128, 8192, -5, None) == -1
+    assert b"keys_hint" in lib.exo_last_error()
+    # the expert launch that routes by itself: the limits of exo_router_topk
     rc = lib.exo_norm_route_gather_qmv_swiglu(one, None, 0.0, one, 1, one, one, one, one, one, one, one, one,
                                               one, 1, 8, 300, 64, 2048, 4, 64, None)
     assert rc == -1 and b"E<=256" in lib.exo_last_error()
