@@ -906,7 +906,7 @@ extern "C" int exo_rope_table(const float* inv_freq, float* table, int S_max, in
 // count.  One sequence of 32 query heads, us per launch, scalar kernel with 8 splits | the
 // matrix-core kernel with 16 | 32 | 64 splits per kv head:
 //   8 kv heads:   2050 keys 9.3 | 10.6;  8000 keys 17.0 | 15.5 | 17.0 | 23.9;  16000 keys
-//                 . | 24.1 | 22.3 | 28.4;  32000 keys 51.1 | 37.3 | 35.8 | 37.6;  130000 keys
+//                 - | 24.1 | 22.3 | 28.4;  32000 keys 51.1 | 37.3 | 35.8 | 37.6;  130000 keys
 //                 178 | 110 | 107 | 111
 //   4 kv heads:   2050 keys 9.3 | 12.6;  8000 keys 15.4 | 16.2 | 18.7 | 27.5;  32000 keys
 //                 49.2 | 37.0 | 31.1 | 34.7;  130000 keys 172 | 104 | 69 | 72

@@ -87,17 +87,25 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
     for (int s = 0; s < STEPS; ++s) qreg[s] = *reinterpret_cast<const uint4*>(qp + s * 16);
   }
 
-  const bf16_t* kbase = p.k + ((size_t)b * p.Hkv + kvh) * (size_t)p.S_max * D;
-  const bf16_t* vbase = p.v + ((size_t)b * p.Hkv + kvh) * (size_t)p.S_max * D;
+  // K/V tiles come through buffer loads: one descriptor per (sequence, kv head) that ends
+  // with the cache (rows past it read as zero; they are masked), a lane offset that never
+  // changes and the tile as the scalar offset - no 64-bit address per load in registers.
+  // A K tile is one contiguous block (16 bytes per thread and load); a V load takes key
+  // tid % 64, chunk tid / 64 + 4 i, so that a thread's stores into V^T are 8 rows of one key.
+  const size_t head_off = ((size_t)b * p.Hkv + kvh) * (size_t)p.S_max * D;
+  const uint32_t head_bytes = (uint32_t)p.S_max * D * 2;
+  const __amdgpu_buffer_rsrc_t rk =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.k + head_off), 0, head_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rv =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.v + head_off), 0, head_bytes, 0x00020000);
+  const uint32_t koff = tid * 16, voff = (tid & (kBN - 1)) * (D * 2) + (tid / kBN) * 16;
   uint4 kreg[LOADS], vreg[LOADS];
   auto load_tile = [&](int kt) {
+    const uint32_t tile = (uint32_t)kt * (kBN * D * 2);
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-      const int vi = tid + i * 256;
-      const int key = min(kt * kBN + vi / VEC, p.S_max - 1);  // rows past the cache end: masked
-      kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)key * D + (vi % VEC) * 8);
-      const int key_v = min(kt * kBN + (vi & (kBN - 1)), p.S_max - 1);
-      vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)key_v * D + (vi / kBN) * 8);
+      kreg[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rk, koff, tile + i * 4096, 0));
+      vreg[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rv, voff + i * 64, tile, 0));
     }
   };
   auto store_tile = [&](int buf) {
@@ -131,6 +139,11 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
 
   load_tile(0);
   store_tile(0);
+  // Every load so far (the Q operand among them) has landed before the loop is entered: left
+  // to itself the compiler requests Q last and then waits, in EVERY iteration, for as many
+  // loads as were issued after each Q register - which in the loop are the tile loads just
+  // requested, so the prefetch would be waited for on the spot.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   if (n_tiles > 1) load_tile(1);
   for (int kt = 0; kt < n_tiles; ++kt) {
     // tile kt is complete in its buffer, and every wave is done reading the other buffer
