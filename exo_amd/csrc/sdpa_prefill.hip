@@ -17,6 +17,13 @@
 // (4, 8, 16 query heads per kv head) they share every K/V tile they stage.  Key tiles of
 // 64 in two LDS buffers: while a tile is computed, the next one goes from registers into the
 // other buffer and the one after that is on its way from memory; one barrier per tile.
+//
+// SPLIT (launches of at most one workgroup per CU, i.e. prompts of about a thousand tokens):
+// eight waves, two teams of four that take the first and the second half of the
+// workgroup's key tiles for the same four units, each with tile buffers of its own; at the end
+// the second team's (O^T, max, sum) pass through LDS and are merged into the first's.  The
+// causal triangle gives a launch of one round workgroups of 1 to N tiles; without the split
+// the heavy ones run on alone, one wave per SIMD, for most of the launch.
 #include "../../include/exo_mi355x.h"
 #include "common.h"
 #include "sdpa_internal.h"
@@ -42,8 +49,8 @@ constexpr int fa_lds_bytes() {
   return 2 * (kBN * (D + kPadK) + D * (kBN + kPadK)) * 2;
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
+template <int D, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 512 : 256, SPLIT ? 1 : 2) void fa_prefill_kernel(const FaParams p) {
   constexpr int STEPS = D / 16;  // MFMA steps over d for S^T
   constexpr int DT = D / 32;     // 32-row tiles of O^T
   constexpr int KS = D + kPadK;  // LDS row stride of K (bf16)
@@ -51,10 +58,12 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   constexpr int VEC = D / 8;     // 16-byte vectors per K/V row
   constexpr int LOADS = kBN * VEC / 256;
   constexpr int BUF = kBN * KS + D * VS;  // bf16 elements of one (K, V^T) tile pair
-  extern __shared__ __attribute__((aligned(16))) bf16_t fa_lds[];  // [2][BUF]
+  extern __shared__ __attribute__((aligned(16))) bf16_t fa_lds[];  // [2][BUF] per team
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x & 255, lane = tid & 63;  // within the team
+  const int team = SPLIT ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  bf16_t* const lds = fa_lds + team * (2 * BUF);
   const int n = lane & 31, kq = lane >> 5;
   const int kvh = blockIdx.y, b = blockIdx.z;
   // Heavy (late) token tiles first - but a launch of up to two workgroups per CU is one round
@@ -64,7 +73,7 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   // 129 -> 109 us; with 2048 launches the same order lost 10 %).
   const int row = (int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z;
   const int rows_per_run = max(1, 256 / (int)gridDim.x);
-  const bool one_round = gridDim.x * gridDim.y * gridDim.z <= 512;  // (longer launches balance
+  const bool one_round = !SPLIT && gridDim.x * gridDim.y * gridDim.z <= 512;  // (longer launches balance
   const bool light_first = one_round && ((row / rows_per_run) & 1);  //  themselves, heavy first)
   const int u0 = (light_first ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x) * 4;
   const int u = u0 + wave;
@@ -77,7 +86,12 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   const int last_w = pos + min(tt * kBM + kBM - 1, p.T - 1);  // last key any row of the wave sees
   const int tt_max = min(u0 + 3, p.units - 1) / p.G;
   const int last_wg = min(pos + min(tt_max * kBM + kBM - 1, p.T - 1), p.S_max - 1);
-  const int n_tiles = last_wg / kBN + 1;
+  const int n_all = last_wg / kBN + 1;  // key tiles of the workgroup
+  // SPLIT: team 0 takes tiles [0, n_all / 2), team 1 the rest - at least as many, and the
+  // ones with the causal edge; the workgroup's barriers are counted by team 1's tiles
+  const int t_first = (SPLIT && team) ? n_all / 2 : 0;
+  const int n_tiles = !SPLIT ? n_all : team ? n_all - n_all / 2 : n_all / 2;
+  const int n_iter = SPLIT ? n_all - n_all / 2 : n_all;
 
   // Q^T operand: lane (query n, half kq) holds d = step*16 + kq*8 .. +8 for every step
   uint4 qreg[STEPS];
@@ -101,7 +115,7 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
   const uint32_t koff = tid * 16, voff = (tid & (kBN - 1)) * (D * 2) + (tid / kBN) * 16;
   uint4 kreg[LOADS], vreg[LOADS];
   auto load_tile = [&](int kt) {
-    const uint32_t tile = (uint32_t)kt * (kBN * D * 2);
+    const uint32_t tile = (uint32_t)(t_first + kt) * (kBN * D * 2);
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       kreg[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rk, koff, tile + i * 4096, 0));
@@ -109,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
     }
   };
   auto store_tile = [&](int buf) {
-    bf16_t* kl = fa_lds + buf * BUF;
+    bf16_t* kl = lds + buf * BUF;
     bf16_t* vl = kl + kBN * KS;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
@@ -137,24 +151,27 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
     for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  load_tile(0);
-  store_tile(0);
+  if (!SPLIT || n_tiles > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
   // Every load so far (the Q operand among them) has landed before the loop is entered: left
   // to itself the compiler requests Q last and then waits, in EVERY iteration, for as many
   // loads as were issued after each Q register - which in the loop are the tile loads just
   // requested, so the prefetch would be waited for on the spot.
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   if (n_tiles > 1) load_tile(1);
-  for (int kt = 0; kt < n_tiles; ++kt) {
+  for (int kt = 0; kt < n_iter; ++kt) {
     // tile kt is complete in its buffer, and every wave is done reading the other buffer
     __syncthreads();
+    if (SPLIT && kt >= n_tiles) continue;  // (team 0 when the tile count is odd)
     if (kt + 1 < n_tiles) {
       store_tile((kt + 1) & 1);
       if (kt + 2 < n_tiles) load_tile(kt + 2);
     }
-    const int key0 = kt * kBN;
+    const int key0 = (t_first + kt) * kBN;
     if (key0 > last_w) continue;  // wave-uniform: nothing visible to this wave's rows
-    const bf16_t* k_lds = fa_lds + (kt & 1) * BUF;
+    const bf16_t* k_lds = lds + (kt & 1) * BUF;
     const bf16_t* v_lds = k_lds + kBN * KS;
 
     // ---- S^T = K Q^T for the two 32-key sub-tiles
@@ -231,6 +248,32 @@ __global__ __launch_bounds__(256, 2) void fa_prefill_kernel(const FaParams p) {
     }
   }
 
+  if (SPLIT) {
+    // the second team's sums: through LDS (lane-contiguous floats per register), merged into
+    // the first team's, which goes on alone
+    float* ex = reinterpret_cast<float*>(fa_lds) + wave * ((DT * 16 + 2) * 64);
+    __syncthreads();  // both teams have finished with their tile buffers
+    if (team == 1) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) ex[(dt * 16 + e) * 64 + lane] = o[dt][e];
+      ex[(DT * 16) * 64 + lane] = m_run;
+      ex[(DT * 16 + 1) * 64 + lane] = l_run;
+    }
+    __syncthreads();
+    if (team == 1) return;  // (no workgroup barrier after this point)
+    const float m1 = ex[(DT * 16) * 64 + lane], l1 = ex[(DT * 16 + 1) * 64 + lane];
+    const float m = fmaxf(m_run, m1);  // finite: key 0 is visible to one of the teams
+    const float a0 = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m);
+    const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+    l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][e] = o[dt][e] * a0 + ex[(dt * 16 + e) * 64 + lane] * a1;
+  }
+
   // ---- out[token][hq*D + d] = O^T[d][token] / l
   if (!active || tt * kBM + n >= p.T) return;
   const float inv = 1.f / l_run;
@@ -265,20 +308,37 @@ int exo_sdpa_prefill_mfma(const bf16_t* q, const bf16_t* k_cache, const bf16_t* 
   p.G = Hq / Hkv;
   p.units = ((T + kBM - 1) / kBM) * p.G;
   const dim3 grid((p.units + 3) / 4, Hkv, B);
-  static bool attr_done = false;  // 70 KiB of LDS for D = 128: above the default limit
-  if (!attr_done) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_prefill_kernel<128>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             fa_lds_bytes<128>());
+  // the split variant where its eight-wave workgroups are one round of one per CU (their two
+  // teams' tile buffers leave room for one) and the heaviest has enough tiles to share out:
+  // 1022 tokens of 32 / 4 heads (256 workgroups) 34.9 -> 30.3 us; with 512 workgroups it is
+  // two rounds and loses to two four-wave workgroups per CU (2046 tokens, 32 / 8: 75 -> 106 us)
+  const bool split = (int64_t)grid.x * grid.y * grid.z <= 256 && T >= 256;
+  // more than 64 KiB of LDS per workgroup: raised once per kernel instance
+  auto raise = [](const void* fn, int bytes, bool* done) {
+    if (*done || bytes <= 64 * 1024) return EXO_OK;
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) {
       exo_set_error("exo_sdpa_prefill: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
       return EXO_ERR_HIP;
     }
-    attr_done = true;
+    *done = true;
+    return EXO_OK;
+  };
+  static bool done[4] = {false, false, false, false};
+  const int lds = (D == 64 ? fa_lds_bytes<64>() : fa_lds_bytes<128>()) * (split ? 2 : 1);
+  int rc;
+  if (D == 64 && !split) {
+    if ((rc = raise(reinterpret_cast<const void*>(fa_prefill_kernel<64, false>), lds, &done[0]))) return rc;
+    fa_prefill_kernel<64, false><<<grid, 256, lds, stream>>>(p);
+  } else if (D == 64) {
+    if ((rc = raise(reinterpret_cast<const void*>(fa_prefill_kernel<64, true>), lds, &done[1]))) return rc;
+    fa_prefill_kernel<64, true><<<grid, 512, lds, stream>>>(p);
+  } else if (!split) {
+    if ((rc = raise(reinterpret_cast<const void*>(fa_prefill_kernel<128, false>), lds, &done[2]))) return rc;
+    fa_prefill_kernel<128, false><<<grid, 256, lds, stream>>>(p);
+  } else {
+    if ((rc = raise(reinterpret_cast<const void*>(fa_prefill_kernel<128, true>), lds, &done[3]))) return rc;
+    fa_prefill_kernel<128, true><<<grid, 512, lds, stream>>>(p);
   }
-  if (D == 64)
-    fa_prefill_kernel<64><<<grid, 256, fa_lds_bytes<64>(), stream>>>(p);
-  else
-    fa_prefill_kernel<128><<<grid, 256, fa_lds_bytes<128>(), stream>>>(p);
   return EXO_OK;
 }

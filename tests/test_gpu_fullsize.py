@@ -227,6 +227,30 @@ def test_prefill_attention_at_config_lengths(device, Hq, Hkv, T, pos, S_max):
     assert_close(n_f32(got), n_f32(ref), what=f"prefill sdpa T={T} pos={pos} {Hq}/{Hkv}")
 
 
+@pytest.mark.parametrize("D,Hq,Hkv,T,pos,S_max", [
+    (128, 32, 4, 1000, 37, 1280),   # ragged chunk behind cached tokens, odd tile count per workgroup
+    (128, 16, 8, 300, 0, 512),      # 2 heads per kv head: a workgroup's waves are different token tiles
+    (128, 4, 4, 257, 5, 384),       # 1 head per kv head, the shortest chunk that takes this layout
+    (64, 8, 2, 260, 0, 320),        # head_dim 64
+    (128, 64, 4, 512, 1536, 2048),  # 16 heads per kv head, a later chunk
+])
+def test_prefill_attention_two_team_layout(device, D, Hq, Hkv, T, pos, S_max):
+    """Launches of at most 256 workgroups and 256 or more tokens run eight waves per workgroup,
+    two teams on the two halves of the key tiles, merged through LDS: every query head against
+    float32 library attention."""
+    g = torch.Generator(device=device).manual_seed(T + pos + D)
+    q = torch.randn(T, Hq * D, device=device, generator=g).bfloat16()
+    k = torch.randn(1, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    v = torch.randn(1, Hkv, S_max, D, device=device, generator=g).bfloat16()
+    out = torch.empty_like(q)
+    ops.sdpa_prefill(q, k, v, torch.tensor([pos], dtype=torch.int32, device=device), out,
+                     D ** -0.5, 1, T, Hq, Hkv, D)
+    heads = list(range(Hq))
+    ref = _causal_ref(q, k[0], v[0], pos, T, heads, Hq, Hkv, D)
+    got = out.view(T, Hq, D).permute(1, 0, 2)
+    assert_close(n_f32(got), n_f32(ref), what=f"two-team prefill sdpa T={T} pos={pos} {Hq}/{Hkv} D={D}")
+
+
 def _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed, keys_hint=0):
     """exo_attn_decode (rope + append + attention) for B sequences at the given lengths,
     against: rope by the oracle, float32 library attention over the cache."""
