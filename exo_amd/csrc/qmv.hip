@@ -1310,8 +1310,9 @@ int check_common(const char* name, int M, int N, int K, int bits, int group_size
 // Exactly two rows over a short reduction run faster on the dot2 kernel with a two-row
 // activation tile (1.3-1.4 x the one-row time) than on the matrix-core GEMV (about 2 x);
 // from three rows on, and for long rows whose activations no longer stay in registers,
-// the matrix cores win.
-inline bool two_rows_on_dot2(int M, int K) { return M == 2 && K <= 8192; }
+// the matrix cores win.  (Rows of more than 4 KiB of codes - 8-bit beyond K = 4096 - would take
+// the two-row tile's instances that spill registers.)
+inline bool two_rows_on_dot2(int M, int K, int bits) { return M == 2 && (int64_t)K * bits <= 8192 * 4; }
 
 // A matrix this small (a MoE router: 128 x 2048 4-bit = 128 KiB) under 2...16 rows is a
 // latency-bound launch: one set of single-row workgroups per row (blockIdx.y), each reading
@@ -1354,7 +1355,7 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
   }
   // two or more rows: the matrix-core GEMV streams W once per tile of up to 16 rows
   // (with a workspace; without one a tile is as many rows as the LDS holds whole)
-  int cap = (M >= 2 && !two_rows_on_dot2(M, K)) ? exo_qmv_mfma_max_rows(K, bits) : 0;
+  int cap = (M >= 2 && !two_rows_on_dot2(M, K, bits)) ? exo_qmv_mfma_max_rows(K, bits) : 0;
   if (cap > 0 && workspace) cap = 16;
   if (cap >= 2) {
     int m0 = 0;
@@ -1441,7 +1442,7 @@ extern "C" int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_we
               (long long)workspace_bytes, (long long)exo_qmv_workspace(2 * N));
   if (M == 0) return EXO_OK;
   // two or more rows: both projections in one matrix-core launch per tile of up to 16 rows
-  if (workspace && M >= 2 && !two_rows_on_dot2(M, K) && exo_qmv_mfma_max_rows(K, bits) > 0) {
+  if (workspace && M >= 2 && !two_rows_on_dot2(M, K, bits) && exo_qmv_mfma_max_rows(K, bits) > 0) {
     int m0 = 0;
     while (M - m0 >= 2) {
       const int mt = (M - m0 < 16) ? (M - m0) : 16;

@@ -69,7 +69,7 @@ def test_embed_bit_exact(device, bits):
 
 QMV_SHAPES = [  # (N, K)
     (256, 4096), (64, 2048), (128, 14336), (96, 768), (64, 1536), (200, 8192), (128, 64),
-    (72, 192),
+    (72, 192), (160, 7168),
 ]
 
 
