@@ -168,7 +168,9 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 // every wave owns 64 of them, so nothing is dequantised twice.  Plain GEMM (inputs of up to
 // 64 rows): blockIdx.z always owns a K range and the tile leaves as a float32 partial.
 // Grouped GEMM (MI = 4: the expert's 128-row tile against 256 weight rows, the wave tile of
-// the 256-row kernel): whole K, the usual epilogue.
+// the 256-row kernel): whole K, the usual epilogue.  The same tile for the plain (gate, up)
+// pair of a long input: per product it stages half the activation bytes of the 256 x 64 tile
+// (the weights, re-read twice as often, are the smaller stream there).
 // DEEP (128-row tiles with SB4): four K steps of weights and three of activations in flight
 // instead of one.  A 128-row tile holds half the arithmetic per K step of the 256-row one, so
 // with one step in flight a workgroup spends most of a step waiting for the next one's loads,
@@ -183,7 +185,7 @@ __device__ __forceinline__ uint32_t dequant_piece(uint32_t lo, uint32_t hi, floa
 template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = false,
           bool WIDE = false, bool DEEP = false, bool KH = false>
 __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const QmmParams p) {
-  static_assert(!WIDE || GROUPED || !PAIR, "the wide pair tile is for the grouped GEMM");
+  static_assert(!WIDE || GROUPED || !PAIR || MI == 4, "the wide pair tile has 128 rows");
   static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
   static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !WIDE && !DEEP),
                 "two K halves per workgroup: the 256-row tile of the plain and the pair GEMM");
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   constexpr int SLOTS = 2;  // activation tiles in LDS
   // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
-  constexpr int XS_ROWS = (WIDE && GROUPED && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
+  constexpr int XS_ROWS = (WIDE && (GROUPED || PAIR) && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
   __shared__ __attribute__((aligned(16))) bf16_t xs[KH ? 2 * SLOTS : SLOTS][XS_ROWS * LDS_STRIDE];
 
   const int tid = threadIdx.x & (kThreads - 1), lane = tid & 63;  // within the team
@@ -484,7 +486,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     buf ^= 1;
   }
 
-  if ((WIDE && !GROUPED) || (!GROUPED && p.ksplit > 1)) {
+  if ((WIDE && !GROUPED && !PAIR) || (!GROUPED && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
     // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
@@ -1029,6 +1031,15 @@ void plan_pair_split(const QmmParams& p, bool have_ws, int* ksplit, int* kc) {
   *ksplit = exo_ceil_div(p.K, c);
 }
 
+#ifndef EXO_QMM_PAIR_WIDE_MIN_M
+#define EXO_QMM_PAIR_WIDE_MIN_M 129
+#endif
+// rows from which the (gate, up) pair takes the 128 x 128 tile with the four waves side by
+// side instead of the 256 x 64 one: ahead at every length measured (14336x4096 pair 4-bit:
+// 600 rows 216 -> 205 us, 1022 rows 303 -> 288, 2046 rows 504 -> 487, 4094 rows 954 -> 919;
+// 12288x4096 8-bit at 600 rows, whose third 256-row tile is mostly empty, 195 -> 139 us)
+constexpr int kPairWideMinM = EXO_QMM_PAIR_WIDE_MIN_M;
+
 template <int BITS>
 void launch_pair(const QmmParams& p, hipStream_t st) {
   const dim3 g2(exo_ceil_div(p.N, 64), exo_ceil_div(p.M, 128), p.ksplit),
@@ -1052,6 +1063,8 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
     // (up to one tall tile per CU: eight waves per tile, as in launch_qmm)
     if (sb4 && (int64_t)g4.x * g4.y <= 256 && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, true, false, false, true><<<g4, 512, 0, st>>>(p);
+    else if (sb4 && p.M >= kPairWideMinM)
+      qmm_kernel<BITS, 4, false, true, true, true><<<dim3(exo_ceil_div(p.N, 128), exo_ceil_div(p.M, 128)), 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
     else

@@ -167,12 +167,14 @@ def test_small_matrix_rows_equal_single_row_launches(device, bits, M, N, K):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("M,N,K", [(300, 256, 512), (129, 100, 192), (513, 192, 1024), (40, 64, 256), (2046, 1000, 320)])
+@pytest.mark.parametrize("M,N,K", [(300, 256, 512), (129, 100, 192), (513, 192, 1024), (40, 64, 256), (2046, 1000, 320),
+                                   (300, 4100, 768), (700, 8200, 768), (260, 4104, 1280)])
 def test_qmm_swiglu_pair(device, bits, M, N, K):
     """Gate and up projections with the SwiGLU in the GEMM's epilogue: the bits of the two
     GEMMs followed by the elementwise kernel (same products, same rounding points), and the
     oracle within tolerance.  Ragged M and N, N not a multiple of 8, K with and without the
-    four-step scale blocks."""
+    four-step scale blocks; the last three shapes are launches of more than 128 tall tiles,
+    which take the 128 x 128 tile with the four waves side by side."""
     g = rand_quantized(N, K, bits, seed=N + 11)
     u = rand_quantized(N, K, bits, seed=N + 12)
     x = rand_bf16((M, K), seed=M + K)
