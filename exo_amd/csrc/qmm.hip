@@ -453,13 +453,49 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
       if (!idle) multiply(wq[u], u & 1, sbc, u);
     }
   }
+  // RING (the 128-row wide tiles: the plain pair's and the grouped GEMM's): the activation tile is a quarter of the
+  // staging area, so four tiles fit; activations (straight into LDS) and weights (four
+  // register stages) are requested three K steps ahead.  Every request is unconditional
+  // (past the end of K the last step again, never multiplied) and the loop body is four steps
+  // long with static stage indices, so that the wait at the end of a step is an exact count:
+  // the two youngest steps' requests may still be out.
+  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4 && (GROUPED || PAIR);  // (8-bit: four
+                                                                                  // stages spill)
+  if (RING) {
+    constexpr int NW = 2 * (BITS / 4);  // weight requests per step
+    WStage wq[4];
+    SBlock sbc, sbn;
+    const int last = ke - BK;
+    load_sb(sbn, kb >> 8);
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      load_x(u, min(kb + u * BK, last));
+      load_w(wq[u], min(kb + u * BK, last));
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    for (int k0 = kb; k0 < ke; k0 += 4 * BK) {
+      sbc = sbn;  // this block's scales: requested a block ago (the first: above)
+      load_sb(sbn, min((k0 >> 8) + 1, (ke >> 8) - 1));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int kn = min(k0 + (u + 3) * BK, last);
+        load_x((u + 3) & 3, kn);
+        load_w(wq[(u + 3) & 3], kn);
+        multiply(wq[u], u, sbc, u);
+        wait_vm(std::integral_constant<int, 2 * (XR + NW)>{});
+        __syncthreads();
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the repeats requested past the end: landed before
+  }                                      // the staging below reuses this memory
   WStage w0, w1;
   SBlock sb0, sb1;  // current block of four K steps, next block
-  if (SB4 && !DEEP) {
+  if (SB4 && !DEEP && !RING) {
     load_sb(sb0, kb >> 8);
     sb1 = sb0;
   }
-  if (!DEEP) {
+  if (!DEEP && !RING) {
     load_x(0, kb);
     if (!idle) load_w(w0, kb);
   }
@@ -469,7 +505,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // The tile and the weights of k+1 are requested first, then tile k is multiplied; every
   // load of the step has landed before the one barrier that ends it.
   int buf = 0;
-  for (int k0 = kb; !DEEP && k0 < ke; k0 += BK) {
+  for (int k0 = kb; !DEEP && !RING && k0 < ke; k0 += BK) {
     const int ks = k0 >> 6;
     if (SB4 && (ks & 3) == 0) {  // a new block: its values arrived during the previous one
       sb0 = sb1;
