@@ -187,8 +187,9 @@ template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = 
 __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const QmmParams p) {
   static_assert(!WIDE || GROUPED || !PAIR || MI == 4, "the wide pair tile has 128 rows");
   static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
-  static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !WIDE && !DEEP),
-                "two K halves per workgroup: the 256-row tile of the plain and the pair GEMM");
+  static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !DEEP && !(WIDE && PAIR)),
+                "two K halves per workgroup: the 256-row tile of the plain and the pair GEMM, "
+                "the wide tile of the plain GEMM");
   constexpr int kThreads = 256;  // of a team
   constexpr int BM = WIDE ? 32 * MI : 64 * MI;
   constexpr int WN = PAIR ? 32 : 64;              // output columns per wave
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   constexpr int SLOTS = 2;  // activation tiles in LDS
   // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
-  constexpr int XS_ROWS = (WIDE && (GROUPED || PAIR) && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
+  constexpr int XS_ROWS = (WIDE && (GROUPED || PAIR || KH) && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
   __shared__ __attribute__((aligned(16))) bf16_t xs[KH ? 2 * SLOTS : SLOTS][XS_ROWS * LDS_STRIDE];
 
   const int tid = threadIdx.x & (kThreads - 1), lane = tid & 63;  // within the team
@@ -279,7 +280,8 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // store instructions): wave instruction r writes chunks [wave*64 + 256*r, +64) in lane
   // order.  Completion is counted by vmcnt.
   constexpr int TILE_BYTES = BM * 128;
-  char* const tiles = reinterpret_cast<char*>(&xs[0][0]) + team * (SLOTS * TILE_BYTES);
+  // (a team's tiles: two, or the four of the ring)
+  char* const tiles = reinterpret_cast<char*>(&xs[0][0]) + team * ((KH && WIDE ? 4 : SLOTS) * TILE_BYTES);
   auto load_x = [&](int buf, int k0) {
 #pragma unroll
     for (int r = 0; r < XR; ++r)
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // (past the end of K the last step again, never multiplied) and the loop body is four steps
   // long with static stage indices, so that the wait at the end of a step is an exact count:
   // the two youngest steps' requests may still be out.
-  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4 && (GROUPED || PAIR);  // (8-bit: four
+  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4 && (GROUPED || PAIR || KH);  // (8-bit: four
                                                                                   // stages spill)
   if (RING) {
     constexpr int NW = 2 * (BITS / 4);  // weight requests per step
@@ -522,7 +524,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     buf ^= 1;
   }
 
-  if ((WIDE && !GROUPED && !PAIR) || (!GROUPED && p.ksplit > 1)) {
+  if ((WIDE && !GROUPED && !PAIR && !KH) || (!GROUPED && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
     // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
@@ -799,6 +801,15 @@ bool plan_wide(int M, int N, int K, const QmmParams& p, bool have_ws, int* kspli
   return true;
 }
 
+#ifndef EXO_QMM_WIDE_HALVES
+#define EXO_QMM_WIDE_HALVES 1
+#endif
+constexpr bool kWideHalves = EXO_QMM_WIDE_HALVES != 0;
+#ifndef EXO_QMM_WIDE_HALVES_MAX_TILES
+#define EXO_QMM_WIDE_HALVES_MAX_TILES 256
+#endif
+constexpr int kWideHalvesMaxTiles = EXO_QMM_WIDE_HALVES_MAX_TILES;
+
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
@@ -840,7 +851,15 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     // 4096x14336: 279 -> 266 us, 6144x4096 under 1022 rows, 192 tiles: 82.0 -> 77.5 us; more
     // tiles than CUs lose (384: 127 -> 144 us, 512: 155 -> 171 us)
     const int64_t tall = (int64_t)g4.x * g4.y;
-    if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
+    // 4-bit, up to one WIDE tile (128 x 256) per CU: the two K halves on that tile instead,
+    // with the ring of four - half the staged activation bytes per product and the weights
+    // three steps ahead (4096x4096 under 2046 rows 89.5 -> 84.8 us, 4096x14336 280 -> 239,
+    // 6144x4096 under 1022 rows 87 -> 78, 8192x8192 under 600 rows 138 -> 122; with up to 512
+    // such tiles it wins on some shapes and loses on others, so 256 it is)
+    const dim3 gw(exo_ceil_div(N, 256), exo_ceil_div(M, 128));
+    if (kWideHalves && sb4 && BITS == 4 && (int64_t)gw.x * gw.y <= kWideHalvesMaxTiles && p.K % 512 == 0 && p.K >= 1024)
+      qmm_kernel<BITS, 4, false, true, false, true, false, true><<<gw, 512, 0, st>>>(p);
+    else if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);

@@ -245,6 +245,22 @@ def test_qmm_split_k(device, bits, M, N, K):
     assert_close(got_r, affine.bf16_round(affine.bf16_round(want) + r), what="qmm split-K + residual")
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(1100, 4100, 1024), (1300, 2052, 1536), (700, 8192, 1024)])
+def test_qmm_eight_wave_tiles(device, bits, M, N, K):
+    """Launches of more than 128 tall tiles but at most one tile per CU run eight waves per
+    tile, two teams on the two halves of K merged through LDS: the wide 128 x 256 tile with
+    the ring of four (4-bit) or the 256 x 128 tile (8-bit).  Ragged M and N, with the residual."""
+    trip = rand_quantized(N, K, bits, seed=M + N)
+    x = rand_bf16((M, K), seed=M * 3 + 1)
+    r = rand_bf16((M, N), seed=M + 5)
+    qw, xt, rt = t_qw(trip, bits, device), t_bf16(x, device), t_bf16(r, device)
+    want = affine.qmm(x, *trip, 64, bits)
+    assert_close(n_f32(ops.qmm(xt, qw)), want, what=f"qmm {M}x{N}x{K} b{bits}")
+    got_r = n_f32(ops.quantized_matmul(xt, qw, residual=rt))
+    assert_close(got_r, affine.bf16_round(affine.bf16_round(want) + r), what="qmm + residual")
+
+
 def test_qmm_residual_and_dispatch(device):
     M, N, K, bits = 40, 192, 256, 4
     trip = rand_quantized(N, K, bits, seed=5)
