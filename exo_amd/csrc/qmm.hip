@@ -197,7 +197,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   constexpr int SLOTS = 2;  // activation tiles in LDS
   // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
-  constexpr int XS_ROWS = (WIDE && (GROUPED || PAIR || KH) && 2 * 32 * MI > BM) ? 2 * 32 * MI : BM;
+  constexpr int XS_ROWS = (WIDE && MI == 4) ? 2 * 32 * MI : BM;
   __shared__ __attribute__((aligned(16))) bf16_t xs[KH ? 2 * SLOTS : SLOTS][XS_ROWS * LDS_STRIDE];
 
   const int tid = threadIdx.x & (kThreads - 1), lane = tid & 63;  // within the team
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // (past the end of K the last step again, never multiplied) and the loop body is four steps
   // long with static stage indices, so that the wait at the end of a step is an exact count:
   // the two youngest steps' requests may still be out.
-  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4 && (GROUPED || PAIR || KH);  // (8-bit: four
+  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4;  // (8-bit: four
                                                                                   // stages spill)
   if (RING) {
     constexpr int NW = 2 * (BITS / 4);  // weight requests per step
@@ -524,7 +524,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     buf ^= 1;
   }
 
-  if ((WIDE && !GROUPED && !PAIR && !KH) || (!GROUPED && p.ksplit > 1)) {
+  if ((WIDE && MI < 4) || (!GROUPED && p.ksplit > 1)) {
     // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
     // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
     // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
@@ -809,6 +809,10 @@ constexpr bool kWideHalves = EXO_QMM_WIDE_HALVES != 0;
 #define EXO_QMM_WIDE_HALVES_MAX_TILES 256
 #endif
 constexpr int kWideHalvesMaxTiles = EXO_QMM_WIDE_HALVES_MAX_TILES;
+#ifndef EXO_QMM_WIDE_RING_MIN_TILES
+#define EXO_QMM_WIDE_RING_MIN_TILES 257
+#endif
+constexpr int kWideRingMinTiles = EXO_QMM_WIDE_RING_MIN_TILES;
 
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
@@ -861,6 +865,11 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
       qmm_kernel<BITS, 4, false, true, false, true, false, true><<<gw, 512, 0, st>>>(p);
     else if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
+    // more wide tiles than CUs: the wide tile with the ring, four waves (6144x4096 under 2046
+    // rows 144 -> 126 us, 4096x14336 under 4094 rows 523 -> 472, 8192x8192 under 2046 rows
+    // 292 -> 270)
+    else if (sb4 && BITS == 4 && (int64_t)gw.x * gw.y >= kWideRingMinTiles)
+      qmm_kernel<BITS, 4, false, true, false, true><<<gw, 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
     else
