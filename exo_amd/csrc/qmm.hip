@@ -801,6 +801,14 @@ bool plan_wide(int M, int N, int K, const QmmParams& p, bool have_ws, int* kspli
   return true;
 }
 
+// The wide tile is 128 rows tall: it streams the weights once per 128 input rows where the
+// 256-row tile streams them once per 256.  That is the smaller stream as long as the matrix
+// stays in the 256 MB last-level cache between passes; a vocabulary-sized one (128256x4096:
+// 295 MB) does not, and ran 10 % slower through the wide tile (2338 -> 2572 us under 2048 rows).
+inline bool weights_stay_cached(int64_t rows, int K, int bits) {
+  return rows * K * bits / 8 <= (int64_t)128 << 20;
+}
+
 #ifndef EXO_QMM_WIDE_HALVES
 #define EXO_QMM_WIDE_HALVES 1
 #endif
@@ -868,7 +876,7 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     // more wide tiles than CUs: the wide tile with the ring, four waves (6144x4096 under 2046
     // rows 144 -> 126 us, 4096x14336 under 4094 rows 523 -> 472, 8192x8192 under 2046 rows
     // 292 -> 270)
-    else if (sb4 && BITS == 4 && (int64_t)gw.x * gw.y >= kWideRingMinTiles)
+    else if (sb4 && BITS == 4 && (int64_t)gw.x * gw.y >= kWideRingMinTiles && weights_stay_cached(N, p.K, BITS))
       qmm_kernel<BITS, 4, false, true, false, true><<<gw, 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
@@ -1127,7 +1135,7 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
     // (up to one tall tile per CU: eight waves per tile, as in launch_qmm)
     if (sb4 && (int64_t)g4.x * g4.y <= 256 && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, true, false, false, true><<<g4, 512, 0, st>>>(p);
-    else if (sb4 && p.M >= kPairWideMinM)
+    else if (sb4 && p.M >= kPairWideMinM && weights_stay_cached(2 * (int64_t)p.N, p.K, BITS))
       qmm_kernel<BITS, 4, false, true, true, true><<<dim3(exo_ceil_div(p.N, 128), exo_ceil_div(p.M, 128)), 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
