@@ -46,6 +46,10 @@
 
 namespace {
 
+#ifndef EXO_QMM_RING8
+#define EXO_QMM_RING8 1
+#endif
+constexpr bool kRing8 = EXO_QMM_RING8 != 0;  // the ring for 8-bit weights too
 constexpr int BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row
 
@@ -461,8 +465,9 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // (past the end of K the last step again, never multiplied) and the loop body is four steps
   // long with static stage indices, so that the wait at the end of a step is an exact count:
   // the two youngest steps' requests may still be out.
-  constexpr bool RING = WIDE && MI == 4 && SB4 && BITS == 4;  // (8-bit: four
-                                                                                  // stages spill)
+  constexpr bool RING = WIDE && MI == 4 && SB4 && (BITS == 4 || kRing8);
+  // (8-bit: two steps ahead - three live stages of 16 registers; four spill)
+  constexpr int AHEAD = BITS == 4 ? 3 : 2;
   if (RING) {
     constexpr int NW = 2 * (BITS / 4);  // weight requests per step
     WStage wq[4];
@@ -470,7 +475,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     const int last = ke - BK;
     load_sb(sbn, kb >> 8);
 #pragma unroll
-    for (int u = 0; u < 3; ++u) {
+    for (int u = 0; u < AHEAD; ++u) {
       load_x(u, min(kb + u * BK, last));
       load_w(wq[u], min(kb + u * BK, last));
     }
@@ -481,11 +486,11 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
       load_sb(sbn, min((k0 >> 8) + 1, (ke >> 8) - 1));
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int kn = min(k0 + (u + 3) * BK, last);
-        load_x((u + 3) & 3, kn);
-        load_w(wq[(u + 3) & 3], kn);
+        const int kn = min(k0 + (u + AHEAD) * BK, last);
+        load_x((u + AHEAD) & 3, kn);
+        load_w(wq[(u + AHEAD) & 3], kn);
         multiply(wq[u], u, sbc, u);
-        wait_vm(std::integral_constant<int, 2 * (XR + NW)>{});
+        wait_vm(std::integral_constant<int, (AHEAD - 1) * (XR + NW)>{});
         __syncthreads();
       }
     }
@@ -869,14 +874,14 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     // 6144x4096 under 1022 rows 87 -> 78, 8192x8192 under 600 rows 138 -> 122; with up to 512
     // such tiles it wins on some shapes and loses on others, so 256 it is)
     const dim3 gw(exo_ceil_div(N, 256), exo_ceil_div(M, 128));
-    if (kWideHalves && sb4 && BITS == 4 && (int64_t)gw.x * gw.y <= kWideHalvesMaxTiles && p.K % 512 == 0 && p.K >= 1024)
+    if (kWideHalves && sb4 && (BITS == 4 || kRing8) && (int64_t)gw.x * gw.y <= kWideHalvesMaxTiles && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, false, true, false, true><<<gw, 512, 0, st>>>(p);
     else if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
       qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
     // more wide tiles than CUs: the wide tile with the ring, four waves (6144x4096 under 2046
     // rows 144 -> 126 us, 4096x14336 under 4094 rows 523 -> 472, 8192x8192 under 2046 rows
     // 292 -> 270)
-    else if (sb4 && BITS == 4 && (int64_t)gw.x * gw.y >= kWideRingMinTiles && weights_stay_cached(N, p.K, BITS))
+    else if (sb4 && (BITS == 4 || kRing8) && (int64_t)gw.x * gw.y >= kWideRingMinTiles && weights_stay_cached(N, p.K, BITS))
       qmm_kernel<BITS, 4, false, true, false, true><<<gw, 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
