@@ -190,7 +190,9 @@ template <int BITS, int MI, bool GROUPED = false, bool SB4 = false, bool PAIR = 
           bool WIDE = false, bool DEEP = false, bool KH = false>
 __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const QmmParams p) {
   static_assert(!WIDE || GROUPED || !PAIR || MI == 4, "the wide pair tile has 128 rows");
-  static_assert(!DEEP || (SB4 && MI == 2 && !WIDE), "the deep pipeline is for 128-row tiles");
+  static_assert(!DEEP || (SB4 && ((MI == 2 && !WIDE) || (WIDE && MI < 4))),
+                "the deep pipeline is for 128-row tiles; on the 32- and 64-row wide tiles the flag "
+                "selects the ring (K ranges long enough to fill it)");
   static_assert(!KH || (MI == 4 && SB4 && !GROUPED && !DEEP && !(WIDE && PAIR)),
                 "two K halves per workgroup: the 256-row tile of the plain and the pair GEMM, "
                 "the wide tile of the plain GEMM");
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   constexpr int XR = BM * 8 / kThreads;  // 16-byte x loads per thread and K step
   constexpr int SLOTS = 2;  // activation tiles in LDS
   // (the grouped wide tile leaves through the staging epilogue: four waves x 32*MI rows)
-  constexpr int XS_ROWS = (WIDE && MI == 4) ? 2 * 32 * MI : BM;
+  constexpr int XS_ROWS = WIDE ? 2 * BM : BM;  // (wide: room for the ring's four tiles)
   __shared__ __attribute__((aligned(16))) bf16_t xs[KH ? 2 * SLOTS : SLOTS][XS_ROWS * LDS_STRIDE];
 
   const int tid = threadIdx.x & (kThreads - 1), lane = tid & 63;  // within the team
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // this workgroup's K range (all of K unless split; a multiple of four K steps)
   const int kb = KH ? team * (p.K >> 1) : GROUPED ? 0 : (int)blockIdx.z * p.kc;
   const int ke = KH ? kb + (p.K >> 1) : GROUPED ? p.K : min(p.K, kb + p.kc);
-  if (DEEP) {
+  if (DEEP && !WIDE) {
     // Four register stages each of weights and of activation chunks, requested four steps
     // ahead; the activations pass through registers into the two LDS tiles one step ahead
     // (no LDS-direct loads here: the compiler makes every LDS read wait for ALL outstanding
@@ -465,9 +467,10 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // (past the end of K the last step again, never multiplied) and the loop body is four steps
   // long with static stage indices, so that the wait at the end of a step is an exact count:
   // the two youngest steps' requests may still be out.
-  constexpr bool RING = WIDE && MI == 4 && SB4 && (BITS == 4 || kRing8);
+  constexpr bool RING = WIDE && SB4 && (BITS == 4 || kRing8) && (MI == 4 || DEEP);
   // (8-bit: two steps ahead - three live stages of 16 registers; four spill)
   constexpr int AHEAD = BITS == 4 ? 3 : 2;
+  static_assert(RING || !(WIDE && DEEP), "a wide tile with the pipeline flag runs the ring");
   if (RING) {
     constexpr int NW = 2 * (BITS / 4);  // weight requests per step
     WStage wq[4];
@@ -827,13 +830,25 @@ constexpr int kWideHalvesMaxTiles = EXO_QMM_WIDE_HALVES_MAX_TILES;
 #endif
 constexpr int kWideRingMinTiles = EXO_QMM_WIDE_RING_MIN_TILES;
 
+#ifndef EXO_QMM_WIDE_RING_MIN_K
+#define EXO_QMM_WIDE_RING_MIN_K 768
+#endif
+constexpr int kWideRingMinK = EXO_QMM_WIDE_RING_MIN_K;
+
 template <int BITS>
 void launch_qmm(const QmmParams& p, hipStream_t st) {
   const int M = p.M, N = p.N;
   if (p.wide) {
     const dim3 g(exo_ceil_div(N, 256), 1, p.ksplit);
-    if (M <= 32)
+    // K ranges of twelve steps or more fill the ring (4096x14336 4-bit at 17 rows 22.3 -> 19.3
+    // us); on short ranges its start-up costs more than it returns (14336x4096: 20.5 -> 21.4)
+    const bool ring = p.kc >= kWideRingMinK;
+    if (M <= 32 && ring)
+      qmm_kernel<BITS, 1, false, true, false, true, true><<<g, 256, 0, st>>>(p);
+    else if (M <= 32)
       qmm_kernel<BITS, 1, false, true, false, true><<<g, 256, 0, st>>>(p);
+    else if (ring)
+      qmm_kernel<BITS, 2, false, true, false, true, true><<<g, 256, 0, st>>>(p);
     else
       qmm_kernel<BITS, 2, false, true, false, true><<<g, 256, 0, st>>>(p);
     const int64_t total = (int64_t)M * N;
