@@ -405,8 +405,11 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
   // the other LDS buffer and its registers are refilled two steps ahead, the current tile
   // is multiplied, the freed weight stage is refilled two steps ahead; one barrier.
   // this workgroup's K range (all of K unless split; a multiple of four K steps)
-  const int kb = KH ? team * (p.K >> 1) : GROUPED ? 0 : (int)blockIdx.z * p.kc;
-  const int ke = KH ? kb + (p.K >> 1) : GROUPED ? p.K : min(p.K, kb + p.kc);
+  // (two teams: the halves of the workgroup's range - all of K unless the launch splits it)
+  const int kr0 = GROUPED ? 0 : (int)blockIdx.z * p.kc;
+  const int klen = GROUPED ? p.K : min(p.K, kr0 + p.kc) - kr0;
+  const int kb = KH ? kr0 + team * (klen >> 1) : kr0;
+  const int ke = KH ? kb + (klen >> 1) : kr0 + klen;
   if (DEEP && !WIDE) {
     // Four register stages each of weights and of activation chunks, requested four steps
     // ahead; the activations pass through registers into the two LDS tiles one step ahead
@@ -532,27 +535,6 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     buf ^= 1;
   }
 
-  if ((WIDE && MI < 4) || (!GROUPED && p.ksplit > 1)) {
-    // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
-    // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
-    // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
-    const size_t one = part_stride(p.M, p.N);
-    float* mine = p.part + (size_t)blockIdx.z * (PAIR ? 2 * one : one);
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int n = PAIR ? n0 + wn + frow : n0 + wn + j * 32 + frow;
-        float* dst = mine + ((PAIR && j) ? one : 0);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
-          if (m < m_end && n < p.N) dst[(size_t)m * p.N + n] = acc[i][j][r];
-        }
-      }
-    return;
-  }
-
   if (KH) {
     // the second team's sums: through LDS (lane-contiguous floats per accumulator register),
     // added to the first team's, which goes on alone
@@ -582,6 +564,28 @@ __global__ __launch_bounds__(KH ? 512 : 256, KH ? 1 : 2) void qmm_kernel(const Q
     __syncthreads();  // the sums have been read: the staging below overwrites this memory
     if (team == 1) return;  // (no workgroup barrier after this point)
   }
+
+  if ((WIDE && MI < 4) || (!GROUPED && p.ksplit > 1)) {
+    // Split-K: the float32 partial tile of this K range goes to the workspace; a second,
+    // small launch adds the ranges in a fixed order (qmm_reduce_kernel).  Pair mode: a range
+    // holds the gate partials followed by the up partials (qmm_reduce_swiglu_kernel).
+    const size_t one = part_stride(p.M, p.N);
+    float* mine = p.part + (size_t)blockIdx.z * (PAIR ? 2 * one : one);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int n = PAIR ? n0 + wn + frow : n0 + wn + j * 32 + frow;
+        float* dst = mine + ((PAIR && j) ? one : 0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+          if (m < m_end && n < p.N) dst[(size_t)m * p.N + n] = acc[i][j][r];
+        }
+      }
+    return;
+  }
+
 
   // Epilogue through LDS.  D[i][j] holds column lane%32 (W row n) and rows
   // 8*(r/4) + 4*(lane/32) + r%4 (token m): a wave first writes its (32*MI) x 64 tile as bf16
@@ -830,6 +834,15 @@ constexpr int kWideHalvesMaxTiles = EXO_QMM_WIDE_HALVES_MAX_TILES;
 #endif
 constexpr int kWideRingMinTiles = EXO_QMM_WIDE_RING_MIN_TILES;
 
+#ifndef EXO_QMM_WIDE_SPLIT
+#define EXO_QMM_WIDE_SPLIT 1
+#endif
+#ifndef EXO_QMM_WIDE_SPLIT_MIN_K
+#define EXO_QMM_WIDE_SPLIT_MIN_K 1024
+#endif
+constexpr bool kWideSplit = EXO_QMM_WIDE_SPLIT != 0;
+constexpr int kWideSplitMinK = EXO_QMM_WIDE_SPLIT_MIN_K;
+constexpr int kWideSplitMinWgs = 160;
 #ifndef EXO_QMM_WIDE_RING_MIN_K
 #define EXO_QMM_WIDE_RING_MIN_K 768
 #endif
@@ -865,7 +878,18 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
   // 1023 rows, exactly 128 tall tiles: 93 -> 77 us), not beyond (192 tall tiles: 88 vs 97 us)
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (M <= 128 || small_grid || p.ksplit > 1) {  // (only the 128-row tile splits K)
-    if (sb4 && p.kc >= kDeepMinK)
+    // K ranges of 1024 or more, all of one length: the wide tile with eight waves, the two
+    // teams on the halves of the workgroup's range (no weight row dequantised twice, the ring,
+    // as many partial tiles as before): 4096x14336 4-bit under 600 rows 145 -> 104 us, 4096x4096
+    // 52 -> 43, 6144x4096 under 300 rows 48 -> 40, 14336x4096 under 128 rows 41 -> 37; launches
+    // that would have fewer than 160 such workgroups lose (2048x4096 under 1022 rows, 128
+    // workgroups: 37 -> 42 us)
+    if (kWideSplit && sb4 && (BITS == 4 || kRing8) && p.ksplit > 1 && M > 64 && p.kc >= kWideSplitMinK &&
+        p.kc % 512 == 0 && p.K % p.kc == 0 &&
+        (int64_t)exo_ceil_div(N, 256) * exo_ceil_div(M, 128) * p.ksplit >= kWideSplitMinWgs)
+      qmm_kernel<BITS, 4, false, true, false, true, false, true>
+          <<<dim3(exo_ceil_div(N, 256), exo_ceil_div(M, 128), p.ksplit), 512, 0, st>>>(p);
+    else if (sb4 && p.kc >= kDeepMinK)
       qmm_kernel<BITS, 2, false, true, false, false, true><<<g2, 256, 0, st>>>(p);
     else if (sb4)
       qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);

@@ -224,13 +224,16 @@ def test_qmm_mfma(device, bits, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(100, 256, 4096), (33, 130, 14336), (128, 1000, 2048), (17, 64, 1024),
                                    (12, 256, 8192), (9, 96, 1024), (1023, 128, 2048), (300, 200, 4096),
                                    (32, 520, 512), (64, 600, 1024), (65, 300, 768), (20, 257, 256),
-                                   (300, 10880, 1024), (1023, 2048, 1024)])
+                                   (300, 10880, 1024), (1023, 2048, 1024), (300, 4100, 4096), (100, 14336, 4096),
+                                   (600, 2052, 4096)])
 def test_qmm_split_k(device, bits, M, N, K):
     """Few output tiles (a short input, or a narrow matrix under a long one): K is split
     over workgroups and the float32 partial tiles are added by a second launch.  Against
     the oracle, against the
     unsplit kernel (same products, another summation order: a few bf16 ulps at most),
-    with the residual, and twice in a row (the counters return to zero)."""
+    with the residual, and twice in a row (the counters return to zero).  The last three
+    shapes have K ranges of 1024 and take the wide tile with eight waves (two teams on the
+    halves of a range)."""
     trip = rand_quantized(N, K, bits, seed=M + N)
     x = rand_bf16((M, K), seed=M * 3 + 1)
     r = rand_bf16((M, N), seed=M + 5)
