@@ -943,7 +943,11 @@ extern "C" int exo_attn_decode_hint(const uint16_t* qkv, uint16_t* k_cache, uint
   // the matrix-core kernel's workgroups; 32 / 4 heads: 4 sequences level, 8 sequences
   // 22.7 -> 18.4 us; 64 / 4 heads: 4 sequences 21.1 -> 19.2, 8 sequences 34.2 -> 23.5 us)
   const int G = Hq / Hkv;
-  const bool long_ctx = keys_hint >= kAttnLongKeys && S_max >= kAttnLongKeys;
+  // (two sequences of 32 / 8 heads - 16 (sequence, kv head) pairs, enough workgroups for the
+  // matrix-core kernel - are level at 2050 keys and ahead beyond: 3000 keys 15.5 -> 14.2 us,
+  // 4096 keys 18.9 -> 16.1, 6144 keys 25.5 -> 19.4)
+  const int long_keys = B * Hkv >= 16 ? EXO_ATTN_MID_KEYS : kAttnLongKeys;
+  const bool long_ctx = keys_hint >= long_keys && S_max >= long_keys;
   if (D == 128 && (G == 4 || G == 8 || G == 16) &&
       ((B * Hq >= 128 && B * Hkv >= 16) || long_ctx)) {
     const int max_sp = keys_hint >= kAttnVeryLongKeys && S_max >= kAttnVeryLongKeys ? kMaxSplitsLong : kMaxSplits;

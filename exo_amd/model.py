@@ -253,7 +253,8 @@ class ShardModel:
         captured step stays valid inside one."""
         n = max(cache.offsets[rsl]) + 1
         return (ops.ATTN_VERY_LONG_KEYS if n >= ops.ATTN_VERY_LONG_KEYS else
-                ops.ATTN_LONG_KEYS if n >= ops.ATTN_LONG_KEYS else 0)
+                ops.ATTN_LONG_KEYS if n >= ops.ATTN_LONG_KEYS else
+                ops.ATTN_MID_KEYS if n >= ops.ATTN_MID_KEYS else 0)
 
     def _run(self, B: int, T: int, cache: ShardKVCache, bf: _Buffers, logits_mode: str,
              rows: slice | None = None):

@@ -563,7 +563,8 @@ def rope_table(inv_freq: torch.Tensor, S_max: int, D: int) -> torch.Tensor:
     return tab
 
 
-ATTN_LONG_KEYS = 6144        # EXO_ATTN_LONG_KEYS of the C header
+ATTN_MID_KEYS = 3072         # EXO_ATTN_MID_KEYS of the C header
+ATTN_LONG_KEYS = 6144        # EXO_ATTN_LONG_KEYS
 ATTN_VERY_LONG_KEYS = 12288  # EXO_ATTN_VERY_LONG_KEYS
 
 

@@ -286,11 +286,13 @@ int exo_attn_decode(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,
 /* exo_attn_decode with the host's knowledge of the context: keys_hint = the number of keys
  * the longest sequence of this step holds, as far as the host knows (0: unknown, which is
  * exo_attn_decode).  From EXO_ATTN_LONG_KEYS keys on (in a cache at least that long) the
- * launch is laid out for long contexts: the matrix-core kernel whatever the head count; from
+ * launch is laid out for long contexts: the matrix-core kernel whatever the head count
+ * (already from EXO_ATTN_MID_KEYS on when B * n_kv_heads is 16 or more); from
  * EXO_ATTN_VERY_LONG_KEYS on with the keys of a kv head over up to 32 workgroups instead of
  * 16.  The hint only selects the layout - any value gives a correct result for any pos[] -
  * so a captured launch stays valid while the context grows; the layouts round differently
  * (within the tolerance of the attention tests). */
+#define EXO_ATTN_MID_KEYS 3072
 #define EXO_ATTN_LONG_KEYS 6144
 #define EXO_ATTN_VERY_LONG_KEYS 12288
 int exo_attn_decode_hint(const uint16_t* qkv, uint16_t* k_cache, uint16_t* v_cache,

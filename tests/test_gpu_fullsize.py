@@ -320,6 +320,19 @@ def test_fused_decode_attention_long_context_layout(device, B, Hq, Hkv, lens, S_
     _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0] + 7, keys_hint=hint)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,lens,S_max", [
+    (2, 32, 8, [3072, 2000], 4096),                    # the first step of the layout
+    (2, 32, 8, [6000, 1], 8192),
+    (3, 32, 8, [4500, 3071, 8192], 8192),
+    (1, 32, 8, [4000], 8192),                          # one sequence: stays on the scalar kernel
+])
+def test_fused_decode_attention_mid_context_layout(device, B, Hq, Hkv, lens, S_max):
+    """exo_attn_decode_hint with the hint at the middle threshold: the matrix-core kernel
+    already from 3072 keys when the step has 16 or more (sequence, kv head) pairs."""
+    _fused_decode_case(device, B, Hq, Hkv, lens, S_max, seed=B * 1000 + lens[0] + 9,
+                       keys_hint=ops.ATTN_MID_KEYS)
+
+
 def test_attention_layouts_share_a_workspace(device):
     """One workspace, zeroed once, taken in turn by the three layouts (their counters sit at
     the same place, the partials of one never reach the counters)."""

@@ -265,7 +265,7 @@ def test_decode_step_recaptures_when_the_context_regime_changes(ckpt, device):
     got = [int(gm.decode_step(cg, 1, feedback=True).next_token[0]) for _ in range(8)]
     assert got == want
     assert cg.offsets[0] == start + 8 and cg.pos.tolist() == [start + 8]
-    for hint in (0, ops.ATTN_LONG_KEYS):  # one capture per regime, both on this cache
+    for hint in (ops.ATTN_MID_KEYS, ops.ATTN_LONG_KEYS):  # one capture per regime, both on this cache
         assert gm._graphs[(1, True, False, 0, 0, hint)][1] is cg
 
 

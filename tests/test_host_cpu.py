@@ -103,20 +103,23 @@ def test_bench_reads_the_committed_counter_summary():
 
 def test_decode_context_regimes():
     """The decode step's attention layout follows the host's count of the longest sequence of
-    the rows it serves: below 6144 keys, from 6144, from 12288 (one captured graph each)."""
+    the rows it serves: below 3072 keys, from 3072, from 6144, from 12288 (one captured graph
+    each)."""
     from types import SimpleNamespace
     from exo_amd import ops
     from exo_amd.model import ShardModel
     cache = SimpleNamespace(offsets=[10, 6142, 6143, 12286, 12287, 40000])
     hint = ShardModel._keys_hint
-    assert hint(cache, slice(0, 1)) == 0 and hint(cache, slice(0, 2)) == 0
+    assert hint(cache, slice(0, 1)) == 0 and hint(cache, slice(0, 2)) == ops.ATTN_MID_KEYS
+    assert hint(SimpleNamespace(offsets=[3070]), slice(0, 1)) == 0
+    assert hint(SimpleNamespace(offsets=[3071]), slice(0, 1)) == ops.ATTN_MID_KEYS
     assert hint(cache, slice(0, 3)) == ops.ATTN_LONG_KEYS          # 6143 cached + the new key
     assert hint(cache, slice(2, 4)) == ops.ATTN_LONG_KEYS
     assert hint(cache, slice(3, 5)) == ops.ATTN_VERY_LONG_KEYS
     assert hint(cache, slice(0, 6)) == ops.ATTN_VERY_LONG_KEYS
     assert (ops.ATTN_LONG_KEYS, ops.ATTN_VERY_LONG_KEYS) == (6144, 12288)
     hdr = (ROOT / "include" / "exo_mi355x.h").read_text()
-    assert "#define EXO_ATTN_LONG_KEYS 6144" in hdr and "#define EXO_ATTN_VERY_LONG_KEYS 12288" in hdr
+    assert "#define EXO_ATTN_MID_KEYS 3072" in hdr and "#define EXO_ATTN_LONG_KEYS 6144" in hdr and "#define EXO_ATTN_VERY_LONG_KEYS 12288" in hdr
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
