@@ -98,6 +98,8 @@ __device__ __forceinline__ void wait_own_stores_done() {
 #define EXO_ERR_HIP (-2)
 
 void exo_set_error(const char* fmt, ...);
+// records the kernel instance a launcher chose (read back with exo_last_variant())
+void exo_note_variant(const char* fmt, ...);
 
 #define EXO_REQUIRE(cond, ...)      \
   do {                              \

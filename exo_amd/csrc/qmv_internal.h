@@ -14,3 +14,11 @@ int exo_qmv_mfma_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
                         const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
                         const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
                         int bits, void* workspace, hipStream_t st);
+
+// 4x4x4 matrix-core GEMV for 1..16 activation rows (qmv_quad.hip): rows of whole 256-byte
+// slices, N a multiple of 4.  w2/s2/b2 non-null: the (gate, up) pair with SwiGLU.
+bool exo_qmv_quad_ok(int M, int N, int K, int bits, bool norm);
+int exo_qmv_quad_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
+                        const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
+                        const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
+                        int bits, hipStream_t st);

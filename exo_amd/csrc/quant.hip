@@ -23,6 +23,20 @@ void exo_set_error(const char* fmt, ...) {
 }
 
 extern "C" const char* exo_last_error(void) { return g_err; }
+
+// Which kernel instance and launch shape the calling thread's latest matmul / attention
+// entry point chose (diagnostic: lets a test assert that a shape reached the instance it
+// was written for).
+static thread_local char g_variant[256] = "";
+
+void exo_note_variant(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_variant, sizeof(g_variant), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* exo_last_variant(void) { return g_variant; }
 extern "C" int exo_abi_version(void) { return 1; }
 extern "C" int exo_dequant_two_roundings(void) { return EXO_DEQUANT_TWO_ROUNDINGS; }
 

@@ -20,6 +20,7 @@ _f = C.c_float
 SIGNATURES: dict[str, tuple] = {
     "exo_abi_version": (_i, []),
     "exo_last_error": (C.c_char_p, []),
+    "exo_last_variant": (C.c_char_p, []),
     "exo_dequant_two_roundings": (_i, []),
     "exo_unpack_codes": (_i, [_vp, _vp, _i64, _i, _vp]),
     "exo_dequantize": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
@@ -100,3 +101,8 @@ def check(rc: int, what: str) -> None:
         if rc == -1:
             raise ValueError(f"{what}: {msg}")
         raise NativeError(f"{what}: {msg} (rc={rc})")
+
+
+def last_variant() -> str:
+    """The kernel instance the calling thread's latest matmul / attention call selected."""
+    return load().exo_last_variant().decode("utf-8", "replace")

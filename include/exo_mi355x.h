@@ -27,6 +27,12 @@ typedef void* exo_stream_t;
 
 int exo_abi_version(void);
 const char* exo_last_error(void);
+/* Diagnostic, no reference counterpart: the kernel instance and launch shape that the
+ * calling thread's latest exo_qmv* / exo_qmm* / exo_gather_* / exo_attn_decode* /
+ * exo_sdpa_* call selected, as text (e.g. "qmm wide ring4 pair bits=4 ..."); thread-local,
+ * empty before the first such call.  Tests use it to assert that a shape reached the
+ * instance it targets. */
+const char* exo_last_variant(void);
 /* 1 if dequantised bf16 weights are formed as bf16(bf16(s*q)+b), 0 if bf16(fma(s,q,b)). */
 int exo_dequant_two_roundings(void);
 
