@@ -857,13 +857,13 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     // us); on short ranges its start-up costs more than it returns (14336x4096: 20.5 -> 21.4)
     const bool ring = p.kc >= kWideRingMinK;
     if (M <= 32 && ring)
-      qmm_kernel<BITS, 1, false, true, false, true, true><<<g, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 1, false, true, false, true, true>", BITS), qmm_kernel<BITS, 1, false, true, false, true, true><<<g, 256, 0, st>>>(p);
     else if (M <= 32)
-      qmm_kernel<BITS, 1, false, true, false, true><<<g, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 1, false, true, false, true>", BITS), qmm_kernel<BITS, 1, false, true, false, true><<<g, 256, 0, st>>>(p);
     else if (ring)
-      qmm_kernel<BITS, 2, false, true, false, true, true><<<g, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true, false, true, true>", BITS), qmm_kernel<BITS, 2, false, true, false, true, true><<<g, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 2, false, true, false, true><<<g, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true, false, true>", BITS), qmm_kernel<BITS, 2, false, true, false, true><<<g, 256, 0, st>>>(p);
     const int64_t total = (int64_t)M * N;
     const int vec_ok = (((uintptr_t)p.y | (uintptr_t)p.residual) & 7) == 0;
     qmm_reduce_kernel<<<dim3(exo_ceil_div(exo_ceil_div(total, 4), 256)), 256, 0, st>>>(
@@ -887,14 +887,14 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     if (kWideSplit && sb4 && (BITS == 4 || kRing8) && p.ksplit > 1 && M > 64 && p.kc >= kWideSplitMinK &&
         p.kc % 512 == 0 && p.K % p.kc == 0 &&
         (int64_t)exo_ceil_div(N, 256) * exo_ceil_div(M, 128) * p.ksplit >= kWideSplitMinWgs)
-      qmm_kernel<BITS, 4, false, true, false, true, false, true>
+      exo_note_variant("qmm_kernel<%d, 4, false, true, false, true, false, true>", BITS), qmm_kernel<BITS, 4, false, true, false, true, false, true>
           <<<dim3(exo_ceil_div(N, 256), exo_ceil_div(M, 128), p.ksplit), 512, 0, st>>>(p);
     else if (sb4 && p.kc >= kDeepMinK)
-      qmm_kernel<BITS, 2, false, true, false, false, true><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true, false, false, true>", BITS), qmm_kernel<BITS, 2, false, true, false, false, true><<<g2, 256, 0, st>>>(p);
     else if (sb4)
-      qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true>", BITS), qmm_kernel<BITS, 2, false, true><<<g2, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 2, false, false><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, false>", BITS), qmm_kernel<BITS, 2, false, false><<<g2, 256, 0, st>>>(p);
     if (p.ksplit > 1) {
       const int64_t total = (int64_t)M * N;
       const int vec_ok = (((uintptr_t)p.y | (uintptr_t)p.residual) & 7) == 0;
@@ -914,18 +914,18 @@ void launch_qmm(const QmmParams& p, hipStream_t st) {
     // such tiles it wins on some shapes and loses on others, so 256 it is)
     const dim3 gw(exo_ceil_div(N, 256), exo_ceil_div(M, 128));
     if (kWideHalves && sb4 && (BITS == 4 || kRing8) && (int64_t)gw.x * gw.y <= kWideHalvesMaxTiles && p.K % 512 == 0 && p.K >= 1024)
-      qmm_kernel<BITS, 4, false, true, false, true, false, true><<<gw, 512, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, false, true, false, true>", BITS), qmm_kernel<BITS, 4, false, true, false, true, false, true><<<gw, 512, 0, st>>>(p);
     else if (sb4 && tall <= 256 && p.K % 512 == 0 && p.K >= 1024)
-      qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, false, false, false, true>", BITS), qmm_kernel<BITS, 4, false, true, false, false, false, true><<<g4, 512, 0, st>>>(p);
     // more wide tiles than CUs: the wide tile with the ring, four waves (6144x4096 under 2046
     // rows 144 -> 126 us, 4096x14336 under 4094 rows 523 -> 472, 8192x8192 under 2046 rows
     // 292 -> 270)
     else if (sb4 && (BITS == 4 || kRing8) && (int64_t)gw.x * gw.y >= kWideRingMinTiles && weights_stay_cached(N, p.K, BITS))
-      qmm_kernel<BITS, 4, false, true, false, true><<<gw, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, false, true>", BITS), qmm_kernel<BITS, 4, false, true, false, true><<<gw, 256, 0, st>>>(p);
     else if (sb4)
-      qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true>", BITS), qmm_kernel<BITS, 4, false, true><<<g4, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 4, false, false><<<g4, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, false>", BITS), qmm_kernel<BITS, 4, false, false><<<g4, 256, 0, st>>>(p);
   }
 }
 
@@ -940,25 +940,25 @@ void launch_grouped(const QmmParams& p, int row_tiles, hipStream_t st) {
   if (sb4 && kGroupedWide) {
     const dim3 grid(exo_ceil_div(p.N, pair ? 128 : 256), row_tiles);
     if (pair)
-      qmm_kernel<BITS, 4, true, true, true, true><<<grid, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, true, true, true, true>", BITS), qmm_kernel<BITS, 4, true, true, true, true><<<grid, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 4, true, true, false, true><<<grid, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, true, true, false, true>", BITS), qmm_kernel<BITS, 4, true, true, false, true><<<grid, 256, 0, st>>>(p);
     return;
   }
   const dim3 grid(exo_ceil_div(p.N, pair ? 64 : 128), row_tiles);
   if (pair) {
     if (sb4 && p.K >= kDeepMinK)
-      qmm_kernel<BITS, 2, true, true, true, false, true><<<grid, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, true, true, true, false, true>", BITS), qmm_kernel<BITS, 2, true, true, true, false, true><<<grid, 256, 0, st>>>(p);
     else if (sb4)
-      qmm_kernel<BITS, 2, true, true, true><<<grid, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, true, true, true>", BITS), qmm_kernel<BITS, 2, true, true, true><<<grid, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 2, true, false, true><<<grid, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, true, false, true>", BITS), qmm_kernel<BITS, 2, true, false, true><<<grid, 256, 0, st>>>(p);
   } else if (sb4 && p.K >= kDeepMinK) {
-    qmm_kernel<BITS, 2, true, true, false, false, true><<<grid, 256, 0, st>>>(p);
+    exo_note_variant("qmm_kernel<%d, 2, true, true, false, false, true>", BITS), qmm_kernel<BITS, 2, true, true, false, false, true><<<grid, 256, 0, st>>>(p);
   } else if (sb4) {
-    qmm_kernel<BITS, 2, true, true><<<grid, 256, 0, st>>>(p);
+    exo_note_variant("qmm_kernel<%d, 2, true, true>", BITS), qmm_kernel<BITS, 2, true, true><<<grid, 256, 0, st>>>(p);
   } else {
-    qmm_kernel<BITS, 2, true, false><<<grid, 256, 0, st>>>(p);
+    exo_note_variant("qmm_kernel<%d, 2, true, false>", BITS), qmm_kernel<BITS, 2, true, false><<<grid, 256, 0, st>>>(p);
   }
 }
 
@@ -1165,11 +1165,11 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
   const bool small_grid = (int64_t)g4.x * g4.y <= 128;
   if (p.M <= 128 || small_grid) {
     if (sb4 && p.kc >= kDeepMinK)
-      qmm_kernel<BITS, 2, false, true, true, false, true><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true, true, false, true>", BITS), qmm_kernel<BITS, 2, false, true, true, false, true><<<g2, 256, 0, st>>>(p);
     else if (sb4)
-      qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, true, true>", BITS), qmm_kernel<BITS, 2, false, true, true><<<g2, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 2, false, false, true><<<g2, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 2, false, false, true>", BITS), qmm_kernel<BITS, 2, false, false, true><<<g2, 256, 0, st>>>(p);
     if (p.ksplit > 1) {
       const int64_t total = (int64_t)p.M * p.N, one = (int64_t)part_stride(p.M, p.N);
       qmm_reduce_swiglu_kernel<<<dim3(exo_ceil_div(exo_ceil_div(total, 4), 256)), 256, 0, st>>>(
@@ -1178,13 +1178,13 @@ void launch_pair(const QmmParams& p, hipStream_t st) {
   } else {
     // (up to one tall tile per CU: eight waves per tile, as in launch_qmm)
     if (sb4 && (int64_t)g4.x * g4.y <= 256 && p.K % 512 == 0 && p.K >= 1024)
-      qmm_kernel<BITS, 4, false, true, true, false, false, true><<<g4, 512, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, true, false, false, true>", BITS), qmm_kernel<BITS, 4, false, true, true, false, false, true><<<g4, 512, 0, st>>>(p);
     else if (sb4 && p.M >= kPairWideMinM && weights_stay_cached(2 * (int64_t)p.N, p.K, BITS))
-      qmm_kernel<BITS, 4, false, true, true, true><<<dim3(exo_ceil_div(p.N, 128), exo_ceil_div(p.M, 128)), 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, true, true>", BITS), qmm_kernel<BITS, 4, false, true, true, true><<<dim3(exo_ceil_div(p.N, 128), exo_ceil_div(p.M, 128)), 256, 0, st>>>(p);
     else if (sb4)
-      qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, true, true>", BITS), qmm_kernel<BITS, 4, false, true, true><<<g4, 256, 0, st>>>(p);
     else
-      qmm_kernel<BITS, 4, false, false, true><<<g4, 256, 0, st>>>(p);
+      exo_note_variant("qmm_kernel<%d, 4, false, false, true>", BITS), qmm_kernel<BITS, 4, false, false, true><<<g4, 256, 0, st>>>(p);
   }
 }
 

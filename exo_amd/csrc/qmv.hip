@@ -1150,6 +1150,7 @@ int launch_ksplit(const QmvParams& p, hipStream_t st) {
   int grid = 256 * per_cu;
   const int max_grid = (p.N + 3) / 4;
   if (grid > max_grid) grid = max_grid;
+  exo_note_variant("qmv_ksplit<%d,%d> grid=%d", BITS, NW, grid);
   qmv_ksplit_kernel<BITS, NW><<<dim3(grid), dim3(64 * NW), 0, st>>>(p);
   return EXO_OK;
 }
@@ -1396,6 +1397,8 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
     }
   }
   if (grid < 1) grid = 1;
+  exo_note_variant("qmv_rows<%d,%d,%d,%d,%s> grid=%dx%d", BITS, MT, NMAT, ITERS, route ? "true" : "false",
+                   grid, pairs);
   kern<<<dim3(grid, pairs), dim3(kThreads), kRowsXR<MT, ITERS, NMAT> ? 0 : pl.lds, st>>>(p);
   return EXO_OK;
 }
@@ -1508,6 +1511,8 @@ int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
     }
     attr_done = true;
   }
+  exo_note_variant("qmv_generic<%d,%d,%d,%s> grid=%dx%d", BITS, MT, NMAT, route ? "true" : "false",
+                   pl.grid, pairs);
   kern<<<dim3(pl.grid, pairs), dim3(kThreads), pl.lds, st>>>(p);
   return EXO_OK;
 }
@@ -1945,6 +1950,7 @@ extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, cons
   const int rw = exo_ceil_div(N, 2 * rpwi) >= 512 ? 2 : 1;
   const dim3 grid(exo_ceil_div(N, rw * rpwi), T);
   const size_t lds = (size_t)topk * ((size_t)p.wpr * 16 + (size_t)(p.wpr / 4) * 8);
+  exo_note_variant("moe_down_combine<%d,%d> grid=%dx%d", bits, rw, (int)grid.x, (int)grid.y);
   if (bits == 4) {
     if (rw == 2)
       moe_down_combine_kernel<4, 2><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);

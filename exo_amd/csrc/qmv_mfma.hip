@@ -506,6 +506,8 @@ int launch(const MfmaParams& p, size_t lds, hipStream_t st) {
     const int per = (NBq + gx - 1) / gx;
     gx = (NBq + per - 1) / per;
   }
+  exo_note_variant("qmv_mfma<%d,%d,%d,%d,%d,%s> grid=%dx%d", BITS, MR, KW, NG, SPS, SBLK ? "true" : "false",
+                   gx, p.ksplit);
   kern<<<dim3(gx, p.ksplit), dim3(64 * KW * NG), lds, st>>>(p);
   return EXO_OK;
 }

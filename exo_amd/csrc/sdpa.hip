@@ -753,6 +753,7 @@ int launch_sdpa(const SdpaParams& p0, hipStream_t st) {
     G /= p.hgroups;
   }
   dim3 grid(MODE != 0 ? p.splits : p.T, p.Hkv * p.hgroups, p.B);
+  exo_note_variant("sdpa_kernel<%d,%d,%d> grid=%dx%dx%d", D, G, MODE, (int)grid.x, (int)grid.y, (int)grid.z);
   switch (G) {
     case 1: sdpa_kernel<D, 1, MODE><<<grid, kThreads, 0, st>>>(p); break;
     case 2: sdpa_kernel<D, 2, MODE><<<grid, kThreads, 0, st>>>(p); break;
@@ -878,6 +879,7 @@ extern "C" int exo_sdpa_decode_static(const uint16_t* q, const uint16_t* k_cache
   const int n_cnt = B * Hq;
   int* cnt = reinterpret_cast<int*>(ws);
   zero_ints_kernel<<<dim3(exo_ceil_div(n_cnt, 256)), 256, 0, (hipStream_t)stream>>>(cnt, n_cnt);
+  EXO_CHECK_LAUNCH("exo_sdpa_decode_static");
   return exo_sdpa_decode(q, k_cache, v_cache, pos, out, ws, scale, B, Hq, Hkv, D, S_max, stream);
 }
 
@@ -957,6 +959,7 @@ extern "C" int exo_attn_decode_hint(const uint16_t* qkv, uint16_t* k_cache, uint
     p.splits = sp;
     p.hgroups = 1;
     const dim3 grid(p.splits, Hkv, B);
+    exo_note_variant("sdpa_decode_mfma<%d> grid=%dx%dx%d", G, (int)grid.x, (int)grid.y, (int)grid.z);
     if (G == 4)
       sdpa_decode_mfma_kernel<4><<<grid, kThreads, 0, (hipStream_t)stream>>>(p);
     else if (G == 8)

@@ -327,6 +327,8 @@ int exo_sdpa_prefill_mfma(const bf16_t* q, const bf16_t* k_cache, const bf16_t* 
   static bool done[4] = {false, false, false, false};
   const int lds = (D == 64 ? fa_lds_bytes<64>() : fa_lds_bytes<128>()) * (split ? 2 : 1);
   int rc;
+  exo_note_variant("fa_prefill<%d,%s> grid=%dx%dx%d", D, split ? "true" : "false", (int)grid.x, (int)grid.y,
+                   (int)grid.z);
   if (D == 64 && !split) {
     if ((rc = raise(reinterpret_cast<const void*>(fa_prefill_kernel<64, false>), lds, &done[0]))) return rc;
     fa_prefill_kernel<64, false><<<grid, 256, lds, stream>>>(p);
