@@ -800,6 +800,9 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 
 // The single-round kernel: EXO_QMV_ONCE_GRID workgroups (one per CU) of up to
 // EXO_QMV_ONCE_MAXW waves, each wave at most RW rows and at most 16 KiB of codes.
+// (off: in the whole decode step the single-round kernel loses - Llama-3.1-8B 1.533 against
+// 1.501 ms per token on one box, repeatedly - although a graph of its launches alone is level
+// or ahead of the row kernel's: 16.0 against 16.5 us for the gate/up pair, 6.0 against 6.4)
 #ifndef EXO_QMV_ONCE
 #define EXO_QMV_ONCE 0
 #endif
@@ -812,8 +815,11 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 #ifndef EXO_QMV_ONCE_MINRW
 #define EXO_QMV_ONCE_MINRW 1
 #endif
+// rows requested before the first product (0: all).  Measured on the 14336x4096 gate/up pair
+// with the fused norm (4 rows per wave): all four 20.4 us, two 17.3, one 16.0 - the more
+// loads a wave queues in front of the ones it needs first, the later those arrive.
 #ifndef EXO_QMV_ONCE_AHEAD
-#define EXO_QMV_ONCE_AHEAD 0  // rows requested before the first product (0: all)
+#define EXO_QMV_ONCE_AHEAD 1
 #endif
 #ifndef EXO_QMV_ONCE_XBARRIER
 #define EXO_QMV_ONCE_XBARRIER 1
@@ -1396,6 +1402,13 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
         }
     }
   }
+#ifdef EXO_QMV_GRID_OVERRIDE  // tuning builds: {N, grid} pairs for launches of one activation row
+  if (single) {
+    static const int ov[][2] = {EXO_QMV_GRID_OVERRIDE};
+    for (auto& o : ov)
+      if (o[0] == p.N * (NMAT == 2 ? -1 : 1) && o[1] > 0) grid = o[1];
+  }
+#endif
   if (grid < 1) grid = 1;
   exo_note_variant("qmv_rows<%d,%d,%d,%d,%s> grid=%dx%d", BITS, MT, NMAT, ITERS, route ? "true" : "false",
                    grid, pairs);
@@ -1467,7 +1480,11 @@ int launch_once(const QmvParams& p, int rw, int nw, hipStream_t st) {
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   if constexpr (MT == 1) {
-   if (p.M == 1 && pairs == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.idx && !p.each_row && !p.route) {
+   // (launches with the fused RMSNorm: the norm and the staging happen once per CU instead of
+   // once per short-lived workgroup - the gate/up pair 16.5 -> 16.0 us, 6144x4096 6.46 -> 6.01;
+   // without a norm the row kernel below is level or ahead)
+   if (p.M == 1 && pairs == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.idx && !p.each_row && !p.route &&
+       p.norm_w) {
     int rw, nw;
     switch (pl.iters) {
       case 1: if (once_shape<NMAT, 1>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 1>(p, rw, nw, st); break;

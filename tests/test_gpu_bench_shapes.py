@@ -286,8 +286,13 @@ def test_decode_launches_reach_their_instances(device):
     nw = t_bf16(affine.bf16_round(rand_bf16((H,), seed=2) * 0.1 + 1.0), device)
     g, u = _packed(I, H, bits, 1, device), _packed(I, H, bits, 2, device)
     ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
-    assert native.last_variant().startswith("qmv_rows<4,1,2,2,false>"), native.last_variant()
+    assert native.last_variant() == "qmv_once<4,2,2,4> grid=256 waves=14", native.last_variant()
     ops.quantized_matmul(x, _packed(6144, H, bits, 3, device), norm_weight=nw, eps=1e-5)
+    assert native.last_variant() == "qmv_once<4,1,2,2> grid=256 waves=12", native.last_variant()
+    xa = t_bf16(rand_bf16((1, H), seed=6), device)
+    ops.quantized_matmul(xa, _packed(H, H, bits, 5, device), residual=x)
+    assert native.last_variant().startswith("qmv_rows<4,1,1,2,false>"), native.last_variant()
+    ops.quantized_matmul(x, _packed(128256, H, bits, 6, device), norm_weight=nw, eps=1e-5)
     assert native.last_variant().startswith("qmv_rows<4,1,1,2,false>"), native.last_variant()
     xi = t_bf16(rand_bf16((1, I), seed=3), device)
     ops.quantized_matmul(xi, _packed(H, I, bits, 4, device))
@@ -301,7 +306,7 @@ def test_decode_launches_reach_their_instances(device):
     # decode attention: one sequence of 32 / 8 heads on the scalar kernel, eight on the matrix cores
     D, Hq, Hkv, S = 128, 32, 8, 2304
     inv = torch.from_numpy(O.rope_inv_freq(D, 5e5, None)).to(device)
-    for B, want in ((1, "sdpa_kernel<128,1,2>"), (8, "sdpa_decode_mfma<4>")):
+    for B, want in ((1, "sdpa_tiles<128,1,true> grid=8x32x1"), (8, "sdpa_decode_mfma<4>")):
         qkv = torch.randn(B, (Hq + 2 * Hkv) * D, device=device).bfloat16()
         kc = torch.randn(B, Hkv, S, D, device=device).bfloat16()
         vc = torch.randn(B, Hkv, S, D, device=device).bfloat16()
