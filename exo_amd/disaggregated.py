@@ -19,7 +19,6 @@ as msgspec's decoders do.
 from __future__ import annotations
 
 import socket
-import socketserver
 import threading
 import time
 from collections import defaultdict
@@ -455,59 +454,104 @@ def ingest_into_cache(result: PrefillResult, cache: ShardKVCache, *, row: int = 
 
 ResolveHandler = Callable[[PrefillRequest, BinaryIO], bool]
 
+_SEND_BUFFER_BYTES = 4 << 20  # what the reference asks of the socket (server.py:55-56)
 
-def _send_error(wfile: BinaryIO, code: int, message: str) -> None:
-    try:
-        write_header(wfile, Header(num_layers=0, dtype="float32"))
-        write_error(wfile, code=code, message=message)
-    except Exception:
+
+class _SocketOut:
+    """Unbuffered binary writer over a connected socket: every write goes out whole and at
+    once, so the peer sees each frame as soon as the engine has produced it."""
+
+    def __init__(self, conn: socket.socket) -> None:
+        self._conn = conn
+
+    def write(self, data) -> int:
+        self._conn.sendall(data)
+        return len(data)
+
+    def flush(self) -> None:
         pass
 
 
-class _PrefillHandler(socketserver.StreamRequestHandler):
-    def setup(self) -> None:
-        super().setup()
-        self.request.setsockopt(socket.IPPROTO_TCP, socket.TCP_NODELAY, 1)
-        self.request.setsockopt(socket.SOL_SOCKET, socket.SO_SNDBUF, 4 * 1024 * 1024)
+class PrefillServer:
+    """TCP front of the prefill service: the interface the reference's runner wires up
+    (``PrefillServer(resolve, host, port)``, ``stop()``; src/exo/worker/disaggregated/
+    server.py:88-110), on a plain accept loop.
 
-    def handle(self) -> None:
-        try:
-            job = read_request(self.rfile)
-        except ConnectionError:
-            return
-        except (ProtocolError, ValueError) as exc:
-            _send_error(self.wfile, 400, f"Bad request: {exc}")
-            return
-        try:
-            picked_up = self.server.resolve(job, self.wfile)  # type: ignore[attr-defined]
-        except Exception as e:
-            _send_error(self.wfile, 500, str(e))
-            return
-        if not picked_up:
-            _send_error(self.wfile, 503, f"Prefill not picked up for request_id={job.request_id!r}")
-
-
-class PrefillServer(socketserver.ThreadingTCPServer):
-    """TCP front of the prefill service (src/exo/worker/disaggregated/server.py:88-110).
-    ``resolve(request, wfile)`` is called on a connection thread; an engine that is
-    single-threaded hands the request to its own thread there and waits."""
-
-    allow_reuse_address = True
-    daemon_threads = True
+    One thread accepts connections; every connection gets a short-lived thread that reads ONE
+    request frame, hands it to ``resolve(request, wfile)`` and closes.  ``resolve`` writes the
+    reply stream itself and returns whether it took the request; an engine that is
+    single-threaded queues the request for its own thread there and waits.  Status replies
+    are a zero-layer header followed by an error frame, as the reference's clients expect:
+    400 for an undecodable request, 500 when ``resolve`` raises, 503 when it declines."""
 
     def __init__(self, resolve: ResolveHandler, host: str, port: int) -> None:
-        super().__init__((host, port), _PrefillHandler)
         self.resolve = resolve
-        self._thread: threading.Thread | None = threading.Thread(
-            target=self.serve_forever, name="prefill-server", daemon=True)
-        self._thread.start()
+        self._sock = socket.create_server((host, port), reuse_port=False)
+        self._sock.settimeout(0.2)  # the accept loop looks at the stop flag between waits
+        self.server_address = self._sock.getsockname()
+        self._stopping = threading.Event()
+        self._acceptor: threading.Thread | None = threading.Thread(
+            target=self._accept_loop, name="prefill-server", daemon=True)
+        self._acceptor.start()
+
+    # -- life cycle
+    def _accept_loop(self) -> None:
+        while not self._stopping.is_set():
+            try:
+                conn, _peer = self._sock.accept()
+            except socket.timeout:
+                continue
+            except OSError:
+                break  # the listening socket was closed
+            threading.Thread(target=self._serve_connection, args=(conn,), name="prefill-conn",
+                             daemon=True).start()
 
     def stop(self) -> None:
-        self.shutdown()
-        self.server_close()
-        if self._thread is not None:
-            self._thread.join(timeout=5)
-            self._thread = None
+        self._stopping.set()
+        try:
+            self._sock.close()
+        finally:
+            if self._acceptor is not None:
+                self._acceptor.join(timeout=5)
+                self._acceptor = None
+
+    # -- one connection
+    @staticmethod
+    def _reply_status(wfile: BinaryIO, code: int, message: str) -> None:
+        """Best effort: the peer may already be gone."""
+        try:
+            write_header(wfile, Header(num_layers=0, dtype="float32"))
+            write_error(wfile, code=code, message=message)
+        except (OSError, ValueError):
+            pass
+
+    def _serve_connection(self, conn: socket.socket) -> None:
+        with conn:
+            conn.settimeout(None)
+            conn.setsockopt(socket.IPPROTO_TCP, socket.TCP_NODELAY, 1)
+            conn.setsockopt(socket.SOL_SOCKET, socket.SO_SNDBUF, _SEND_BUFFER_BYTES)
+            rfile, wfile = conn.makefile("rb"), _SocketOut(conn)
+            try:
+                status: tuple[int, str] | None = None
+                try:
+                    request = read_request(rfile)
+                except ConnectionError:
+                    return  # closed without sending a request
+                except (ProtocolError, ValueError) as exc:
+                    request, status = None, (400, f"Bad request: {exc}")
+                if request is not None:
+                    try:
+                        if not self.resolve(request, wfile):
+                            status = (503, f"Prefill not picked up for request_id={request.request_id!r}")
+                    except Exception as exc:  # the engine's failure becomes the peer's error frame
+                        status = (500, str(exc))
+                if status is not None:
+                    self._reply_status(wfile, *status)
+            finally:
+                try:
+                    rfile.close()
+                except OSError:
+                    pass
 
 
 def remote_prefill(prompt_tokens, cache: ShardKVCache, on_prefill_progress=None, *, endpoint: str,
