@@ -41,7 +41,7 @@ constexpr int kBlocks = 64;      // slices per row
 constexpr int kMaxSlice = 4096;  // elements per slice (two 8-element chunks per thread)
 constexpr int kMaxEdits = EXO_SAMPLER_MAX_CONTEXT + EXO_SAMPLER_MAX_BANNED;
 constexpr int kTop = EXO_SAMPLER_TOP_LOGPROBS;
-constexpr int kMaxCand = 320;  // top-20 candidates: up to 300 ties at the 20th place
+constexpr int kMaxCand = 32;    // values strictly above the 20th largest: 19 at most
 constexpr int kBuckets = 512;  // key >> 7: sign and exponent
 constexpr int kFine = 128;     // key & 127: mantissa, in value order inside a bucket
 constexpr int kTargets = 3;    // 0: k-th largest (top-k), 1: nucleus edge (top-p), 2: 20th largest
@@ -60,7 +60,12 @@ struct RowWs {
   unsigned long long above_m[kTargets];
   int edit_idx[kMaxEdits];
   float edit_val[kMaxEdits];
-  unsigned long long cand[kMaxCand];  // key << 32 | index
+  unsigned long long cand[kMaxCand];  // key << 32 | index, values strictly above the 20th largest
+  // tokens whose value EQUALS the 20th largest, per slice: the first kTop of them in
+  // vocabulary order (a flat row has thousands; which of them make the list must not depend
+  // on the order in which workgroups arrive)
+  int tie_n[kBlocks];
+  int tie_idx[kBlocks][kTop];
 };
 constexpr size_t kRowWsBytes = (sizeof(RowWs) + 255) / 256 * 256;
 
@@ -618,18 +623,51 @@ __global__ __launch_bounds__(256) void sample_weights_kernel(
   int i0[2];
   load_share(logits + (size_t)row * V, g, ed, xv, i0);
   if (want_top) {
+    // strictly above the 20th largest value: at most 19 tokens in the whole row, any order
+    // (the select launch ranks them); equal to it: this slice's first kTop in vocabulary
+    // order, by a scan over the threads (chunk 0 of every thread precedes chunk 1 of any)
+    __shared__ int s_tiew[4];
+    int base = 0;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < 2; ++u) {
+      int mine = 0;
 #pragma unroll
       for (int k = 0; k < 8; ++k)
         if (i0[u] + k < g.hi) {
           const int key = key_of(xv[8 * u + k]);
-          if (key >= kt) {
+          if (key > kt) {
             const int slot = atomicAdd(&w->cand_n, 1);
             if (slot < kMaxCand)
               w->cand[slot] = ((unsigned long long)key << 32) | (unsigned int)(i0[u] + k);
+          } else if (key == kt) {
+            ++mine;
           }
         }
+      int inc = mine;
+      const int ln = threadIdx.x & 63, wv = threadIdx.x >> 6;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(inc, o, 64);
+        if (ln >= o) inc += up;
+      }
+      if (ln == 63) s_tiew[wv] = inc;
+      __syncthreads();
+      int before = base;
+      for (int q = 0; q < wv; ++q) before += s_tiew[q];
+      const int round_total = s_tiew[0] + s_tiew[1] + s_tiew[2] + s_tiew[3];
+      int at = before + inc - mine;  // ties of this slice in front of this thread's chunk
+      if (mine > 0 && at < kTop) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (i0[u] + k < g.hi && key_of(xv[8 * u + k]) == kt) {
+            if (at < kTop) w->tie_idx[blockIdx.x][at] = i0[u] + k;
+            ++at;
+          }
+      }
+      __syncthreads();
+      base += round_total;
+    }
+    if (threadIdx.x == 0) w->tie_n[blockIdx.x] = min(base, kTop);
   }
   if (!sampling) return;
   const float thr = keep_threshold(p, table_thr, mx);
@@ -795,10 +833,16 @@ __global__ __launch_bounds__(256) void sample_select_kernel(
     }
     tok = s_tok;
     x_tok = s_x;
+    if (tok < 0 || tok >= V) {  // no token was kept (min_p above 1, logits that are not numbers)
+      tok = mi;
+      x_tok = mx;
+    }
   }
+  tok = min(max(tok, 0), V - 1);
   if (want_top && top_idx && top_val) {
-    // rank the candidates: higher key first, lower index first among equals
-    const int n = min(w->cand_n, kMaxCand);
+    // the tokens strictly above the 20th largest value, ranked: higher key first, lower index
+    // first among equals; then the tokens equal to it, lowest ids first (slices in order)
+    const int n = min(w->cand_n, kTop - 1);
     for (int c = tid; c < n; c += 256) {
       const unsigned long long me = w->cand[c];
       const unsigned int mk = (unsigned int)(me >> 32), mi2 = (unsigned int)me;
@@ -808,14 +852,21 @@ __global__ __launch_bounds__(256) void sample_select_kernel(
         const unsigned int ok = (unsigned int)(ot >> 32), oi = (unsigned int)ot;
         rank += (ok > mk || (ok == mk && oi < mi2)) ? 1 : 0;
       }
-      if (rank < kTop) {
-        top_idx[(size_t)row * kTop + rank] = (int)mi2;
-        top_val[(size_t)row * kTop + rank] = value_of((int)mk) - lse;
-      }
+      top_idx[(size_t)row * kTop + rank] = (int)mi2;
+      top_val[(size_t)row * kTop + rank] = value_of((int)mk) - lse;
     }
-    for (int c = n + tid; c < kTop; c += 256) {  // vocabularies of fewer than 20 tokens
-      top_idx[(size_t)row * kTop + c] = -1;
-      top_val[(size_t)row * kTop + c] = -INFINITY;
+    if (tid == 0) {
+      int at = n;
+      const float tv = value_of(w->key_top) - lse;
+      for (int b = 0; b < kBlocks && at < kTop; ++b)
+        for (int j = 0; j < w->tie_n[b] && at < kTop; ++j, ++at) {
+          top_idx[(size_t)row * kTop + at] = w->tie_idx[b][j];
+          top_val[(size_t)row * kTop + at] = tv;
+        }
+      for (; at < kTop; ++at) {  // vocabularies of fewer than 20 tokens
+        top_idx[(size_t)row * kTop + at] = -1;
+        top_val[(size_t)row * kTop + at] = -INFINITY;
+      }
     }
   }
   if (tid == 0) {
@@ -859,6 +910,7 @@ extern "C" int exo_sample(const uint16_t* logits, const exo_sampler_params* para
   const bool edits = mode & EXO_SAMPLE_EDITS, want_top = mode & EXO_SAMPLE_TOP;
   EXO_REQUIRE(!edits || hist_cap == 0 || (history && hist_len),
               "exo_sample: the penalty processors need the history ring");
+  EXO_REQUIRE(!history || hist_cap > 0, "exo_sample: a history ring of zero entries (hist_cap=0)");
   EXO_REQUIRE(!want_top || (top_idx && top_val), "exo_sample: top-logprob outputs missing");
   EXO_REQUIRE(!(mode & EXO_SAMPLE_DRAW) || draws, "exo_sample: draw counters missing");
   if (rows == 0) return EXO_OK;

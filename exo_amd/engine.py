@@ -183,7 +183,7 @@ class ShardBatchGenerator:
             max_tokens = self.max_seq - len(toks) - 2
             if max_tokens <= 0:
                 raise ValueError(f"prompt of {len(toks)} tokens exceeds the cache ({self.max_seq})")
-        settings = SamplerSettings.from_task(task_params, self._eos())
+        settings = SamplerSettings.from_task(task_params, self._eos(), zero_seed_is_default=False)
         row = len(self.rows)
         # prefix cache lookup (batch_generate.py:164-181): bench requests opt in
         use_prefix = self.kv_prefix_cache is not None and (

@@ -59,8 +59,12 @@ class SamplerSettings:
     seed: int = 42
 
     @staticmethod
-    def from_task(task, eos_token_ids=()) -> "SamplerSettings":
-        """generate.py:599-619: penalties from the task, EOS banned in bench mode."""
+    def from_task(task, eos_token_ids=(), zero_seed_is_default=True) -> "SamplerSettings":
+        """generate.py:599-619: penalties from the task, EOS banned in bench mode.
+
+        The single-request generator reads the seed as `task.seed or 42` (generate.py:547: seed 0
+        becomes 42), the batch generator as `seed if seed is not None else 42`
+        (batch_generate.py:182: seed 0 stays 0); `zero_seed_is_default` picks between them."""
         rp = task.repetition_penalty
         if rp is not None and rp < 0:
             raise ValueError("repetition_penalty must be a non-negative float")
@@ -74,7 +78,8 @@ class SamplerSettings:
             if task.repetition_context_size is not None else 20,
             presence_penalty=task.presence_penalty, frequency_penalty=task.frequency_penalty,
             banned=list(eos_token_ids or []) if task.bench else [],
-            seed=task.seed or 42)
+            seed=(task.seed or 42) if zero_seed_is_default
+            else (task.seed if task.seed is not None else 42))
 
     # ---- what the row needs
     @property

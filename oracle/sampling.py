@@ -24,6 +24,13 @@ commonly stated ones and are "parity unpinned" against mlx_lm itself:
     (itself included) exceeds 1 - top_p; min-p keeps i iff p_i >= min_p * p_max; top-k keeps
     the k most likely (here: every token tied with the k-th as well); the filters compose to
     one value threshold; the draw is from softmax(logprobs / temp) over the kept tokens.
+Which tokens the processors see: here, at the step that samples token k, the context is the
+last two prompt tokens followed by tokens 0..k-1 - the order of mlx_lm's sequential generator
+(and of src/exo/worker/engines/mlx/generator/generate.py).  The reference's batched step
+lags by one: it calls the processors with ``self.tokens[e]`` (opt_batch_gen.py:75) and appends
+the token being fed only afterwards (:127), so its step k does not yet see token k-1.  The
+device path follows the sequential order in both engines, on purpose: one definition for both,
+and a token repeated at once is penalised at once.
 The random stream is this build's own (Philox-4x32-10 keyed by the request seed, one block
 per draw): MLX's generator cannot be reproduced without MLX.  What IS pinned: Philox
 against the published known-answer vectors, the filters against independent torch

@@ -286,9 +286,9 @@ def test_decode_launches_reach_their_instances(device):
     nw = t_bf16(affine.bf16_round(rand_bf16((H,), seed=2) * 0.1 + 1.0), device)
     g, u = _packed(I, H, bits, 1, device), _packed(I, H, bits, 2, device)
     ops.qmv_swiglu(x, g, u, norm_weight=nw, eps=1e-5)
-    assert native.last_variant() == "qmv_once<4,2,2,4> grid=256 waves=14", native.last_variant()
+    assert native.last_variant() == "qmv_rows<4,1,2,2,false> grid=1792x1", native.last_variant()
     ops.quantized_matmul(x, _packed(6144, H, bits, 3, device), norm_weight=nw, eps=1e-5)
-    assert native.last_variant() == "qmv_once<4,1,2,2> grid=256 waves=12", native.last_variant()
+    assert native.last_variant().startswith("qmv_rows<4,1,1,2,false>"), native.last_variant()
     xa = t_bf16(rand_bf16((1, H), seed=6), device)
     ops.quantized_matmul(xa, _packed(H, H, bits, 5, device), residual=x)
     assert native.last_variant().startswith("qmv_rows<4,1,1,2,false>"), native.last_variant()

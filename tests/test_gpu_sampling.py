@@ -155,6 +155,50 @@ def test_sample_modes_and_reuse(device):
     np.testing.assert_allclose(ds.lse.cpu().numpy()[:rows], lse.cpu().numpy(), rtol=1e-6)
 
 
+def test_top_logprobs_of_flat_and_tied_rows(device):
+    """Rows with thousands of tokens at the 20th largest value: an all-equal row (a zeroed or
+    saturated head), a row of three distinct values, a row with 12 tokens above a plateau that
+    spans several slices of the row. The lowest ids among the equals are reported, whatever
+    order the workgroups of the launch arrive in; checked on repeated launches."""
+    V, rows = 128256, 4
+    logits = np.zeros((rows, V), np.float32)
+    logits[1] = np.repeat(np.array([1.0, -2.0, 0.5], np.float32), V // 3)[:V]
+    logits[2, :] = -1.0
+    logits[2, 5000:90000] = 0.25                      # plateau over slices 2..44
+    logits[2, [7, 120000, 64000, 3, 99999, 2049, 2048, 4095, 4096, 70001, 11, 128255]] = \
+        np.array([5, 5, 4, 4, 3, 3, 3, 2, 2, 1, 1, 0.5], np.float32)
+    logits[3] = rand_bf16((1, V), seed=3, scale=2.0)[0]
+    logits[3, 100000:100040] = logits[3].max() + 1   # 40 equal maxima in one slice
+    lt = t_bf16(logits, device)
+    ds = DeviceSampler(rows, V, device)
+    sets = [SamplerSettings(temperature=0.0) for _ in range(rows)]
+    for rep in range(3):
+        for i, s in enumerate(sets):
+            ds.set_row(i, s, [])
+        ds.top_idx.fill_(-7)
+        ds.sample(lt, rows, MODE_TOP)
+        torch.cuda.synchronize()
+        _check_rows(ds, logits, sets, [[] for _ in sets], [0] * rows, want_top=True)
+    assert ds.top_idx[0].cpu().tolist() == list(range(20))
+    assert ds.top_idx[3].cpu().tolist() == list(range(100000, 100020))
+
+
+def test_sample_with_no_token_kept_falls_back_to_the_argmax(device):
+    """min_p above 1 keeps no token (the threshold lies above the maximum): the step returns the
+    arg max of the processed logits, never an id outside the vocabulary."""
+    V = 1000
+    logits = rand_bf16((2, V), seed=21, scale=2.0)
+    lt = t_bf16(logits, device)
+    ds = DeviceSampler(2, V, device)
+    ds.set_row(0, SamplerSettings(temperature=0.7, min_p=1.5), [])
+    ds.set_row(1, SamplerSettings(temperature=0.7, min_p=1.5, top_k=5, banned=[int(np.argmax(logits[1]))]), [])
+    ds.sample(lt, 2, ds.mode(2))
+    torch.cuda.synchronize()
+    x1 = logits[1].copy()
+    x1[int(np.argmax(logits[1]))] = -np.inf
+    assert ds.token[:2].cpu().tolist() == [int(np.argmax(logits[0])), int(np.argmax(x1))]
+
+
 def test_sample_draws_follow_the_distribution(device):
     """4000 draws of one row (counter 0..3999) against the exact probabilities of its kept
     tokens: a chi-square bound that a wrong weight, threshold or CDF order would break."""
@@ -196,3 +240,11 @@ def test_sample_argument_errors(device):
     assert lib.exo_sample(1, 1, None, None, None, 1, None, None, None, None, None, None, 1, 0, 1, 1000, 0, 0, None) == -1
     assert lib.exo_sample(1, 1, None, None, None, 1, None, None, None, None, None, None, 256, 1 << 30, 1, 300000, 0, 0, None) == -1
     assert b"exceeds" in lib.exo_last_error()
+    # a history ring without entries
+    lg = torch.zeros(1, 1000, dtype=torch.bfloat16, device=device)
+    assert lib.exo_sample(lg.data_ptr(), ds.params.data_ptr(), ds.history.data_ptr(),
+                          ds.hist_len.data_ptr(), ds.draws.data_ptr(), ds.token.data_ptr(),
+                          ds.logprob.data_ptr(), ds.lse.data_ptr(), None, None, None, None,
+                          ds.workspace.data_ptr(), ds.workspace.numel(), 1, 1000, 0, MODE_EDITS,
+                          None) == -1
+    assert b"hist_cap" in lib.exo_last_error()

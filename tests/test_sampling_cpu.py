@@ -131,6 +131,13 @@ def test_sampler_record_layout():
     b = SamplerSettings.from_task(TextGenerationTaskParams(model="m", temperature=0.0, bench=True), [2, 3])
     assert b.banned == [2, 3] and b.edits and not b.draws
     assert not SamplerSettings(repetition_penalty=1.2, repetition_context=1000).on_device()
+    # seed 0: 42 for the single-request generator (generate.py:547, `seed or 42`), 0 for the
+    # batch generator (batch_generate.py:182, `is not None`)
+    z = TextGenerationTaskParams(model="m", seed=0)
+    assert SamplerSettings.from_task(z).seed == 42
+    assert SamplerSettings.from_task(z, zero_seed_is_default=False).seed == 0
+    assert SamplerSettings.from_task(TextGenerationTaskParams(model="m"),
+                                     zero_seed_is_default=False).seed == 42
     assert PARAMS_DTYPE.names[-1] == "banned"
 
 
