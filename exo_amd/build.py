@@ -15,7 +15,7 @@ from pathlib import Path
 PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libexo_mi355x.so"
-SOURCES = ["quant.hip", "qmv.hip", "qmv_mfma.hip", "qmv_quad.hip", "qmm.hip", "sdpa.hip", "sdpa_prefill.hip", "elementwise.hip", "kvwire.hip", "sampling.hip"]
+SOURCES = ["quant.hip", "qmv.hip", "qmv_mfma.hip", "qmv_quad.hip", "qmv_w16.hip", "qmm.hip", "sdpa.hip", "sdpa_prefill.hip", "elementwise.hip", "kvwire.hip", "sampling.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -1669,6 +1669,11 @@ extern "C" int exo_qmv(const uint16_t* x, const uint32_t* w, const uint16_t* sca
 #ifndef EXO_QMV_QUAD_MAX_M
 #define EXO_QMV_QUAD_MAX_M 4
 #endif
+// From this many activation rows the 16x16x32 matrix-core kernel (qmv_w16.hip) takes the
+// matrices its shape rules admit, in tiles of 16 rows.
+#ifndef EXO_QMV_W16_MIN_M
+#define EXO_QMV_W16_MIN_M 5
+#endif
 
 static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float eps,
                          const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -1696,6 +1701,17 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
     rc = exo_qmv_quad_launch(x, norm_weight, eps, w, scales, biases, nullptr, nullptr, nullptr,
                              residual, y, M, N, K, bits, (hipStream_t)stream);
     if (rc) return rc;
+    EXO_CHECK_LAUNCH("exo_qmv");
+    return EXO_OK;
+  }
+  if (M >= EXO_QMV_W16_MIN_M && exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, residual != nullptr)) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int mt = (M - m0 < 16) ? (M - m0) : 16;
+      rc = exo_qmv_w16_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases, nullptr,
+                              nullptr, nullptr, residual ? residual + (size_t)m0 * N : nullptr,
+                              y + (size_t)m0 * N, mt, N, K, (hipStream_t)stream);
+      if (rc) return rc;
+    }
     EXO_CHECK_LAUNCH("exo_qmv");
     return EXO_OK;
   }
@@ -1792,6 +1808,16 @@ extern "C" int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_we
     rc = exo_qmv_quad_launch(x, norm_weight, eps, wg, sg, bg, wu, su, bu, nullptr, y, M, N, K, bits,
                              (hipStream_t)stream);
     if (rc) return rc;
+    EXO_CHECK_LAUNCH("exo_qmv_swiglu");
+    return EXO_OK;
+  }
+  if (M >= EXO_QMV_W16_MIN_M && exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, false)) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int mt = (M - m0 < 16) ? (M - m0) : 16;
+      rc = exo_qmv_w16_launch(x + (size_t)m0 * K, norm_weight, eps, wg, sg, bg, wu, su, bu, nullptr,
+                              y + (size_t)m0 * N, mt, N, K, (hipStream_t)stream);
+      if (rc) return rc;
+    }
     EXO_CHECK_LAUNCH("exo_qmv_swiglu");
     return EXO_OK;
   }

@@ -1,0 +1,446 @@
+// Fused dequant-GEMV for up to 16 activation rows on v_mfma_f32_16x16x32_bf16 (4-bit codes).
+//
+// The instruction multiplies A[16][32] by B[32][16]: lane l holds A[l%16][8*(l/16) .. +8],
+// B[8*(l/16) .. +8][l%16], and D[4*(l/16) + r][l%16] in register r.  Here A is the activations
+// (row = activation row m), B a block of 16 weight rows (column = weight row j), so a lane's
+// four results belong to ONE weight row: scale and bias of a quantisation group are one value
+// per lane.
+//  * a wave instruction loads 16 rows x 64 contiguous bytes (128 codes = two groups of a row):
+//    lane (lane/4, lane%4) takes 16-byte chunk lane%4 of row lane/4, so that the four lanes of
+//    a quad read 64 contiguous bytes.  A product wants 8 codes (one word) of row j in lane
+//    (j, kg): the words change lanes through the LDS crossbar (ds_bpermute_b32, no LDS memory)
+//    when the block is consumed - two permutes and one select per product, because the four
+//    K slots of a product must come from one group (= two chunks x four words).
+//  * a wave owns SL such 64-byte slices of every row block of its workgroup; the matching
+//    activations stay in registers in operand order for the whole launch.  The waves of a
+//    workgroup together cover K; their partial sums meet in LDS once per phase of row blocks.
+//  * codes become (128+nibble) bf16 pairs with one v_and_or_b32 each (exact).  Per group:
+//      acc += s * D + (b - 128 s) * Sx        D = sum (128+q) x,  Sx = sum x   (float32)
+//  * DEPTH row blocks of weights are in flight per wave (register buffers in rotation); every
+//    refill is issued whether or not a block is left (past the end it is out of the buffer's
+//    range and moves no data), so that the number of loads in flight at each wait is a constant.
+#include "../../include/exo_mi355x.h"
+#include "common.h"
+#include "qmv_internal.h"
+
+namespace {
+
+struct W16Params {
+  const bf16_t* x;       // [M, K]
+  const bf16_t* norm_w;  // [K] or null: fused RMSNorm of x
+  float eps;
+  const uint32_t* w[2];  // packed [N, K/8]   ([1]: the up matrix of a (gate, up) pair)
+  const bf16_t* s[2];    // [N, K/64]
+  const bf16_t* b[2];
+  const bf16_t* residual;  // [M, N] or null
+  bf16_t* y;               // [M, N]
+  int M, N, K;
+  int row_bytes;  // K / 2
+  int G;          // K / 64
+  int blocks;     // N / 16
+  int ph;         // row blocks per workgroup at most (LDS holds their partial sums)
+  int lw;         // lanes of a wave that hold results: 16 * ceil(M / 4)
+};
+
+__device__ __forceinline__ float sumsq8(const uint4& v) {
+  return bf_lo(v.x) * bf_lo(v.x) + bf_hi(v.x) * bf_hi(v.x) + bf_lo(v.y) * bf_lo(v.y) +
+         bf_hi(v.y) * bf_hi(v.y) + bf_lo(v.z) * bf_lo(v.z) + bf_hi(v.z) * bf_hi(v.z) +
+         bf_lo(v.w) * bf_lo(v.w) + bf_hi(v.w) * bf_hi(v.w);
+}
+__device__ __forceinline__ void norm8(uint4& xv, const uint4& wv, float inv) {
+  xv.x = pack_bf2(bf_lo(xv.x) * inv * bf_lo(wv.x), bf_hi(xv.x) * inv * bf_hi(wv.x));
+  xv.y = pack_bf2(bf_lo(xv.y) * inv * bf_lo(wv.y), bf_hi(xv.y) * inv * bf_hi(wv.y));
+  xv.z = pack_bf2(bf_lo(xv.z) * inv * bf_lo(wv.z), bf_hi(xv.z) * inv * bf_hi(wv.z));
+  xv.w = pack_bf2(bf_lo(xv.w) * inv * bf_lo(wv.w), bf_hi(xv.w) * inv * bf_hi(wv.w));
+}
+// the 8 activations of one packed word in the order of the unpacked nibble pairs:
+// (x0,x4),(x1,x5),(x2,x6),(x3,x7); `sum` = their sum
+__device__ __forceinline__ uint4 pair_order(const uint4& xv, float& sum) {
+  uint4 o;
+  o.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);
+  o.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);
+  o.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);
+  o.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);
+  sum = (bf_lo(o.x) + bf_hi(o.x)) + (bf_lo(o.y) + bf_hi(o.y)) + (bf_lo(o.z) + bf_hi(o.z)) +
+        (bf_lo(o.w) + bf_hi(o.w));
+  return o;
+}
+
+template <int SL>
+struct SbWord;  // (scale or bias) of the 2*SL groups of a wave's slices: SL words of two bf16
+template <>
+struct SbWord<1> {
+  uint32_t v[1];
+  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, int vo, int so) {
+    v[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, vo, so, 0);
+  }
+};
+template <>
+struct SbWord<2> {
+  uint32_t v[2];
+  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, int vo, int so) {
+    const auto t = __builtin_amdgcn_raw_buffer_load_b64(r, vo, so, 0);
+    const uint2 u = __builtin_bit_cast(uint2, t);
+    v[0] = u.x;
+    v[1] = u.y;
+  }
+};
+
+// NMAT matrices (2: the (gate, up) pair with SwiGLU), SL 64-byte slices of K per wave, DEPTH
+// row blocks in flight per wave.
+// NORM: fused RMSNorm of the activations.
+template <int NMAT, int SL, int DEPTH, bool NORM>
+__global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
+  extern __shared__ float red[];  // [ph][NMAT][nw][4][lw]
+  __shared__ float s_part[16][16];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, kg = lane >> 4;  // operand layout: weight row (or activation row), K slot
+  const int lr = lane >> 2, lc = lane & 3;  // load layout: row of the block, chunk of the slice
+
+  // contiguous, balanced range of row blocks of this workgroup
+  const int qbase = p.blocks / (int)gridDim.x, qrem = p.blocks - qbase * (int)gridDim.x;
+  const int q0 = (int)blockIdx.x * qbase + min((int)blockIdx.x, qrem);
+  const int nq = qbase + ((int)blockIdx.x < qrem ? 1 : 0);
+  if (nq <= 0) return;
+
+  struct Buf {
+    uint4 w[NMAT][SL];
+    SbWord<SL> s[NMAT], b[NMAT];
+  };
+  // buffer resources over exactly this workgroup's rows (a refill past them returns zeros)
+  __amdgpu_buffer_rsrc_t rw[NMAT], rs[NMAT], rb[NMAT];
+#pragma unroll
+  for (int a = 0; a < NMAT; ++a) {
+    rw[a] = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(reinterpret_cast<const char*>(p.w[a]) + (size_t)q0 * 16 * p.row_bytes), 0,
+        nq * 16 * p.row_bytes, 0x00020000);
+    rs[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.s[a] + (size_t)q0 * 16 * p.G), 0,
+                                              nq * 16 * p.G * 2, 0x00020000);
+    rb[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.b[a] + (size_t)q0 * 16 * p.G), 0,
+                                              nq * 16 * p.G * 2, 0x00020000);
+  }
+  const int wofs = lr * p.row_bytes + wave * (SL * 64) + lc * 16;
+  const int sofs = (j * p.G + wave * (SL * 2)) * 2;  // this lane's weight row, the wave's groups
+  // PIN (the issues in front of the loop): the loads leave in program order - weights, then
+  // scales and biases, buffer by buffer, as in the loop.  The compiler counts the loads still
+  // in flight at each wait; where the order in front of the loop differs from the order in the
+  // loop it has to assume the worse of the two and waits for a whole buffer too many.
+  auto issue_w = [&](Buf& bf, int q, bool pin) {  // q: row block of this workgroup's range (past it: zeros)
+    const int wq = q * 16 * p.row_bytes;  // uniform: scalar offset
+    if (pin) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a)
+        bf.w[a][sl] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(rw[a], wofs + sl * 64, wq, 0));
+    if (pin) __builtin_amdgcn_sched_barrier(0);
+  };
+  auto issue_sb = [&](Buf& bf, int q, bool pin) {
+    const int sq = q * 16 * p.G * 2;
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a) {
+      bf.s[a].load(rs[a], sofs, sq);
+      bf.b[a].load(rb[a], sofs, sq);
+    }
+    if (pin) __builtin_amdgcn_sched_barrier(0);
+  };
+  auto issue = [&](Buf& bf, int q, bool pin) {
+    issue_w(bf, q, pin);
+    issue_sb(bf, q, pin);
+  };
+
+  // ---- activations: lane (m = j, kg) holds, for product (sl, g, h), the 8 elements of row m
+  // that the weight word of lane (., kg) covers: word 4*(2g + kg%2) + 2h + kg/2 of the slice
+  uint4 xa[SL][2][2];
+  float sx[SL][2][4];  // group sums of the activation rows 4*kg + r of this lane's results
+  Buf buf[DEPTH];
+  {
+    // range-checked loads: lanes of rows m >= M get zeros
+    const __amdgpu_buffer_rsrc_t rx =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.x), 0, p.M * p.K * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(NORM ? p.norm_w : p.x), 0, p.K * 2, 0x00020000);
+    const int lane_word = 4 * (kg & 1) + (kg >> 1);  // + 8g + 2h: the word of product (g, h)
+    const int xofs = (j * p.K + lane_word * 8) * 2, nofs = lane_word * 16;
+    const int wave_ofs = wave * (SL * 256);  // bytes of activations in front of the wave's slices
+    uint4 nraw[SL][2][2];  // the same words of the norm weights (loads return in order: before the weights)
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int wo = (sl * 16 + 8 * g + 2 * h) * 16;
+          xa[sl][g][h] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rx, xofs + wo, wave_ofs, 0));
+          if (NORM)
+            nraw[sl][g][h] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rn, nofs + wo, wave_ofs, 0));
+        }
+    // the activation loads go first (they are waited for first), then the weights - with the
+    // fused norm only the first block: the raw words, the norm weights and every buffer at
+    // once do not fit the registers, and a spilled value is reloaded behind a wait for ALL
+    // outstanding loads
+    if (NORM) {
+      issue_w(buf[0], 0, true);
+    } else {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) issue(buf[d], d, true);
+    }
+    if (NORM) {
+      // rows past the waves of this workgroup count as zero in the fixed-order sum below
+      if (wave + nw < 16 && lane < 16) {
+        for (int w2 = wave + nw; w2 < 16; w2 += nw) s_part[w2][lane] = 0.f;
+      }
+    }
+    if (NORM) {  // fused RMSNorm: every wave holds its slices of every row
+      float ss = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) ss += sumsq8(xa[sl][g][h]);
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      if (lane < 16) s_part[wave][lane] = ss;
+      __syncthreads();
+      // the waves' sums of row m in wave order: lane (m, kg) adds waves kg, kg+4, kg+8, kg+12
+      float t = (s_part[kg][j] + s_part[kg + 4][j]) + (s_part[kg + 8][j] + s_part[kg + 12][j]);
+      t += __shfl_xor(t, 16, 64);
+      t += __shfl_xor(t, 32, 64);
+      const float inv = rsqrtf(t / (float)p.K + p.eps);
+#pragma unroll
+      for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) norm8(xa[sl][g][h], nraw[sl][g][h], inv);
+    }
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        float gs = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float s1;
+          xa[sl][g][h] = pair_order(xa[sl][g][h], s1);
+          gs += s1;
+        }
+        gs += __shfl_xor(gs, 16, 64);
+        gs += __shfl_xor(gs, 32, 64);  // every lane (m, .) holds the group sum of row m
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sx[sl][g][r] = __shfl(gs, 4 * kg + r, 64);
+      }
+    if (NORM) {
+      issue_sb(buf[0], 0, true);
+#pragma unroll
+      for (int d = 1; d < DEPTH; ++d) issue(buf[d], d, true);
+    }
+  }
+
+  uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
+  asm volatile("" : "+s"(kmask));
+  asm volatile("" : "+v"(kmagic));
+  // The lane's coordinates once more, from the hardware lane count: values derived from the
+  // first copy would have to live through the register-tight set-up above, and the compiler
+  // spilled one of them - a spilled value is reloaded behind a wait for ALL outstanding loads.
+  const int lane_l = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const int jl = lane_l & 15, kgl = lane_l >> 4;
+  const bool hi_half = kgl >= 2;
+  const int lw = p.lw;
+
+  // one row block of this wave's slices; leaves the wave's partial sums in LDS slot `slot`
+  auto consume = [&](const Buf& bf, int slot) {
+    floatx4 acc[NMAT];
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a) acc[a] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          // lane (j, kg) takes its words from the lane that loaded chunk 2g + kg%2 of row j
+          const int src = (4 * jl + 2 * g + (kgl & 1)) * 4;
+          const uint32_t q0w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].x);
+          const uint32_t q1w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].y);
+          const uint32_t q2w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].z);
+          const uint32_t q3w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].w);
+          floatx4 dq = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t wd = h == 0 ? (hi_half ? q1w : q0w) : (hi_half ? q3w : q2w);
+            uint4 bw;
+            bw.x = (wd & kmask) | kmagic;
+            bw.y = ((wd >> 4) & kmask) | kmagic;
+            bw.z = ((wd >> 8) & kmask) | kmagic;
+            bw.w = ((wd >> 12) & kmask) | kmagic;
+            dq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[sl][g][h]),
+                                                        __builtin_bit_cast(bf16x8_t, bw), dq, 0, 0, 0);
+          }
+          const uint32_t sw = bf.s[a].v[sl], bwd = bf.b[a].v[sl];
+          const float sc = g == 0 ? bf_lo(sw) : bf_hi(sw);
+          const float bi = g == 0 ? bf_lo(bwd) : bf_hi(bwd);
+          const float t = fmaf(-128.f, sc, bi);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            acc[a][r] = fmaf(sc, dq[r], acc[a][r]);
+            acc[a][r] = fmaf(t, sx[sl][g][r], acc[a][r]);
+          }
+        }
+    if (lane_l < lw) {
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          red[((((size_t)slot * NMAT + a) * nw + wave) * 4 + r) * lw + lane_l] = acc[a][r];
+    }
+  };
+
+  // the phase's results: sum over the waves in a fixed order, epilogue, store
+  auto finish_phase = [&](int q_first, int n, bool res) {
+    __syncthreads();
+    for (int idx = tid; idx < n * p.M * 16; idx += (int)blockDim.x) {
+      const int jj = idx & 15, m = (idx >> 4) % p.M, slot = (idx >> 4) / p.M;
+      const int src_lane = (m >> 2) * 16 + jj, r = m & 3;
+      float tot[NMAT];
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a) {
+        const float* src = &red[(((size_t)slot * NMAT + a) * nw * 4 + r) * lw + src_lane];
+        float t = 0.f;
+        for (int w = 0; w < nw; ++w) t += src[(size_t)w * 4 * lw];
+        tot[a] = t;
+      }
+      const int row = (q0 + q_first + slot) * 16 + jj;
+      const size_t o = (size_t)m * p.N + row;
+      float out;
+      if (NMAT == 2) {  // SwiGLU on the bf16-rounded projections
+        const float g = bf2f(f2bf(tot[0])), up = bf2f(f2bf(tot[NMAT - 1]));
+        out = g / (1.f + __expf(-g)) * up;
+      } else {
+        out = tot[0];
+        if (res && p.residual) out = bf2f(f2bf(out)) + bf2f(p.residual[o]);
+      }
+      p.y[o] = f2bf(out);
+    }
+    __syncthreads();
+  };
+
+  int slot = 0, q_first = 0;
+  for (int base = 0;; base += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (base + d < nq) {
+        consume(buf[d], slot);
+        ++slot;
+      }
+      issue(buf[d], base + d + DEPTH, false);
+    }
+    if (base + DEPTH >= nq) break;
+  }
+  // (One phase: the launcher gives a workgroup no more row blocks than the LDS holds partial
+  // sums for.  A reduction inside the streaming loop - even an empty conditional block that
+  // resets `slot` - makes the compiler wait for a whole buffer too many at the first block of
+  // every round.)
+  finish_phase(q_first, slot, true);
+}
+
+constexpr size_t kRedBudget = 128 * 1024;  // LDS for the partial sums of a phase
+
+template <int NMAT, int SL, int DEPTH, bool NORM>
+int launch_w16n(W16Params p, int nw, hipStream_t st) {
+  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM>;
+  p.lw = 16 * ((p.M + 3) / 4);
+  const size_t per_block = (size_t)NMAT * nw * 4 * p.lw * sizeof(float);
+  const int ph = (int)(kRedBudget / per_block);  // row blocks whose partial sums fit the LDS
+  // one workgroup per CU; more rounds of 256 where a workgroup's share would not fit the LDS
+  int grid = 256;
+  while ((p.blocks + grid - 1) / grid > ph) grid += 256;
+  if (grid > p.blocks) grid = p.blocks;
+  const int nq = (p.blocks + grid - 1) / grid;
+  p.ph = nq;
+  const size_t lds = per_block * nq;
+  static bool attr_done = false;
+  if (!attr_done && lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) {
+      exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+      return EXO_ERR_HIP;
+    }
+    attr_done = true;
+  }
+  exo_note_variant("qmv_w16<%d,%d,%d,%s> grid=%d waves=%d phase=%d", NMAT, SL, DEPTH,
+                   NORM ? "norm" : "plain", grid, nw, ph);
+  kern<<<dim3(grid), dim3(64 * nw), lds, st>>>(p);
+  return EXO_OK;
+}
+template <int NMAT, int SL, int DEPTH>
+int launch_w16(const W16Params& p, int nw, hipStream_t st) {
+  return p.norm_w ? launch_w16n<NMAT, SL, DEPTH, true>(p, nw, st)
+                  : launch_w16n<NMAT, SL, DEPTH, false>(p, nw, st);
+}
+
+// 64-byte slices per wave and waves per workgroup for rows of `row_bytes`
+bool w16_shape(int row_bytes, int* sl_out, int* nw_out) {
+  if (row_bytes % 64) return false;
+  const int slices = row_bytes / 64;
+  for (int sl = 1; sl <= 2; sl *= 2) {
+    if (slices % sl) continue;
+    const int nw = slices / sl;
+    if (nw > 16 || nw < 4) continue;
+    *sl_out = sl;
+    *nw_out = nw;
+    return true;
+  }
+  return false;
+}
+
+}  // namespace
+
+bool exo_qmv_w16_ok(int M, int N, int K, int bits, bool residual) {
+  int sl, nw;
+  if (M < 1 || M > 16 || N % 16 || N < 16 || bits != 4 || K % 128) return false;
+  if ((int64_t)N * K / 2 >= (1ll << 31)) return false;
+  if (!w16_shape(K / 2, &sl, &nw)) return false;
+  (void)residual;
+  return true;
+}
+
+int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
+                       const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
+                       const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
+                       hipStream_t st) {
+  W16Params p;
+  p.x = x;
+  p.norm_w = norm_w;
+  p.eps = eps;
+  p.w[0] = w;
+  p.s[0] = s;
+  p.b[0] = b;
+  p.w[1] = w2 ? w2 : w;
+  p.s[1] = s2 ? s2 : s;
+  p.b[1] = b2 ? b2 : b;
+  p.residual = residual;
+  p.y = y;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.row_bytes = K / 2;
+  p.G = K / 64;
+  p.blocks = N / 16;
+  p.ph = 1;
+  p.lw = 64;
+  int sl = 0, nw = 0;
+  if (!exo_qmv_w16_ok(M, N, K, 4, residual != nullptr) || !w16_shape(p.row_bytes, &sl, &nw)) {
+    exo_set_error("exo_qmv: shape M=%d N=%d K=%d not covered by the 16x16x32 kernel", M, N, K);
+    return EXO_ERR_ARG;
+  }
+  const bool pair = w2 != nullptr;
+  if (sl == 1) return pair ? launch_w16<2, 1, 3>(p, nw, st) : launch_w16<1, 1, 4>(p, nw, st);
+  return pair ? launch_w16<2, 2, 2>(p, nw, st) : launch_w16<1, 2, 3>(p, nw, st);
+}
