@@ -34,7 +34,7 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 #define EXO_QUAD_ABL 0  // timing-only ablations (wrong results): 1 no products, 2 no lane permutation
 #endif
 #ifndef EXO_QMV_QUAD_MAX_DEPTH
-#define EXO_QMV_QUAD_MAX_DEPTH 4
+#define EXO_QMV_QUAD_MAX_DEPTH 6
 #endif
 constexpr int kQuadMaxDepth = EXO_QMV_QUAD_MAX_DEPTH;  // row quads in flight per wave, at most
 
@@ -130,10 +130,18 @@ __device__ __forceinline__ float quad_bcast(float v) {
 template <int BITS, int NMAT, int MSETS, int MU, int SL>
 __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const QuadParams p) {
   constexpr int MROWS = (MSETS - 1) * 4 + MU;  // activation rows with a result
-  // row quads in flight per wave: as many register buffers (6 registers per matrix and slice)
-  // as fit beside the activation operands without spilling - a spilled load result is waited
-  // for on the spot
-  constexpr int DEPTH0 = NMAT * SL == 1 ? 4 : ((NMAT * SL == 2 && SL == 1 && MSETS == 1) ? 3 : 2);
+  // row quads in flight per wave.  With 16 waves per CU the depth hardly matters (gate/up pair
+  // at two | four rows, us: depth 1 17.6 | 20.0, 2 17.3 | 19.8, 3 18.4 | 21.0, 4 18.6 | 21.4,
+  // 5 19.9 | 22.2; 4096x4096: depth 1 4.9 | 6.3, 2 5.2 | 6.3, 4 5.3 | 6.6, 6 5.8 | 7.1): two
+  // buffers, and no spill (a spilled load result is waited for on the spot)
+#ifndef EXO_QUAD_DEPTH_ONE
+#define EXO_QUAD_DEPTH_ONE 2
+#endif
+#ifndef EXO_QUAD_DEPTH_PAIR
+#define EXO_QUAD_DEPTH_PAIR 2
+#endif
+  constexpr int DEPTH0 = NMAT * SL == 1 ? EXO_QUAD_DEPTH_ONE
+                                        : ((NMAT * SL == 2 && SL == 1 && MSETS == 1) ? EXO_QUAD_DEPTH_PAIR : 2);
   constexpr int DEPTH = DEPTH0 > kQuadMaxDepth ? kQuadMaxDepth : DEPTH0;
   constexpr int CHUNK_EL = 128 / BITS;            // elements of a 16-byte chunk: 32 / 16
   constexpr int CPG = 64 / CHUNK_EL;              // chunks per quantisation group: 2 / 4
@@ -178,8 +186,13 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
   const int wofs = lj * p.row_bytes + wave * (SL * 256) + lb * 16;
   // group of this lane's chunk: 256 bytes hold 16 chunks = 16 / CPG groups
   const int sofs = (lj * p.G + wave * (SL * (16 / CPG)) + lb / CPG) * 2;
-  auto issue = [&](Buf& bf, int q) {  // q: row quad of this workgroup's range (past it: zeros)
+  // PIN (the issues in front of the loop): the loads leave in program order, buffer by buffer,
+  // as in the loop.  The compiler counts the loads still in flight at each wait; where the
+  // order in front of the loop differs from the order in the loop it assumes the worse of the
+  // two and waits for a whole buffer too many.
+  auto issue = [&](Buf& bf, int q, bool pin = false) {  // q: row quad of this workgroup's range (past it: zeros)
     const int wq = q * 4 * p.row_bytes, sq = q * 4 * p.G * 2;  // uniform: scalar offsets
+    if (pin) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl)
 #pragma unroll
@@ -193,6 +206,7 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
         bf.s[a][sl] = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs[a], sofs + sl * (16 / CPG) * 2, sq, 0);
         bf.b[a][sl] = (bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rb[a], sofs + sl * (16 / CPG) * 2, sq, 0);
 #endif
+        if (pin) __builtin_amdgcn_sched_barrier(0);
       }
   };
   Buf buf[DEPTH];
@@ -248,7 +262,7 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
       if (p.norm_w) nraw[t] = load_word_x<BITS>(p.norm_w, wi0 + t);
     }
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) issue(buf[d], d);
+    for (int d = 0; d < DEPTH; ++d) issue(buf[d], d, true);
     if (p.norm_w) {  // fused RMSNorm: every wave holds its slice of every row
 #pragma unroll
       for (int set = 0; set < MSETS; ++set) {
@@ -283,7 +297,7 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
     // several slices per wave (long rows; the launcher sends no fused norm here): one slice at
     // a time, so that the raw words of a slice are dead before the next ones arrive
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) issue(buf[d], d);
+    for (int d = 0; d < DEPTH; ++d) issue(buf[d], d, true);
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl)
 #pragma unroll
@@ -329,8 +343,13 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
         wd[1] = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_src, (int)bf.w[a][sl].y);
         wd[2] = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_src, (int)bf.w[a][sl].z);
         wd[3] = (uint32_t)__builtin_amdgcn_ds_bpermute(perm_src, (int)bf.w[a][sl].w);
-        const uint32_t sbw = (uint32_t)__builtin_amdgcn_ds_bpermute(
-            perm_src, (int)((uint32_t)bf.s[a][sl] | ((uint32_t)bf.b[a][sl] << 16)));
+        // (pinned here: packed any earlier - the compiler moves the two cheap operations in
+        // front of the branch around this block, to the end of the previous round - the wait
+        // for the scale loads drains the buffers that were just refilled)
+        uint32_t s_raw = bf.s[a][sl], b_raw = bf.b[a][sl];
+        asm volatile("" : "+v"(s_raw), "+v"(b_raw));
+        const uint32_t sbw =
+            (uint32_t)__builtin_amdgcn_ds_bpermute(perm_src, (int)(s_raw | (b_raw << 16)));
 #endif
         const float sc = bf_lo(sbw), bi = bf_hi(sbw);
         float4_t dq[MSETS];
@@ -425,12 +444,11 @@ __global__ __launch_bounds__(MSETS == 4 ? 512 : 1024) void qmv_quad_kernel(const
       issue(buf[d], base + d + DEPTH);
     }
     if (base + DEPTH >= nq) break;
-    if (slot + DEPTH > p.ph) {
-      finish_phase(q_first, slot, false);
-      q_first += slot;
-      slot = 0;
-    }
   }
+  // (One phase: the launcher gives a workgroup no more row quads than the LDS holds partial
+  // sums for.  A reduction inside the streaming loop - even an empty conditional block that
+  // resets `slot` - makes the compiler wait for a whole buffer too many at the first quad of
+  // every round.)
   finish_phase(q_first, slot, true);
 }
 
@@ -440,24 +458,18 @@ template <int BITS, int NMAT, int MSETS, int MU, int SL>
 int launch_quad(QuadParams p, int nw, hipStream_t st) {
   auto kern = qmv_quad_kernel<BITS, NMAT, MSETS, MU, SL>;
   constexpr int MROWS = (MSETS - 1) * 4 + MU;
-  // one round of workgroups: two per CU up to 8 waves, one beyond; at least one row quad each
+  // one round of workgroups: two per CU up to 8 waves, one beyond; more rounds where a
+  // workgroup's row quads would not fit the LDS with their partial sums
   const int per_cu = (nw <= 8 && MSETS < 4) ? 2 : 1;
+  const size_t per_quad = (size_t)NMAT * MROWS * nw * 16 * sizeof(float);
+  const size_t budget = per_cu == 2 ? kRedBudget : 2 * kRedBudget;
+  const int ph = (int)(budget / per_quad);
   int grid = 256 * per_cu;
+  while ((p.quads + grid - 1) / grid > ph) grid += 256 * per_cu;
   if (grid > p.quads) grid = p.quads;
   const int nq = (p.quads + grid - 1) / grid;
-  const size_t per_quad = (size_t)NMAT * MROWS * nw * 16 * sizeof(float);
-  int ph = (int)(kRedBudget / per_quad);
-  if (ph > nq) ph = nq;
-  // a phase holds one round of the register buffers at least; a residual is added in the
-  // last phase only, so such a launch has one phase
-  const int need = (p.residual && NMAT == 1) ? nq : (nq < 8 ? nq : 8);
-  if (ph < need) ph = need;
-  p.ph = ph;
-  const size_t lds = per_quad * ph;
-  if (lds > 150 * 1024) {
-    exo_set_error("exo_qmv: %d row quads per workgroup need %zu bytes of LDS", nq, lds);
-    return EXO_ERR_ARG;
-  }
+  p.ph = nq;
+  const size_t lds = per_quad * nq;
   static bool attr_done = false;
   if (!attr_done && lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

@@ -25,6 +25,10 @@
 
 namespace {
 
+#ifndef EXO_W16_ABL
+#define EXO_W16_ABL 0  // timing-only ablations (wrong results): 1 no products, 2 no lane permutation, 4 no group epilogue, 8 no unpacking
+#endif
+
 struct W16Params {
   const bf16_t* x;       // [M, K]
   const bf16_t* norm_w;  // [K] or null: fused RMSNorm of x
@@ -40,6 +44,7 @@ struct W16Params {
   int blocks;     // N / 16
   int ph;         // row blocks per workgroup at most (LDS holds their partial sums)
   int lw;         // lanes of a wave that hold results: 16 * ceil(M / 4)
+  int red_bytes;  // LDS bytes of the partial sums; the staged scales and biases follow
 };
 
 __device__ __forceinline__ float sumsq8(const uint4& v) {
@@ -89,7 +94,13 @@ struct SbWord<2> {
 // NMAT matrices (2: the (gate, up) pair with SwiGLU), SL 64-byte slices of K per wave, DEPTH
 // row blocks in flight per wave.
 // NORM: fused RMSNorm of the activations.
-template <int NMAT, int SL, int DEPTH, bool NORM>
+// SBLDS: the scales and biases of ALL the workgroup's rows are staged in LDS in front of the
+// loop, with whole-line loads (one 16-byte chunk per thread and array).  Loaded per block by
+// the lanes that need them - 8 bytes each out of 16 different lines per instruction, every
+// line touched again by each of the 16 waves - they cost 4.5 of the 24 us of the 14336x4096
+// pair (measured with the loads taken out).  Needs K a multiple of 512 and LDS for them beside
+// the partial sums (up to 8 activation rows).
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS>
 __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   extern __shared__ float red[];  // [ph][NMAT][nw][4][lw]
   __shared__ float s_part[16][16];
@@ -135,23 +146,45 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     for (int sl = 0; sl < SL; ++sl)
 #pragma unroll
       for (int a = 0; a < NMAT; ++a)
+#if (EXO_W16_ABL & 16)  // timing only: 8 rows x 128 bytes per instruction (SL == 2)
+        bf.w[a][sl] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                       rw[a], ((lane >> 3) + 8 * sl) * p.row_bytes + wave * (SL * 64) + (lane & 7) * 16, wq, 0));
+#elif (EXO_W16_ABL & 32)  // timing only: 4 rows x 256 bytes per instruction, two waves share 256 bytes
+        bf.w[a][sl] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                       rw[a], ((lane >> 4) + 4 * sl + 8 * (wave & 1)) * p.row_bytes + (wave >> 1) * 256 + (lane & 15) * 16, wq, 0));
+#else
         bf.w[a][sl] = __builtin_bit_cast(
             uint4, __builtin_amdgcn_raw_buffer_load_b128(rw[a], wofs + sl * 64, wq, 0));
+#endif
     if (pin) __builtin_amdgcn_sched_barrier(0);
   };
   auto issue_sb = [&](Buf& bf, int q, bool pin) {
     const int sq = q * 16 * p.G * 2;
+#if (EXO_W16_ABL & 64)  // timing only: no scale / bias loads
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+      for (int sl = 0; sl < SL; ++sl) bf.s[a].v[sl] = bf.b[a].v[sl] = 0x3c003c00u + sq;
+#else
 #pragma unroll
     for (int a = 0; a < NMAT; ++a) {
       bf.s[a].load(rs[a], sofs, sq);
       bf.b[a].load(rb[a], sofs, sq);
     }
+#endif
     if (pin) __builtin_amdgcn_sched_barrier(0);
   };
   auto issue = [&](Buf& bf, int q, bool pin) {
     issue_w(bf, q, pin);
-    issue_sb(bf, q, pin);
+    if (!SBLDS) issue_sb(bf, q, pin);
   };
+  // staged scales / biases: array (matrix a, scale|bias) x local row x (G + 4) bf16 (rows
+  // padded by 8 bytes: the 16 rows a wave reads at once then sit in different banks)
+  char* const sb_lds = reinterpret_cast<char*>(red) + p.red_bytes;
+  const int sb_row = p.G * 2 + 8, sb_arr = p.ph * 16 * sb_row;
+  char* const nw_lds = sb_lds + (SBLDS ? NMAT * 2 * sb_arr : 0);  // the norm weights, K bf16
 
   // ---- activations: lane (m = j, kg) holds, for product (sl, g, h), the 8 elements of row m
   // that the weight word of lane (., kg) covers: word 4*(2g + kg%2) + 2h + kg/2 of the slice
@@ -167,7 +200,20 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     const int lane_word = 4 * (kg & 1) + (kg >> 1);  // + 8g + 2h: the word of product (g, h)
     const int xofs = (j * p.K + lane_word * 8) * 2, nofs = lane_word * 16;
     const int wave_ofs = wave * (SL * 256);  // bytes of activations in front of the wave's slices
-    uint4 nraw[SL][2][2];  // the same words of the norm weights (loads return in order: before the weights)
+    // staging: chunk tid of each array (past the workgroup's rows: out of range, no traffic)
+    // (the norm weights too: chunk tid; every lane reads its words back after the barrier -
+    // loaded per lane they are 16 times the bytes, one copy per activation row, and their
+    // registers are live across the barrier beside everything else)
+    uint4 nstg = make_uint4(0, 0, 0, 0);
+    if (NORM) nstg = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rn, tid * 16, 0, 0));
+    uint4 stg[NMAT][2];
+    if (SBLDS) {
+#pragma unroll
+      for (int a = 0; a < NMAT; ++a) {
+        stg[a][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs[a], tid * 16, 0, 0));
+        stg[a][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[a], tid * 16, 0, 0));
+      }
+    }
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl)
 #pragma unroll
@@ -176,18 +222,30 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
         for (int h = 0; h < 2; ++h) {
           const int wo = (sl * 16 + 8 * g + 2 * h) * 16;
           xa[sl][g][h] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rx, xofs + wo, wave_ofs, 0));
-          if (NORM)
-            nraw[sl][g][h] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rn, nofs + wo, wave_ofs, 0));
         }
     // the activation loads go first (they are waited for first), then the weights - with the
-    // fused norm only the first block: the raw words, the norm weights and every buffer at
-    // once do not fit the registers, and a spilled value is reloaded behind a wait for ALL
+    // fused norm only the first block: beside the raw words and the staging registers every
+    // buffer at once does not fit, and a spilled value is reloaded behind a wait for ALL
     // outstanding loads
-    if (NORM) {
-      issue_w(buf[0], 0, true);
-    } else {
 #pragma unroll
-      for (int d = 0; d < DEPTH; ++d) issue(buf[d], d, true);
+    for (int d = 0; d < (NORM ? 1 : DEPTH); ++d) issue(buf[d], d, true);
+    auto stage_sb = [&](const uint4 (&v)[NMAT][2]) {
+      const int cpr = p.G >> 3;  // 16-byte chunks per row
+      const int row = tid / cpr, col = tid - row * cpr;
+      if (row < nq * 16) {
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            uint2* dst = reinterpret_cast<uint2*>(sb_lds + (a * 2 + t) * sb_arr + row * sb_row + col * 16);
+            dst[0] = make_uint2(v[a][t].x, v[a][t].y);
+            dst[1] = make_uint2(v[a][t].z, v[a][t].w);
+          }
+      }
+    };
+    if (SBLDS && !NORM) {
+      stage_sb(stg);
+      __syncthreads();
     }
     if (NORM) {
       // rows past the waves of this workgroup count as zero in the fixed-order sum below
@@ -206,6 +264,8 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
       ss += __shfl_xor(ss, 16, 64);
       ss += __shfl_xor(ss, 32, 64);
       if (lane < 16) s_part[wave][lane] = ss;
+      if (SBLDS) stage_sb(stg);
+      if (tid * 16 < p.K * 2) *reinterpret_cast<uint4*>(nw_lds + tid * 16) = nstg;
       __syncthreads();
       // the waves' sums of row m in wave order: lane (m, kg) adds waves kg, kg+4, kg+8, kg+12
       float t = (s_part[kg][j] + s_part[kg + 4][j]) + (s_part[kg + 8][j] + s_part[kg + 12][j]);
@@ -217,7 +277,10 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
 #pragma unroll
         for (int g = 0; g < 2; ++g)
 #pragma unroll
-          for (int h = 0; h < 2; ++h) norm8(xa[sl][g][h], nraw[sl][g][h], inv);
+          for (int h = 0; h < 2; ++h) {
+            const int wo = (sl * 16 + 8 * g + 2 * h) * 16;
+            norm8(xa[sl][g][h], *reinterpret_cast<const uint4*>(nw_lds + wave_ofs + nofs + wo), inv);
+          }
     }
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl)
@@ -236,7 +299,6 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
         for (int r = 0; r < 4; ++r) sx[sl][g][r] = __shfl(gs, 4 * kg + r, 64);
       }
     if (NORM) {
-      issue_sb(buf[0], 0, true);
 #pragma unroll
       for (int d = 1; d < DEPTH; ++d) issue(buf[d], d, true);
     }
@@ -266,31 +328,55 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
         for (int g = 0; g < 2; ++g) {
           // lane (j, kg) takes its words from the lane that loaded chunk 2g + kg%2 of row j
           const int src = (4 * jl + 2 * g + (kgl & 1)) * 4;
+#if (EXO_W16_ABL & 2)
+          const uint32_t q0w = bf.w[a][sl].x + src, q1w = bf.w[a][sl].y, q2w = bf.w[a][sl].z, q3w = bf.w[a][sl].w;
+#else
           const uint32_t q0w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].x);
           const uint32_t q1w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].y);
           const uint32_t q2w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].z);
           const uint32_t q3w = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)bf.w[a][sl].w);
+#endif
           floatx4 dq = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const uint32_t wd = h == 0 ? (hi_half ? q1w : q0w) : (hi_half ? q3w : q2w);
             uint4 bw;
+#if (EXO_W16_ABL & 8)
+            bw.x = wd; bw.y = wd ^ kmagic; bw.z = wd | kmagic; bw.w = wd & kmagic;
+#else
             bw.x = (wd & kmask) | kmagic;
             bw.y = ((wd >> 4) & kmask) | kmagic;
             bw.z = ((wd >> 8) & kmask) | kmagic;
             bw.w = ((wd >> 12) & kmask) | kmagic;
+#endif
+#if (EXO_W16_ABL & 1)
+            dq[0] += __builtin_bit_cast(float, bw.x ^ bw.y ^ bw.z ^ bw.w ^ xa[sl][g][h].x);
+#else
             dq = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[sl][g][h]),
                                                         __builtin_bit_cast(bf16x8_t, bw), dq, 0, 0, 0);
+#endif
           }
-          const uint32_t sw = bf.s[a].v[sl], bwd = bf.b[a].v[sl];
+          uint32_t sw, bwd;
+          if (SBLDS) {
+            const char* base = sb_lds + (slot * 16 + jl) * sb_row + (wave * SL + sl) * 4;
+            sw = *reinterpret_cast<const uint32_t*>(base + (a * 2) * sb_arr);
+            bwd = *reinterpret_cast<const uint32_t*>(base + (a * 2 + 1) * sb_arr);
+          } else {
+            sw = bf.s[a].v[sl];
+            bwd = bf.b[a].v[sl];
+          }
           const float sc = g == 0 ? bf_lo(sw) : bf_hi(sw);
           const float bi = g == 0 ? bf_lo(bwd) : bf_hi(bwd);
+#if (EXO_W16_ABL & 4)
+          acc[a][0] += dq[0] * sc + dq[1] + dq[2] + dq[3] + bi;
+#else
           const float t = fmaf(-128.f, sc, bi);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             acc[a][r] = fmaf(sc, dq[r], acc[a][r]);
             acc[a][r] = fmaf(t, sx[sl][g][r], acc[a][r]);
           }
+#endif
         }
     if (lane_l < lw) {
 #pragma unroll
@@ -349,40 +435,57 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   finish_phase(q_first, slot, true);
 }
 
-constexpr size_t kRedBudget = 128 * 1024;  // LDS for the partial sums of a phase
+constexpr size_t kLdsBudget = 144 * 1024;  // LDS for partial sums and staged scales (the norm weights: 8 KB more)
 
-template <int NMAT, int SL, int DEPTH, bool NORM>
-int launch_w16n(W16Params p, int nw, hipStream_t st) {
-  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM>;
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS>
+int launch_w16s(W16Params p, int nw, hipStream_t st) {
+  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM, SBLDS>;
   p.lw = 16 * ((p.M + 3) / 4);
   const size_t per_block = (size_t)NMAT * nw * 4 * p.lw * sizeof(float);
-  const int ph = (int)(kRedBudget / per_block);  // row blocks whose partial sums fit the LDS
+  const size_t sb_block = SBLDS ? (size_t)NMAT * 2 * 16 * (p.G * 2 + 8) : 0;
+  int ph = (int)(kLdsBudget / (per_block + sb_block));  // row blocks a workgroup can hold
+  // staging: one 16-byte chunk per thread and array
+  if (SBLDS && ph > 32 * nw / p.G) ph = 32 * nw / p.G;
+  if (ph < 1) {
+    exo_set_error("exo_qmv: internal: no LDS for one row block (M=%d K=%d)", p.M, p.K);
+    return EXO_ERR_ARG;
+  }
   // one workgroup per CU; more rounds of 256 where a workgroup's share would not fit the LDS
   int grid = 256;
   while ((p.blocks + grid - 1) / grid > ph) grid += 256;
   if (grid > p.blocks) grid = p.blocks;
   const int nq = (p.blocks + grid - 1) / grid;
   p.ph = nq;
-  const size_t lds = per_block * nq;
+  p.red_bytes = (int)(per_block * nq);
+  const size_t lds = (per_block + sb_block) * nq + (NORM ? (size_t)p.K * 2 : 0);
   static bool attr_done = false;
   if (!attr_done && lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024);
     if (e != hipSuccess) {
       exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
       return EXO_ERR_HIP;
     }
     attr_done = true;
   }
-  exo_note_variant("qmv_w16<%d,%d,%d,%s> grid=%d waves=%d phase=%d", NMAT, SL, DEPTH,
-                   NORM ? "norm" : "plain", grid, nw, ph);
+  exo_note_variant("qmv_w16<%d,%d,%d,%s,%s> grid=%d waves=%d blocks=%d", NMAT, SL, DEPTH,
+                   NORM ? "norm" : "plain", SBLDS ? "staged" : "direct", grid, nw, nq);
   kern<<<dim3(grid), dim3(64 * nw), lds, st>>>(p);
   return EXO_OK;
 }
 template <int NMAT, int SL, int DEPTH>
 int launch_w16(const W16Params& p, int nw, hipStream_t st) {
-  return p.norm_w ? launch_w16n<NMAT, SL, DEPTH, true>(p, nw, st)
-                  : launch_w16n<NMAT, SL, DEPTH, false>(p, nw, st);
+  // staged scales where they fit the LDS beside the partial sums of one round of 256 workgroups
+  // (the 14336-row pair: up to 12 activation rows) and one chunk per thread covers them
+  const int grid1 = p.blocks < 256 ? p.blocks : 256, nq1 = (p.blocks + grid1 - 1) / grid1;
+  const size_t need1 = ((size_t)NMAT * nw * 4 * 16 * ((p.M + 3) / 4) * sizeof(float) +
+                        (size_t)NMAT * 2 * 16 * (p.G * 2 + 8)) * nq1;
+  const bool staged = p.G % 8 == 0 && need1 <= kLdsBudget && nq1 <= 32 * nw / p.G && !(EXO_W16_ABL & 128);
+  if (p.norm_w)
+    return staged ? launch_w16s<NMAT, SL, DEPTH, true, true>(p, nw, st)
+                  : launch_w16s<NMAT, SL, DEPTH, true, false>(p, nw, st);
+  return staged ? launch_w16s<NMAT, SL, DEPTH, false, true>(p, nw, st)
+                : launch_w16s<NMAT, SL, DEPTH, false, false>(p, nw, st);
 }
 
 // 64-byte slices per wave and waves per workgroup for rows of `row_bytes`
@@ -441,6 +544,9 @@ int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const u
     return EXO_ERR_ARG;
   }
   const bool pair = w2 != nullptr;
-  if (sl == 1) return pair ? launch_w16<2, 1, 3>(p, nw, st) : launch_w16<1, 1, 4>(p, nw, st);
-  return pair ? launch_w16<2, 2, 2>(p, nw, st) : launch_w16<1, 2, 3>(p, nw, st);
+#ifndef EXO_W16_DEPTH
+#define EXO_W16_DEPTH 2
+#endif
+  if (sl == 1) return pair ? launch_w16<2, 1, EXO_W16_DEPTH>(p, nw, st) : launch_w16<1, 1, EXO_W16_DEPTH>(p, nw, st);
+  return pair ? launch_w16<2, 2, 2>(p, nw, st) : launch_w16<1, 2, EXO_W16_DEPTH>(p, nw, st);
 }
