@@ -1704,12 +1704,13 @@ static int norm_qmv_impl(const uint16_t* x, const uint16_t* norm_weight, float e
     EXO_CHECK_LAUNCH("exo_qmv");
     return EXO_OK;
   }
-  if (M >= EXO_QMV_W16_MIN_M && exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, residual != nullptr)) {
+  if (M >= EXO_QMV_W16_MIN_M &&
+      exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, norm_weight != nullptr, false, workspace != nullptr)) {
     for (int m0 = 0; m0 < M; m0 += 16) {
       const int mt = (M - m0 < 16) ? (M - m0) : 16;
       rc = exo_qmv_w16_launch(x + (size_t)m0 * K, norm_weight, eps, w, scales, biases, nullptr,
                               nullptr, nullptr, residual ? residual + (size_t)m0 * N : nullptr,
-                              y + (size_t)m0 * N, mt, N, K, (hipStream_t)stream);
+                              y + (size_t)m0 * N, mt, N, K, workspace, (hipStream_t)stream);
       if (rc) return rc;
     }
     EXO_CHECK_LAUNCH("exo_qmv");
@@ -1811,11 +1812,11 @@ extern "C" int exo_norm_qmv_swiglu_ws(const uint16_t* x, const uint16_t* norm_we
     EXO_CHECK_LAUNCH("exo_qmv_swiglu");
     return EXO_OK;
   }
-  if (M >= EXO_QMV_W16_MIN_M && exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, false)) {
+  if (M >= EXO_QMV_W16_MIN_M && exo_qmv_w16_ok(M < 16 ? M : 16, N, K, bits, norm_weight != nullptr, true, false)) {
     for (int m0 = 0; m0 < M; m0 += 16) {
       const int mt = (M - m0 < 16) ? (M - m0) : 16;
       rc = exo_qmv_w16_launch(x + (size_t)m0 * K, norm_weight, eps, wg, sg, bg, wu, su, bu, nullptr,
-                              y + (size_t)m0 * N, mt, N, K, (hipStream_t)stream);
+                              y + (size_t)m0 * N, mt, N, K, nullptr, (hipStream_t)stream);
       if (rc) return rc;
     }
     EXO_CHECK_LAUNCH("exo_qmv_swiglu");

@@ -23,11 +23,12 @@ int exo_qmv_quad_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const 
                         const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
                         int bits, hipStream_t st);
 
-// 16x16x32 matrix-core GEMV for up to 16 activation rows (qmv_w16.hip): 4-bit codes, rows of
-// 4..32 whole 64-byte slices (K of 512 to 4096), N a multiple of 16.  w2/s2/b2 non-null: the
-// (gate, up) pair with SwiGLU.
-bool exo_qmv_w16_ok(int M, int N, int K, int bits, bool residual);
+// 16x16x32 matrix-core GEMV for up to 16 activation rows (qmv_w16.hip): 4-bit codes, N a
+// multiple of 16, rows of 4..32 whole 64-byte slices (K of 512 to 4096) - longer rows with a
+// workspace (the split-K workspace of exo_qmv_mfma_workspace(N)), no fused norm and a single
+// matrix: K then splits over 2..8 workgroups.  w2/s2/b2 non-null: the (gate, up) pair with SwiGLU.
+bool exo_qmv_w16_ok(int M, int N, int K, int bits, bool norm, bool pair, bool has_workspace);
 int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
                        const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
                        const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
-                       hipStream_t st);
+                       void* workspace, hipStream_t st);

@@ -45,7 +45,21 @@ struct W16Params {
   int ph;         // row blocks per workgroup at most (LDS holds their partial sums)
   int lw;         // lanes of a wave that hold results: 16 * ceil(M / 4)
   int red_bytes;  // LDS bytes of the partial sums; the staged scales and biases follow
+  // K split over `kparts` workgroups per group of row blocks (long rows: the activations of
+  // a whole row would not fit the registers): workgroup i takes part i % kparts, Gp groups
+  // of every row; float32 partial results meet in `part`, the last workgroup of a group to
+  // arrive adds them in part order
+  int kparts, Gp;
+  float* part;    // [kparts][M][N]
+  int* counters;  // [block groups], zero between launches
 };
+
+__device__ __forceinline__ void st_dev(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_dev(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ float sumsq8(const uint4& v) {
   return bf_lo(v.x) * bf_lo(v.x) + bf_hi(v.x) * bf_hi(v.x) + bf_lo(v.y) * bf_lo(v.y) +
@@ -100,10 +114,14 @@ struct SbWord<2> {
 // line touched again by each of the 16 waves - they cost 4.5 of the 24 us of the 14336x4096
 // pair (measured with the loads taken out).  Needs K a multiple of 512 and LDS for them beside
 // the partial sums (up to 8 activation rows).
-template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS>
+// KSPLIT: K split over several workgroups (single matrix, no fused norm).  An instance of its
+// own: compiled into the others, the hand-over code costs them 0.5 us per launch untaken.
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false>
 __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
+  constexpr bool KSPLIT_OK = KSPLIT && NMAT == 1 && !NORM;
   extern __shared__ float red[];  // [ph][NMAT][nw][4][lw]
   __shared__ float s_part[16][16];
+  __shared__ int s_last;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,10 +130,14 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   const int lr = lane >> 2, lc = lane & 3;  // load layout: row of the block, chunk of the slice
 
   // contiguous, balanced range of row blocks of this workgroup
-  const int qbase = p.blocks / (int)gridDim.x, qrem = p.blocks - qbase * (int)gridDim.x;
-  const int q0 = (int)blockIdx.x * qbase + min((int)blockIdx.x, qrem);
-  const int nq = qbase + ((int)blockIdx.x < qrem ? 1 : 0);
+  const int kparts = KSPLIT_OK ? p.kparts : 1;
+  const int kpart = (int)blockIdx.x % kparts, bgroup = (int)blockIdx.x / kparts;
+  const int ngroups = (int)gridDim.x / kparts;
+  const int qbase = p.blocks / ngroups, qrem = p.blocks - qbase * ngroups;
+  const int q0 = bgroup * qbase + min(bgroup, qrem);
+  const int nq = qbase + (bgroup < qrem ? 1 : 0);
   if (nq <= 0) return;
+  const int g_first = kpart * p.Gp;  // first quantisation group of this workgroup's part of K
 
   struct Buf {
     uint4 w[NMAT][SL];
@@ -133,8 +155,8 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     rb[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.b[a] + (size_t)q0 * 16 * p.G), 0,
                                               nq * 16 * p.G * 2, 0x00020000);
   }
-  const int wofs = lr * p.row_bytes + wave * (SL * 64) + lc * 16;
-  const int sofs = (j * p.G + wave * (SL * 2)) * 2;  // this lane's weight row, the wave's groups
+  const int wofs = lr * p.row_bytes + g_first * 32 + wave * (SL * 64) + lc * 16;
+  const int sofs = (j * p.G + g_first + wave * (SL * 2)) * 2;  // this lane's weight row, the wave's groups
   // PIN (the issues in front of the loop): the loads leave in program order - weights, then
   // scales and biases, buffer by buffer, as in the loop.  The compiler counts the loads still
   // in flight at each wait; where the order in front of the loop differs from the order in the
@@ -183,7 +205,7 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   // staged scales / biases: array (matrix a, scale|bias) x local row x (G + 4) bf16 (rows
   // padded by 8 bytes: the 16 rows a wave reads at once then sit in different banks)
   char* const sb_lds = reinterpret_cast<char*>(red) + p.red_bytes;
-  const int sb_row = p.G * 2 + 8, sb_arr = p.ph * 16 * sb_row;
+  const int sb_row = p.Gp * 2 + 8, sb_arr = p.ph * 16 * sb_row;
   char* const nw_lds = sb_lds + (SBLDS ? NMAT * 2 * sb_arr : 0);  // the norm weights, K bf16
 
   // ---- activations: lane (m = j, kg) holds, for product (sl, g, h), the 8 elements of row m
@@ -199,7 +221,8 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
         const_cast<bf16_t*>(NORM ? p.norm_w : p.x), 0, p.K * 2, 0x00020000);
     const int lane_word = 4 * (kg & 1) + (kg >> 1);  // + 8g + 2h: the word of product (g, h)
     const int xofs = (j * p.K + lane_word * 8) * 2, nofs = lane_word * 16;
-    const int wave_ofs = wave * (SL * 256);  // bytes of activations in front of the wave's slices
+    // bytes of activations in front of the wave's slices
+    const int wave_ofs = g_first * 128 + wave * (SL * 256);
     // staging: chunk tid of each array (past the workgroup's rows: out of range, no traffic)
     // (the norm weights too: chunk tid; every lane reads its words back after the barrier -
     // loaded per lane they are 16 times the bytes, one copy per activation row, and their
@@ -208,10 +231,13 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     if (NORM) nstg = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rn, tid * 16, 0, 0));
     uint4 stg[NMAT][2];
     if (SBLDS) {
+      // thread -> (local row, 16-byte chunk of the row's part); past the rows: out of range
+      const int cpr = p.Gp >> 3, row = tid / cpr, col = tid - row * cpr;
+      const int so = row < nq * 16 ? (row * p.G + g_first) * 2 + col * 16 : 0x7ffffff0;
 #pragma unroll
       for (int a = 0; a < NMAT; ++a) {
-        stg[a][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs[a], tid * 16, 0, 0));
-        stg[a][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[a], tid * 16, 0, 0));
+        stg[a][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs[a], so, 0, 0));
+        stg[a][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[a], so, 0, 0));
       }
     }
 #pragma unroll
@@ -230,7 +256,7 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
 #pragma unroll
     for (int d = 0; d < (NORM ? 1 : DEPTH); ++d) issue(buf[d], d, true);
     auto stage_sb = [&](const uint4 (&v)[NMAT][2]) {
-      const int cpr = p.G >> 3;  // 16-byte chunks per row
+      const int cpr = p.Gp >> 3;  // 16-byte chunks per row
       const int row = tid / cpr, col = tid - row * cpr;
       if (row < nq * 16) {
 #pragma unroll
@@ -403,6 +429,10 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
       }
       const int row = (q0 + q_first + slot) * 16 + jj;
       const size_t o = (size_t)m * p.N + row;
+      if (KSPLIT_OK && p.kparts > 1) {  // (single matrices only) this part's share of the sum
+        st_dev(&p.part[(size_t)kpart * p.M * p.N + o], tot[0]);
+        continue;
+      }
       float out;
       if (NMAT == 2) {  // SwiGLU on the bf16-rounded projections
         const float g = bf2f(f2bf(tot[0])), up = bf2f(f2bf(tot[NMAT - 1]));
@@ -414,6 +444,28 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
       p.y[o] = f2bf(out);
     }
     __syncthreads();
+  };
+  // Split K: the last of a group's workgroups to arrive adds the parts in part order (the result
+  // does not depend on arrival order) and writes y; the counter returns to zero.
+  auto merge_parts = [&](int n) {
+    wait_own_stores_done();  // this wave's device-scope partial stores have completed
+    __syncthreads();
+    if (tid == 0) {
+      int* cnt = &p.counters[bgroup];
+      const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == p.kparts - 1);
+      if (s_last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int idx = tid; idx < n * p.M * 16; idx += (int)blockDim.x) {
+      const int jj = idx & 15, m = (idx >> 4) % p.M, slot = (idx >> 4) / p.M;
+      const size_t o = (size_t)m * p.N + (q0 + slot) * 16 + jj;
+      float t = 0.f;
+      for (int kp = 0; kp < p.kparts; ++kp) t += ld_dev(&p.part[(size_t)kp * p.M * p.N + o]);
+      if (p.residual) t = bf2f(f2bf(t)) + bf2f(p.residual[o]);
+      p.y[o] = f2bf(t);
+    }
   };
 
   int slot = 0, q_first = 0;
@@ -433,28 +485,32 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   // resets `slot` - makes the compiler wait for a whole buffer too many at the first block of
   // every round.)
   finish_phase(q_first, slot, true);
+  if (KSPLIT_OK && p.kparts > 1) merge_parts(slot);
 }
 
 constexpr size_t kLdsBudget = 144 * 1024;  // LDS for partial sums and staged scales (the norm weights: 8 KB more)
 
-template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS>
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false>
 int launch_w16s(W16Params p, int nw, hipStream_t st) {
-  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM, SBLDS>;
+  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM, SBLDS, KSPLIT>;
   p.lw = 16 * ((p.M + 3) / 4);
   const size_t per_block = (size_t)NMAT * nw * 4 * p.lw * sizeof(float);
-  const size_t sb_block = SBLDS ? (size_t)NMAT * 2 * 16 * (p.G * 2 + 8) : 0;
+  const size_t sb_block = SBLDS ? (size_t)NMAT * 2 * 16 * (p.Gp * 2 + 8) : 0;
   int ph = (int)(kLdsBudget / (per_block + sb_block));  // row blocks a workgroup can hold
   // staging: one 16-byte chunk per thread and array
-  if (SBLDS && ph > 32 * nw / p.G) ph = 32 * nw / p.G;
+  if (SBLDS && ph > 32 * nw / p.Gp) ph = 32 * nw / p.Gp;
   if (ph < 1) {
     exo_set_error("exo_qmv: internal: no LDS for one row block (M=%d K=%d)", p.M, p.K);
     return EXO_ERR_ARG;
   }
-  // one workgroup per CU; more rounds of 256 where a workgroup's share would not fit the LDS
-  int grid = 256;
-  while ((p.blocks + grid - 1) / grid > ph) grid += 256;
-  if (grid > p.blocks) grid = p.blocks;
-  const int nq = (p.blocks + grid - 1) / grid;
+  // one workgroup per CU (kparts workgroups per group of row blocks); more rounds where a
+  // workgroup's share would not fit the LDS
+  const int round = 256 / p.kparts;
+  int groups = round;
+  while ((p.blocks + groups - 1) / groups > ph) groups += round;
+  if (groups > p.blocks) groups = p.blocks;
+  const int grid = groups * p.kparts;
+  const int nq = (p.blocks + groups - 1) / groups;
   p.ph = nq;
   p.red_bytes = (int)(per_block * nq);
   const size_t lds = (per_block + sb_block) * nq + (NORM ? (size_t)p.K * 2 : 0);
@@ -468,8 +524,8 @@ int launch_w16s(W16Params p, int nw, hipStream_t st) {
     }
     attr_done = true;
   }
-  exo_note_variant("qmv_w16<%d,%d,%d,%s,%s> grid=%d waves=%d blocks=%d", NMAT, SL, DEPTH,
-                   NORM ? "norm" : "plain", SBLDS ? "staged" : "direct", grid, nw, nq);
+  exo_note_variant("qmv_w16<%d,%d,%d,%s,%s> grid=%d waves=%d blocks=%d kparts=%d", NMAT, SL, DEPTH,
+                   NORM ? "norm" : "plain", SBLDS ? "staged" : "direct", grid, nw, nq, p.kparts);
   kern<<<dim3(grid), dim3(64 * nw), lds, st>>>(p);
   return EXO_OK;
 }
@@ -477,10 +533,18 @@ template <int NMAT, int SL, int DEPTH>
 int launch_w16(const W16Params& p, int nw, hipStream_t st) {
   // staged scales where they fit the LDS beside the partial sums of one round of 256 workgroups
   // (the 14336-row pair: up to 12 activation rows) and one chunk per thread covers them
-  const int grid1 = p.blocks < 256 ? p.blocks : 256, nq1 = (p.blocks + grid1 - 1) / grid1;
+  const int round = 256 / p.kparts;
+  const int groups1 = p.blocks < round ? p.blocks : round, nq1 = (p.blocks + groups1 - 1) / groups1;
   const size_t need1 = ((size_t)NMAT * nw * 4 * 16 * ((p.M + 3) / 4) * sizeof(float) +
-                        (size_t)NMAT * 2 * 16 * (p.G * 2 + 8)) * nq1;
-  const bool staged = p.G % 8 == 0 && need1 <= kLdsBudget && nq1 <= 32 * nw / p.G && !(EXO_W16_ABL & 128);
+                        (size_t)NMAT * 2 * 16 * (p.Gp * 2 + 8)) * nq1;
+  const bool staged = p.Gp % 8 == 0 && need1 <= kLdsBudget && nq1 <= 32 * nw / p.Gp && !(EXO_W16_ABL & 128);
+  if (p.kparts > 1) {
+    if constexpr (NMAT == 1)
+      return staged ? launch_w16s<1, SL, DEPTH, false, true, true>(p, nw, st)
+                    : launch_w16s<1, SL, DEPTH, false, false, true>(p, nw, st);
+    exo_set_error("exo_qmv: internal: split K with a matrix pair");
+    return EXO_ERR_ARG;
+  }
   if (p.norm_w)
     return staged ? launch_w16s<NMAT, SL, DEPTH, true, true>(p, nw, st)
                   : launch_w16s<NMAT, SL, DEPTH, true, false>(p, nw, st);
@@ -503,21 +567,35 @@ bool w16_shape(int row_bytes, int* sl_out, int* nw_out) {
   return false;
 }
 
+// parts of K (workgroups per group of row blocks) for rows of `row_bytes`: 1 where a row's
+// activations fit the registers of one workgroup, else - with a workspace, without a fused norm
+// or a second matrix - the smallest split into equal parts of whole 16-byte scale chunks
+int w16_parts(int row_bytes, bool can_split, int* sl_out, int* nw_out) {
+  if (w16_shape(row_bytes, sl_out, nw_out)) return 1;
+  if (!can_split || row_bytes % 64) return 0;
+  const int slices = row_bytes / 64;  // one slice = two quantisation groups
+  for (int kp = 2; kp <= 8; ++kp)
+    if (slices % kp == 0 && (2 * slices / kp) % 8 == 0 && w16_shape(row_bytes / kp, sl_out, nw_out))
+      return kp;
+  return 0;
+}
+
 }  // namespace
 
-bool exo_qmv_w16_ok(int M, int N, int K, int bits, bool residual) {
+bool exo_qmv_w16_ok(int M, int N, int K, int bits, bool norm, bool pair, bool has_workspace) {
   int sl, nw;
   if (M < 1 || M > 16 || N % 16 || N < 16 || bits != 4 || K % 128) return false;
   if ((int64_t)N * K / 2 >= (1ll << 31)) return false;
-  if (!w16_shape(K / 2, &sl, &nw)) return false;
-  (void)residual;
+  const int kp = w16_parts(K / 2, has_workspace && !norm && !pair, &sl, &nw);
+  if (kp == 0) return false;
+  if (kp > 1 && (N / 16) * 4 > 64 * 1024) return false;  // counters: one per group of row blocks
   return true;
 }
 
 int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const uint32_t* w,
                        const bf16_t* s, const bf16_t* b, const uint32_t* w2, const bf16_t* s2,
                        const bf16_t* b2, const bf16_t* residual, bf16_t* y, int M, int N, int K,
-                       hipStream_t st) {
+                       void* workspace, hipStream_t st) {
   W16Params p;
   p.x = x;
   p.norm_w = norm_w;
@@ -538,12 +616,21 @@ int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const u
   p.blocks = N / 16;
   p.ph = 1;
   p.lw = 64;
+  p.red_bytes = 0;
+  const bool pair = w2 != nullptr;
   int sl = 0, nw = 0;
-  if (!exo_qmv_w16_ok(M, N, K, 4, residual != nullptr) || !w16_shape(p.row_bytes, &sl, &nw)) {
+  const int kp = exo_qmv_w16_ok(M, N, K, 4, norm_w != nullptr, pair, workspace != nullptr)
+                     ? w16_parts(p.row_bytes, workspace && !norm_w && !pair, &sl, &nw)
+                     : 0;
+  if (kp == 0) {
     exo_set_error("exo_qmv: shape M=%d N=%d K=%d not covered by the 16x16x32 kernel", M, N, K);
     return EXO_ERR_ARG;
   }
-  const bool pair = w2 != nullptr;
+  p.kparts = kp;
+  p.Gp = p.G / kp;
+  // the workspace of the split-K GEMV: counters (64 KiB), then the float32 partial results
+  p.counters = reinterpret_cast<int*>(workspace);
+  p.part = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + 64 * 1024) : nullptr;
 #ifndef EXO_W16_DEPTH
 #define EXO_W16_DEPTH 2
 #endif
