@@ -302,7 +302,17 @@ def test_decode_launches_reach_their_instances(device):
     assert native.last_variant().startswith("qmv_quad<4,2,1,4,1>"), native.last_variant()
     x8 = t_bf16(rand_bf16((8, H), seed=5), device)
     ops.qmv_swiglu(x8, g, u, norm_weight=nw, eps=1e-5)
-    assert native.last_variant().startswith("qmv_mfma<4,4,"), native.last_variant()
+    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,staged> grid=256 waves=16 blocks=4"), native.last_variant()
+    x16 = t_bf16(rand_bf16((16, H), seed=7), device)
+    ops.qmv_swiglu(x16, g, u, norm_weight=nw, eps=1e-5)
+    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,direct>"), native.last_variant()
+    # the down projection under 8 rows: K split over four workgroups per group of row blocks
+    xi8 = t_bf16(rand_bf16((8, I), seed=8), device)
+    ops.quantized_matmul(xi8, _packed(H, I, bits, 4, device), residual=x8)
+    assert native.last_variant().startswith("qmv_w16<1,2,2,plain,staged> grid=256 waves=14 blocks=4 kparts=4"), \
+        native.last_variant()
+    ops.quantized_matmul(x8, _packed(6144, H, bits, 3, device), norm_weight=nw, eps=1e-5)
+    assert native.last_variant().startswith("qmv_w16<1,2,2,norm,staged>"), native.last_variant()
     # decode attention: one sequence of 32 / 8 heads on the scalar kernel, eight on the matrix cores
     D, Hq, Hkv, S = 128, 32, 8, 2304
     inv = torch.from_numpy(O.rope_inv_freq(D, 5e5, None)).to(device)

@@ -81,14 +81,14 @@ def test_qmv_launch_shapes(device, N, K, bits):
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("N,K", SWEEP_SHAPES)
 def test_qmatmul_sweep_shapes(device, bits, N, K):
-    """Every (N,K) of the qmatmul sweep at M = 1, 2, 3, 4, 16 (GEMV kernels), 24, 32 and 64
+    """Every (N,K) of the qmatmul sweep at M = 1, 2, 3, 4, 5, 8, 12, 16 (GEMV kernels), 24, 32 and 64
     (the 256-column GEMM tile with K split up to 16 ways) and 128 (128-row tile), plus M = 2048
     where the output stays small."""
     qw = _packed(N, K, bits, seed=N + K + bits, device=device)
     rows = np.unique(np.concatenate([[0, 1, N - 2, N - 1], np.random.default_rng(N + K).integers(0, N, 188)]))
     sub = _rows_np(qw, rows)
     wd = ops.dequantize(qw).float()            # [N,K]; bit-exact vs the oracle in its own test
-    for M in [1, 2, 3, 4, 16, 24, 32, 64, 128] + ([2048] if N <= 14336 else []):
+    for M in [1, 2, 3, 4, 5, 8, 12, 16, 24, 32, 64, 128] + ([2048] if N <= 14336 else []):
         x = rand_bf16((M, K), seed=M + K)
         xt = t_bf16(x, device)
         y = ops.quantized_matmul(xt, qw)
