@@ -25,6 +25,9 @@
 
 namespace {
 
+#ifndef EXO_W16_PAIR8
+#define EXO_W16_PAIR8 1  // the (gate, up) pair in blocks of 8 rows of both matrices where that fits
+#endif
 #ifndef EXO_W16_ABL
 #define EXO_W16_ABL 0  // timing-only ablations (wrong results): 1 no products, 2 no lane permutation, 4 no group epilogue, 8 no unpacking
 #endif
@@ -116,9 +119,18 @@ struct SbWord<2> {
 // the partial sums (up to 8 activation rows).
 // KSPLIT: K split over several workgroups (single matrix, no fused norm).  An instance of its
 // own: compiled into the others, the hand-over code costs them 0.5 us per launch untaken.
-template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false>
+// P8 (the (gate, up) pair as ONE operand block: NMAT == 1, staged scales): the 16 columns of a
+// product are 8 rows of the gate matrix and the same 8 rows of the up matrix.  A workgroup's
+// share is then counted in blocks of 8 rows of both - 14336 rows are 1792 blocks, seven for each
+// of 256 workgroups, where blocks of 16 rows leave half the workgroups with four and half with
+// three.  Per-lane addresses (two matrices in one load instruction), clamped to the
+// workgroup's last block instead of range-checked.
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false, bool P8 = false>
 __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
+  static_assert(!P8 || (NMAT == 1 && SBLDS && !KSPLIT), "pair-of-8 mode: one operand block, staged scales");
   constexpr bool KSPLIT_OK = KSPLIT && NMAT == 1 && !NORM;
+  constexpr int RPB = P8 ? 8 : 16;     // rows of a matrix per block
+  constexpr int NS = P8 ? 2 : NMAT;    // matrices with scales to stage
   extern __shared__ float red[];  // [ph][NMAT][nw][4][lw]
   __shared__ float s_part[16][16];
   __shared__ int s_last;
@@ -144,18 +156,24 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     SbWord<SL> s[NMAT], b[NMAT];
   };
   // buffer resources over exactly this workgroup's rows (a refill past them returns zeros)
-  __amdgpu_buffer_rsrc_t rw[NMAT], rs[NMAT], rb[NMAT];
+  __amdgpu_buffer_rsrc_t rw[NMAT], rs[NS], rb[NS];
 #pragma unroll
-  for (int a = 0; a < NMAT; ++a) {
+  for (int a = 0; a < NMAT; ++a)
     rw[a] = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<char*>(reinterpret_cast<const char*>(p.w[a]) + (size_t)q0 * 16 * p.row_bytes), 0,
-        nq * 16 * p.row_bytes, 0x00020000);
-    rs[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.s[a] + (size_t)q0 * 16 * p.G), 0,
-                                              nq * 16 * p.G * 2, 0x00020000);
-    rb[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.b[a] + (size_t)q0 * 16 * p.G), 0,
-                                              nq * 16 * p.G * 2, 0x00020000);
+        const_cast<char*>(reinterpret_cast<const char*>(p.w[a]) + (size_t)q0 * RPB * p.row_bytes), 0,
+        nq * RPB * p.row_bytes, 0x00020000);
+#pragma unroll
+  for (int a = 0; a < NS; ++a) {
+    rs[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.s[a] + (size_t)q0 * RPB * p.G), 0,
+                                              nq * RPB * p.G * 2, 0x00020000);
+    rb[a] = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.b[a] + (size_t)q0 * RPB * p.G), 0,
+                                              nq * RPB * p.G * 2, 0x00020000);
   }
   const int wofs = lr * p.row_bytes + g_first * 32 + wave * (SL * 64) + lc * 16;
+  // P8: this lane's row of its matrix (lanes of block rows 0..7: gate, 8..15: up), first block
+  const uint32_t* const w_mine = (P8 && lr >= 8) ? p.w[1] : p.w[0];
+  const char* const w_lane = reinterpret_cast<const char*>(w_mine) +
+                             (size_t)(q0 * RPB + (lr & (RPB - 1))) * p.row_bytes + wave * (SL * 64) + lc * 16;
   const int sofs = (j * p.G + g_first + wave * (SL * 2)) * 2;  // this lane's weight row, the wave's groups
   // PIN (the issues in front of the loop): the loads leave in program order - weights, then
   // scales and biases, buffer by buffer, as in the loop.  The compiler counts the loads still
@@ -164,22 +182,18 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   auto issue_w = [&](Buf& bf, int q, bool pin) {  // q: row block of this workgroup's range (past it: zeros)
     const int wq = q * 16 * p.row_bytes;  // uniform: scalar offset
     if (pin) __builtin_amdgcn_sched_barrier(0);
+    if constexpr (P8) {
+      const char* src = w_lane + (size_t)min(q, nq - 1) * (8 * p.row_bytes);
 #pragma unroll
-    for (int sl = 0; sl < SL; ++sl)
+      for (int sl = 0; sl < SL; ++sl) bf.w[0][sl] = *reinterpret_cast<const uint4*>(src + sl * 64);
+    } else {
 #pragma unroll
-      for (int a = 0; a < NMAT; ++a)
-#if (EXO_W16_ABL & 16)  // timing only: 8 rows x 128 bytes per instruction (SL == 2)
-        bf.w[a][sl] = __builtin_bit_cast(
-            uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                       rw[a], ((lane >> 3) + 8 * sl) * p.row_bytes + wave * (SL * 64) + (lane & 7) * 16, wq, 0));
-#elif (EXO_W16_ABL & 32)  // timing only: 4 rows x 256 bytes per instruction, two waves share 256 bytes
-        bf.w[a][sl] = __builtin_bit_cast(
-            uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                       rw[a], ((lane >> 4) + 4 * sl + 8 * (wave & 1)) * p.row_bytes + (wave >> 1) * 256 + (lane & 15) * 16, wq, 0));
-#else
-        bf.w[a][sl] = __builtin_bit_cast(
-            uint4, __builtin_amdgcn_raw_buffer_load_b128(rw[a], wofs + sl * 64, wq, 0));
-#endif
+      for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a)
+          bf.w[a][sl] = __builtin_bit_cast(
+              uint4, __builtin_amdgcn_raw_buffer_load_b128(rw[a], wofs + sl * 64, wq, 0));
+    }
     if (pin) __builtin_amdgcn_sched_barrier(0);
   };
   auto issue_sb = [&](Buf& bf, int q, bool pin) {
@@ -205,8 +219,8 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   // staged scales / biases: array (matrix a, scale|bias) x local row x (G + 4) bf16 (rows
   // padded by 8 bytes: the 16 rows a wave reads at once then sit in different banks)
   char* const sb_lds = reinterpret_cast<char*>(red) + p.red_bytes;
-  const int sb_row = p.Gp * 2 + 8, sb_arr = p.ph * 16 * sb_row;
-  char* const nw_lds = sb_lds + (SBLDS ? NMAT * 2 * sb_arr : 0);  // the norm weights, K bf16
+  const int sb_row = p.Gp * 2 + 8, sb_arr = p.ph * RPB * sb_row;
+  char* const nw_lds = sb_lds + (SBLDS ? NS * 2 * sb_arr : 0);  // the norm weights, K bf16
 
   // ---- activations: lane (m = j, kg) holds, for product (sl, g, h), the 8 elements of row m
   // that the weight word of lane (., kg) covers: word 4*(2g + kg%2) + 2h + kg/2 of the slice
@@ -229,13 +243,13 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     // registers are live across the barrier beside everything else)
     uint4 nstg = make_uint4(0, 0, 0, 0);
     if (NORM) nstg = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rn, tid * 16, 0, 0));
-    uint4 stg[NMAT][2];
+    uint4 stg[NS][2];
     if (SBLDS) {
       // thread -> (local row, 16-byte chunk of the row's part); past the rows: out of range
       const int cpr = p.Gp >> 3, row = tid / cpr, col = tid - row * cpr;
-      const int so = row < nq * 16 ? (row * p.G + g_first) * 2 + col * 16 : 0x7ffffff0;
+      const int so = row < nq * RPB ? (row * p.G + g_first) * 2 + col * 16 : 0x7ffffff0;
 #pragma unroll
-      for (int a = 0; a < NMAT; ++a) {
+      for (int a = 0; a < NS; ++a) {
         stg[a][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs[a], so, 0, 0));
         stg[a][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[a], so, 0, 0));
       }
@@ -255,12 +269,12 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
     // outstanding loads
 #pragma unroll
     for (int d = 0; d < (NORM ? 1 : DEPTH); ++d) issue(buf[d], d, true);
-    auto stage_sb = [&](const uint4 (&v)[NMAT][2]) {
+    auto stage_sb = [&](const uint4 (&v)[NS][2]) {
       const int cpr = p.Gp >> 3;  // 16-byte chunks per row
       const int row = tid / cpr, col = tid - row * cpr;
-      if (row < nq * 16) {
+      if (row < nq * RPB) {
 #pragma unroll
-        for (int a = 0; a < NMAT; ++a)
+        for (int a = 0; a < NS; ++a)
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
             uint2* dst = reinterpret_cast<uint2*>(sb_lds + (a * 2 + t) * sb_arr + row * sb_row + col * 16);
@@ -383,7 +397,11 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
 #endif
           }
           uint32_t sw, bwd;
-          if (SBLDS) {
+          if (P8) {  // this lane's column: row jl % 8 of the gate (jl < 8) or the up matrix
+            const char* base = sb_lds + (slot * 8 + (jl & 7)) * sb_row + (wave * SL + sl) * 4 + (jl >> 3) * 2 * sb_arr;
+            sw = *reinterpret_cast<const uint32_t*>(base);
+            bwd = *reinterpret_cast<const uint32_t*>(base + sb_arr);
+          } else if (SBLDS) {
             const char* base = sb_lds + (slot * 16 + jl) * sb_row + (wave * SL + sl) * 4;
             sw = *reinterpret_cast<const uint32_t*>(base + (a * 2) * sb_arr);
             bwd = *reinterpret_cast<const uint32_t*>(base + (a * 2 + 1) * sb_arr);
@@ -416,6 +434,22 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
   // the phase's results: sum over the waves in a fixed order, epilogue, store
   auto finish_phase = [&](int q_first, int n, bool res) {
     __syncthreads();
+    if constexpr (P8) {
+      for (int idx = tid; idx < n * p.M * 8; idx += (int)blockDim.x) {
+        const int jj = idx & 7, m = (idx >> 3) % p.M, slot = (idx >> 3) / p.M;
+        const float* src = &red[(((size_t)slot * nw * 4) + (m & 3)) * lw + (m >> 2) * 16 + jj];
+        float tg = 0.f, tu = 0.f;
+        for (int w = 0; w < nw; ++w) {
+          tg += src[(size_t)w * 4 * lw];
+          tu += src[(size_t)w * 4 * lw + 8];
+        }
+        // SwiGLU on the bf16-rounded projections
+        const float g = bf2f(f2bf(tg)), up = bf2f(f2bf(tu));
+        p.y[(size_t)m * p.N + (q0 + q_first + slot) * 8 + jj] = f2bf(g / (1.f + __expf(-g)) * up);
+      }
+      __syncthreads();
+      return;
+    }
     for (int idx = tid; idx < n * p.M * 16; idx += (int)blockDim.x) {
       const int jj = idx & 15, m = (idx >> 4) % p.M, slot = (idx >> 4) / p.M;
       const int src_lane = (m >> 2) * 16 + jj, r = m & 3;
@@ -490,15 +524,18 @@ __global__ __launch_bounds__(1024) void qmv_w16_kernel(const W16Params p) {
 
 constexpr size_t kLdsBudget = 144 * 1024;  // LDS for partial sums and staged scales (the norm weights: 8 KB more)
 
-template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false>
+template <int NMAT, int SL, int DEPTH, bool NORM, bool SBLDS, bool KSPLIT = false, bool P8 = false>
 int launch_w16s(W16Params p, int nw, hipStream_t st) {
-  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM, SBLDS, KSPLIT>;
+  auto kern = qmv_w16_kernel<NMAT, SL, DEPTH, NORM, SBLDS, KSPLIT, P8>;
+  constexpr int RPB = P8 ? 8 : 16, NS = P8 ? 2 : NMAT;
+  p.blocks = p.N / RPB;
   p.lw = 16 * ((p.M + 3) / 4);
   const size_t per_block = (size_t)NMAT * nw * 4 * p.lw * sizeof(float);
-  const size_t sb_block = SBLDS ? (size_t)NMAT * 2 * 16 * (p.Gp * 2 + 8) : 0;
+  const size_t sb_block = SBLDS ? (size_t)NS * 2 * RPB * (p.Gp * 2 + 8) : 0;
   int ph = (int)(kLdsBudget / (per_block + sb_block));  // row blocks a workgroup can hold
   // staging: one 16-byte chunk per thread and array
-  if (SBLDS && ph > 32 * nw / p.Gp) ph = 32 * nw / p.Gp;
+  const int stage_max = 64 * nw / (RPB * (p.Gp / 8));
+  if (SBLDS && ph > stage_max) ph = stage_max;
   if (ph < 1) {
     exo_set_error("exo_qmv: internal: no LDS for one row block (M=%d K=%d)", p.M, p.K);
     return EXO_ERR_ARG;
@@ -524,8 +561,8 @@ int launch_w16s(W16Params p, int nw, hipStream_t st) {
     }
     attr_done = true;
   }
-  exo_note_variant("qmv_w16<%d,%d,%d,%s,%s> grid=%d waves=%d blocks=%d kparts=%d", NMAT, SL, DEPTH,
-                   NORM ? "norm" : "plain", SBLDS ? "staged" : "direct", grid, nw, nq, p.kparts);
+  exo_note_variant("qmv_w16<%d,%d,%d,%s,%s> grid=%d waves=%d blocks=%d kparts=%d", P8 ? 2 : NMAT, SL, DEPTH,
+                   NORM ? "norm" : "plain", P8 ? "pair8" : (SBLDS ? "staged" : "direct"), grid, nw, nq, p.kparts);
   kern<<<dim3(grid), dim3(64 * nw), lds, st>>>(p);
   return EXO_OK;
 }
@@ -538,6 +575,19 @@ int launch_w16(const W16Params& p, int nw, hipStream_t st) {
   const size_t need1 = ((size_t)NMAT * nw * 4 * 16 * ((p.M + 3) / 4) * sizeof(float) +
                         (size_t)NMAT * 2 * 16 * (p.Gp * 2 + 8)) * nq1;
   const bool staged = p.Gp % 8 == 0 && need1 <= kLdsBudget && nq1 <= 32 * nw / p.Gp && !(EXO_W16_ABL & 128);
+  if constexpr (NMAT == 2) {
+    // the pair in blocks of 8 rows of both matrices where their share of one round of 256
+    // workgroups fits the LDS with staged scales: 14336 rows are seven such blocks per
+    // workgroup, against four or three blocks of 16 rows (8 activation rows: 20.4 -> us)
+    const int blocks8 = p.N / 8, g8 = blocks8 < 256 ? blocks8 : 256, nq8 = (blocks8 + g8 - 1) / g8;
+    const size_t need8 = ((size_t)nw * 4 * 16 * ((p.M + 3) / 4) * sizeof(float) +
+                          (size_t)2 * 2 * 8 * (p.Gp * 2 + 8)) * nq8;
+    if (p.N % 8 == 0 && p.Gp % 8 == 0 && need8 <= kLdsBudget && nq8 <= 64 * nw / (8 * (p.Gp / 8)) &&
+        EXO_W16_PAIR8) {
+      return p.norm_w ? launch_w16s<1, SL, DEPTH, true, true, false, true>(p, nw, st)
+                      : launch_w16s<1, SL, DEPTH, false, true, false, true>(p, nw, st);
+    }
+  }
   if (p.kparts > 1) {
     if constexpr (NMAT == 1)
       return staged ? launch_w16s<1, SL, DEPTH, false, true, true>(p, nw, st)
@@ -613,7 +663,7 @@ int exo_qmv_w16_launch(const bf16_t* x, const bf16_t* norm_w, float eps, const u
   p.K = K;
   p.row_bytes = K / 2;
   p.G = K / 64;
-  p.blocks = N / 16;
+  p.blocks = N / 16;  // (the launcher sets the count for its block size)
   p.ph = 1;
   p.lw = 64;
   p.red_bytes = 0;

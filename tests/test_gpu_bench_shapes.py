@@ -302,10 +302,10 @@ def test_decode_launches_reach_their_instances(device):
     assert native.last_variant().startswith("qmv_quad<4,2,1,4,1>"), native.last_variant()
     x8 = t_bf16(rand_bf16((8, H), seed=5), device)
     ops.qmv_swiglu(x8, g, u, norm_weight=nw, eps=1e-5)
-    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,staged> grid=256 waves=16 blocks=4"), native.last_variant()
+    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,pair8> grid=256 waves=16 blocks=7"), native.last_variant()
     x16 = t_bf16(rand_bf16((16, H), seed=7), device)
     ops.qmv_swiglu(x16, g, u, norm_weight=nw, eps=1e-5)
-    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,direct>"), native.last_variant()
+    assert native.last_variant().startswith("qmv_w16<2,2,2,norm,pair8> grid=256 waves=16 blocks=7"), native.last_variant()
     # the down projection under 8 rows: K split over four workgroups per group of row blocks
     xi8 = t_bf16(rand_bf16((8, I), seed=8), device)
     ops.quantized_matmul(xi8, _packed(H, I, bits, 4, device), residual=x8)
