@@ -121,6 +121,49 @@ def test_qmv_swiglu(device, bits, M):
     assert_close(got, want, what="qmv_swiglu")
 
 
+W16_SHAPES = [  # (N, K): rows of 6 | 8 | 14 | 16 waves x 1 | 2 slices, K split 2 | 4 ways
+    (4112, 768), (2064, 1024), (1008, 2560), (1040, 3584), (528, 4096), (272, 8192), (304, 14336),
+]
+
+
+@pytest.mark.parametrize("N,K", W16_SHAPES)
+@pytest.mark.parametrize("M", [5, 8, 11, 16])
+def test_qmv_16x16x32_kernel_shapes(device, N, K, M):
+    """The 16x16x32 matrix-core GEMV (4-bit, 5..16 rows) over its wave /
+    slice layouts: plain, with residual, with the fused RMSNorm (rows of up to 4096 elements),
+    and the (gate, up) pair with SwiGLU; every result against the oracle, every launch asserted
+    to have reached that kernel."""
+    bits = 4
+    trip = rand_quantized(N, K, bits, seed=N + K)
+    qw = t_qw(trip, bits, device)
+    x = rand_bf16((M, K), seed=M + K, scale=1.5)
+    xt = t_bf16(x, device)
+    want = affine.qmm(x, *trip, 64, bits)
+    got = ops.quantized_matmul(xt, qw)
+    assert native.last_variant().startswith("qmv_w16<1,"), native.last_variant()
+    if K > 4096:
+        assert "kparts=1" not in native.last_variant(), native.last_variant()
+    assert_close(n_f32(got), want, what=f"w16 {M}x{N}x{K}")
+    r = rand_bf16((M, N), seed=N + 3)
+    got = ops.quantized_matmul(xt, qw, residual=t_bf16(r, device))
+    assert native.last_variant().startswith("qmv_w16<1,"), native.last_variant()
+    assert_close(n_f32(got), affine.bf16_round(affine.bf16_round(want) + r), what=f"w16 residual {M}x{N}x{K}")
+    # the split-K workspace is left clean: the same launch again gives the same bits
+    again = ops.quantized_matmul(xt, qw, residual=t_bf16(r, device))
+    assert torch.equal(got.view(torch.int16), again.view(torch.int16))
+    if K <= 4096:
+        w = affine.bf16_round(rand_bf16((K,), seed=6) * 0.1 + 1.0)
+        xn = O.rms_norm(x, w, 1e-5)
+        got = ops.quantized_matmul(xt, qw, norm_weight=t_bf16(w, device), eps=1e-5)
+        assert native.last_variant().startswith("qmv_w16<1,") and "norm" in native.last_variant(), native.last_variant()
+        assert_close(n_f32(got), affine.qmm(xn, *trip, 64, bits), what=f"w16 norm {M}x{N}x{K}")
+        up = rand_quantized(N, K, bits, seed=N + K + 1)
+        got = ops.qmv_swiglu(xt, qw, t_qw(up, bits, device), norm_weight=t_bf16(w, device), eps=1e-5)
+        assert native.last_variant().startswith("qmv_w16<2,"), native.last_variant()
+        assert_close(n_f32(got), O.swiglu(affine.qmm(xn, *trip, 64, bits), affine.qmm(xn, *up, 64, bits)),
+                     what=f"w16 pair {M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("M,N,K", [(8, 1000, 4096), (3, 96, 14336), (16, 2080, 2048), (5, 14336, 512)])
 def test_qmv_swiglu_rows_equal_separate_launches(device, bits, M, N, K):
