@@ -1188,7 +1188,10 @@ struct DownCombineParams {
 constexpr int kDownMaxIters = 4;  // 16-byte chunks per lane and expert row
 constexpr int kDownMaxTopk = 8;
 
-template <int BITS, int kDownRW>
+// ITERS: 16-byte chunks per lane and row, a template parameter so that no weight load sits
+// behind a branch (a value loaded behind one is waited for where the branches join, in front
+// of the loads of the following rows)
+template <int BITS, int kDownRW, int ITERS>
 __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
     const DownCombineParams p) {
   extern __shared__ uint4 smem[];
@@ -1211,9 +1214,20 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
   e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // memory safety only: the host rejects such ids
   const float score = bf2f(p.scores[(size_t)t * p.topk + slot]);
 
-  // every weight load of this wave goes out first
-  uint4 wv[kDownRW][kDownMaxIters];
-  bf16_t sv[kDownRW][kDownMaxIters], bv[kDownRW][kDownMaxIters];
+  // The first 256 words of this slot's activation row are requested first (they sit in L2 and
+  // are waited for with the weight loads still in flight - loads return in order), then every
+  // weight load of the wave, then the row is staged: word wi -> xs[(j*4 + w4) * LPR + sl] in
+  // dot2 order, per-chunk sums to sx[chunk]; four consecutive lanes hold one chunk
+  const bf16_t* xt = p.x + ((size_t)t * p.topk + slot) * p.K;
+  uint4 raw0[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) raw0[u] = load_word_x<BITS>(xt, min(u * 64 + lane, p.wpr - 1));
+  __builtin_amdgcn_sched_barrier(0);  // (left alone, the compiler moves these behind the weight loads)
+  uint4 wv[kDownRW][ITERS];
+  // (scale, bias): one 32-bit register each - held as 16-bit values the compiler packs two of
+  // them into a register and waits for each pair right behind its loads, so that a row's loads
+  // went out only once the previous row's scales had arrived
+  uint32_t sv[kDownRW][ITERS], bv[kDownRW][ITERS];
 #pragma unroll
   for (int i = 0; i < kDownRW; ++i) {
     const int row = min(row0 + i * rpwi + sub, p.N - 1);  // rows past N: not stored
@@ -1222,23 +1236,19 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
     const bf16_t* sp = p.s + r * G + (sl >> GSHIFT);
     const bf16_t* bp = p.b + r * G + (sl >> GSHIFT);
 #pragma unroll
-    for (int j = 0; j < kDownMaxIters; ++j)
-      if (j < p.iters) {
-        wv[i][j] = *reinterpret_cast<const uint4*>(wp + (size_t)j * lpr * 4);
-        sv[i][j] = sp[j * (lpr >> GSHIFT)];
-        bv[i][j] = bp[j * (lpr >> GSHIFT)];
-      }
+    for (int j = 0; j < ITERS; ++j) {
+      wv[i][j] = *reinterpret_cast<const uint4*>(wp + (size_t)j * lpr * 4);
+      sv[i][j] = sp[j * (lpr >> GSHIFT)];
+      bv[i][j] = bp[j * (lpr >> GSHIFT)];
+    }
   }
 
-  // stage this slot's activation row: word wi -> xs[(j*4 + w4) * LPR + sl] in dot2 order,
-  // per-chunk sums to sx[chunk]; four consecutive lanes hold one chunk
   {
-    const bf16_t* xt = p.x + ((size_t)t * p.topk + slot) * p.K;
     for (int base = 0; base < p.wpr; base += 64 * 4) {
       uint4 raw[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        raw[u] = load_word_x<BITS>(xt, min(base + u * 64 + lane, p.wpr - 1));
+        raw[u] = base == 0 ? raw0[u] : load_word_x<BITS>(xt, min(base + u * 64 + lane, p.wpr - 1));
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int wi = base + u * 64 + lane;
@@ -1269,8 +1279,7 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
   for (int i = 0; i < kDownRW; ++i) {
     float acc = 0.f;
 #pragma unroll
-    for (int j = 0; j < kDownMaxIters; ++j)
-      if (j < p.iters) {
+    for (int j = 0; j < ITERS; ++j) {
         const float2 sm = sx[(j << p.lpr_log2) + sl];
         float d = -sm.x;
 #pragma unroll
@@ -1283,8 +1292,8 @@ __global__ __launch_bounds__(64 * kDownMaxTopk) void moe_down_combine_kernel(
           d = dot2_bf16(pr[2], xv.z, d);
           d = dot2_bf16(pr[3], xv.w, d);
         }
-        acc = fmaf(bf2f(sv[i][j]), d, acc);
-        acc = fmaf(bf2f(bv[i][j]), sm.y, acc);
+        acc = fmaf(bf_lo(sv[i][j]), d, acc);
+        acc = fmaf(bf_lo(bv[i][j]), sm.y, acc);
       }
     acc = group_sum(acc, lpr);
     if (sl == 0) contrib[slot][i * rpwi + sub] = bf2f(f2bf(bf2f(f2bf(acc)) * score));
@@ -1994,18 +2003,18 @@ extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, cons
   const int rw = exo_ceil_div(N, 2 * rpwi) >= 512 ? 2 : 1;
   const dim3 grid(exo_ceil_div(N, rw * rpwi), T);
   const size_t lds = (size_t)topk * ((size_t)p.wpr * 16 + (size_t)(p.wpr / 4) * 8);
-  exo_note_variant("moe_down_combine<%d,%d> grid=%dx%d", bits, rw, (int)grid.x, (int)grid.y);
-  if (bits == 4) {
-    if (rw == 2)
-      moe_down_combine_kernel<4, 2><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
-    else
-      moe_down_combine_kernel<4, 1><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
-  } else {
-    if (rw == 2)
-      moe_down_combine_kernel<8, 2><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
-    else
-      moe_down_combine_kernel<8, 1><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
-  }
+  exo_note_variant("moe_down_combine<%d,%d,%d> grid=%dx%d", bits, rw, pl.iters, (int)grid.x, (int)grid.y);
+#define EXO_DOWN_CASE(B_, RW_, IT_)                                                       \
+  if (bits == B_ && rw == RW_ && pl.iters == IT_)                                          \
+    moe_down_combine_kernel<B_, RW_, IT_><<<grid, 64 * topk, lds, (hipStream_t)stream>>>(p);
+#define EXO_DOWN_ITERS(B_, RW_) \
+  EXO_DOWN_CASE(B_, RW_, 1) EXO_DOWN_CASE(B_, RW_, 2) EXO_DOWN_CASE(B_, RW_, 3) EXO_DOWN_CASE(B_, RW_, 4)
+  EXO_DOWN_ITERS(4, 1)
+  EXO_DOWN_ITERS(4, 2)
+  EXO_DOWN_ITERS(8, 1)
+  EXO_DOWN_ITERS(8, 2)
+#undef EXO_DOWN_ITERS
+#undef EXO_DOWN_CASE
   EXO_CHECK_LAUNCH("exo_gather_qmv_combine");
   return EXO_OK;
 }
