@@ -117,8 +117,10 @@ __device__ __forceinline__ uint4 permute_word(const uint4& xv, float& stored, fl
   return o;
 }
 
-template <int MT, int ITERS, int NMAT>
-constexpr bool kRowsXR = (MT == 1 && ITERS <= 2 && NMAT == 1);
+// (ROUTE: the (gate, up) pair of a routed expert - two rows per wave or so, where a
+// workgroup-wide staging with its barriers costs more than four waves normalising alike)
+template <int MT, int ITERS, int NMAT, bool ROUTE = false>
+constexpr bool kRowsXR = (MT == 1 && ITERS <= 2 && (NMAT == 1 || ROUTE));
 
 template <int BITS>
 __device__ __forceinline__ uint4 load_word_x(const bf16_t* base, int wi) {
@@ -541,10 +543,26 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // Base pointers of this workgroup's matrices.  Gather modes: the expert of its pair.
   // Routing mode: wave 0 repeats the routing of the token, the others wait at one barrier;
   // called once the activation loads are on their way, so that their latency covers it.
+  // In the register-resident layout every wave repeats it from logits it requested first
+  // (route_raw): no barrier at all.
+  constexpr bool XR = kRowsXR<MT, ITERS, NMAT, ROUTE>;
   __shared__ int s_expert;
+  uint32_t route_raw[4] = {0, 0, 0, 0};
   auto select_matrices = [&]() {
     size_t ew = 0, eg = 0;
-    if (ROUTE && p.route) {
+    if (ROUTE && XR && p.route) {
+      const int t = pair / p.topk, slot = pair - t * p.topk;
+      int my_id;
+      float my_p, tot;
+      route_topk_regs(route_raw, p.E, p.topk, lane, my_id, my_p, tot);
+      if (blockIdx.x == 0 && slot == 0 && wave == 0 && lane < p.topk) {
+        p.route_idx[(size_t)t * p.topk + lane] = my_id;
+        p.route_scores[(size_t)t * p.topk + lane] = route_score(my_p, tot, p.route_renorm);
+      }
+      const int e = __builtin_amdgcn_readlane(my_id, slot);
+      ew = (size_t)e * p.N * p.wpr;
+      eg = (size_t)e * p.N * G;
+    } else if (ROUTE && p.route) {
       const int t = pair / p.topk, slot = pair - t * p.topk;
       if (wave == 0) {
         int my_id;
@@ -620,7 +638,6 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // XR: a single activation row whose share per lane (ITERS * 64 bytes) fits in
   // registers.  Every wave then holds the whole row across its lanes: no LDS, no
   // barrier, and the fused RMSNorm needs only a wave reduction.
-  constexpr bool XR = kRowsXR<MT, ITERS, NMAT>;
   uint4 xr[XR ? ITERS : 1][4];
   float2 sxr[XR ? ITERS : 1];
   int xlane = lane;
@@ -713,18 +730,28 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
   // the weight loads still outstanding), then two weight batches, then the LDS staging.
   Batch buf[NBUF];
   if (XR) {
-    if (nrows <= 0 && !(ROUTE && p.route)) return;  // (routing mode: every wave meets the barrier)
+    if (nrows <= 0) return;  // (wave 0 of a workgroup, which records the routing, always has rows)
+    // (no branch, so that the order of the requests below is the order written: launched
+    // with expert ids instead of logits, the instance loads one activation in their place)
+    if (ROUTE) {
+      route_load(p.route ? p.route + (size_t)(pair / p.topk) * p.E : xin, p.route ? p.E : 1, lane, route_raw);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     uint4 raw[ITERS][4], nwv[ITERS][4];
+    // without a norm the weight words are loaded from the activations and not used: a
+    // branch per load would split the requests over basic blocks
+    const bf16_t* nw_src = p.norm_w ? p.norm_w : xin;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j)
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int wi = 4 * chunk_of<BITS, ITERS>(j, lane) + t;
         raw[j][t] = load_word_x<BITS>(xin, wi);
-        if (p.norm_w) nwv[j][t] = load_word_x<BITS>(p.norm_w, wi);
+        nwv[j][t] = load_word_x<BITS>(nw_src, wi);
       }
+    // (the routing waits for its logits only: the activation loads above go out before that wait)
+    if (ROUTE) __builtin_amdgcn_sched_barrier(0);
     select_matrices();
-    if (nrows <= 0) return;
     issue(buf[0], r0);
     if (p.norm_w) {
       float ss = 0.f;
@@ -755,7 +782,9 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
     // the second batch only now: the raw activations and norm weights are dead, so
     // the register peak stays at what the main loop needs
     asm volatile("" ::: "memory");
-    if (nrows > R) issue(buf[1], r0 + R);
+#pragma unroll
+    for (int b = 1; b < NBUF; ++b)
+      if (nrows > b * R) issue(buf[b], r0 + b * R);
   } else {
     XStage<BITS, MT, ITERS> xst;
     stage_x_load<BITS, MT, ITERS>(p, xin, xst);
@@ -1345,10 +1374,15 @@ bool make_plan(int N, int K, int bits, int mt, Plan* pl) {
   return true;
 }
 
+#ifndef EXO_QMV_GATHER_WGS  // tuning builds: workgroups of a gather launch in all
+#define EXO_QMV_GATHER_WGS 0
+#endif
 template <int BITS, int MT, int NMAT, int ITERS>
 int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   constexpr bool CAN_ROUTE = MT == 1 && NMAT == 2;
-  const bool route = CAN_ROUTE && p.route;
+  // (the routing instance also takes the launches with given expert ids: one arithmetic for
+  // both, so routing inside the launch changes no bit of the result)
+  const bool route = CAN_ROUTE && (p.route || p.idx);
   auto kern = route ? qmv_rows_kernel<BITS, MT, NMAT, ITERS, CAN_ROUTE>
                     : qmv_rows_kernel<BITS, MT, NMAT, ITERS, false>;
   static bool attr_set[2] = {false, false};
@@ -1386,12 +1420,16 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   if (grid > max_grid) grid = max_grid;
   if (pairs > 1 && !p.each_row) {  // (rows of one small matrix keep the single-row grid)
     // gather mode (one launch covers `pairs` (token, slot) products, blockIdx.y each): every
-    // workgroup stages and normalises its token's activations first, so two rows per wave
-    // at least, and about 1536 workgroups in all.  Measured, workgroups per pair: 768x2048
-    // 4-bit (gate, up), 8 pairs: 192 7.3 us, 96 6.3, 64 6.4, 48 6.7; 32 pairs: 192 19.1 us,
-    // 96 14.4, 48 12.9, 32 13.4; 1536x4096 8-bit, 8 pairs: 384 25.0 us, 192 22.2, 128 22.9.
+    // wave normalises its token's activations first, so two rows per wave at least, and a
+    // grid that is resident at once (three workgroups per CU at this kernel's registers).
+    // Measured in the whole decode step, workgroups in all -> tokens/s: 768x2048 4-bit
+    // (gate, up), 8 pairs: 256 624, 384 628, 512 643, 768 627, 1536 (one row per wave) 551;
+    // 16 pairs: 512 966, 768 973, 1024 944, 1536 957; 32 pairs: 256 1289, 512 1385, 768 1384,
+    // 1536 1400; 64 pairs: 512 2050, 768 2074, 1536 2064; 128 pairs: 512 2814, 768 2956,
+    // 1536 2891; 1536x4096, 8 pairs: 512 480, 768 482, 1024 480, 1536 471.
+    const int wgs = EXO_QMV_GATHER_WGS > 0 ? EXO_QMV_GATHER_WGS : ((pairs <= 8 && ITERS == 1) ? 512 : 768);
+    const int share = wgs / pairs < 1 ? 1 : wgs / pairs;
     const int two_rows = (p.N + 2 * kWaves - 1) / (2 * kWaves);
-    const int share = 1536 / pairs < 1 ? 1 : 1536 / pairs;
     grid = two_rows < share ? two_rows : share;
   }
   if (single) {
@@ -1421,7 +1459,8 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   if (grid < 1) grid = 1;
   exo_note_variant("qmv_rows<%d,%d,%d,%d,%s> grid=%dx%d", BITS, MT, NMAT, ITERS, route ? "true" : "false",
                    grid, pairs);
-  kern<<<dim3(grid, pairs), dim3(kThreads), kRowsXR<MT, ITERS, NMAT> ? 0 : pl.lds, st>>>(p);
+  const bool in_regs = route ? kRowsXR<MT, ITERS, NMAT, CAN_ROUTE> : kRowsXR<MT, ITERS, NMAT>;
+  kern<<<dim3(grid, pairs), dim3(kThreads), in_regs ? 0 : pl.lds, st>>>(p);
   return EXO_OK;
 }
 

@@ -45,14 +45,24 @@ __device__ __forceinline__ float wave_sum_uniform(float v) {
 // selection finds the largest probability and, among equals, the lowest expert id; a
 // taken key becomes 0.  On return lane j < k holds the expert id and the probability of
 // the j-th selection (descending), `tot` the sum of the k probabilities in every lane.
-__device__ __forceinline__ void route_topk_wave(const bf16_t* __restrict__ logits, int E, int k,
-                                                int lane, int& my_id, float& my_p, float& tot) {
+// The logits of one token as raw 16-bit patterns, lane l holding experts l, l + 64, l + 128 and
+// l + 192.  Unconditional loads (indices past E re-read the last logit, dropped afterwards) into
+// 32-bit registers: the four requests go out back to back and one wait covers them.
+__device__ __forceinline__ void route_load(const bf16_t* __restrict__ logits, int E, int lane,
+                                           uint32_t (&raw)[4]) {
+  const uint16_t* l16 = reinterpret_cast<const uint16_t*>(logits);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) raw[i] = l16[min(lane + 64 * i, E - 1)];
+}
+
+__device__ __forceinline__ void route_topk_regs(const uint32_t (&raw)[4], int E, int k, int lane,
+                                                int& my_id, float& my_p, float& tot) {
   float v[4];
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int e = lane + 64 * i;
-    v[i] = (e < E) ? bf2f(logits[e]) : -INFINITY;
+    v[i] = (e < E) ? __builtin_bit_cast(float, raw[i] << 16) : -INFINITY;
     mx = fmaxf(mx, v[i]);
   }
   mx = wave_max_f32_uniform(mx);
@@ -87,6 +97,13 @@ __device__ __forceinline__ void route_topk_wave(const bf16_t* __restrict__ logit
       my_p = bv;
     }
   }
+}
+
+__device__ __forceinline__ void route_topk_wave(const bf16_t* __restrict__ logits, int E, int k,
+                                                int lane, int& my_id, float& my_p, float& tot) {
+  uint32_t raw[4];
+  route_load(logits, E, lane, raw);
+  route_topk_regs(raw, E, k, lane, my_id, my_p, tot);
 }
 
 // score of a selection as the block uses it: the probability, or (renorm) the probability
