@@ -58,6 +58,7 @@ def measure_kernels(model, torch, reps: int = 20):
     is served from cache) is captured into a HIP graph and timed with events on the
     launch stream; average launch duration = elapsed / launches."""
     from exo_amd import ops
+    from exo_amd.model import capture_graph
 
     c = model.cfg
     dev = model.device
@@ -92,7 +93,7 @@ def measure_kernels(model, torch, reps: int = 20):
             fn(L)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with capture_graph(g):
             for L in model.layers:
                 fn(L)
         g.replay()
@@ -118,7 +119,7 @@ def measure_kernels(model, torch, reps: int = 20):
         ops.quantized_matmul(xh, q, out=y_v, norm_weight=nw, eps=eps)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with capture_graph(g):
         for q in heads:
             ops.quantized_matmul(xh, q, out=y_v, norm_weight=nw, eps=eps)
     g.replay()
@@ -313,6 +314,7 @@ def qmatmul_sweep(args):
     import torch
 
     from exo_amd import native, ops
+    from exo_amd.model import capture_graph
     from exo_amd.ops import QuantizedWeight
 
     native.load()
@@ -340,7 +342,7 @@ def qmatmul_sweep(args):
                     f()
                 torch.cuda.synchronize()
                 gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr):
+                with capture_graph(gr):
                     for f in fns:
                         f()
                 gr.replay()

@@ -17,6 +17,8 @@ prefill attention.
 
 from __future__ import annotations
 
+import contextlib
+import gc
 import math
 
 import torch
@@ -27,6 +29,23 @@ from .config import ModelConfig
 from .ops import QuantizedWeight
 
 GEMV_MAX_ROWS = ops.QMV_MAX_M
+
+
+@contextlib.contextmanager
+def capture_graph(graph: "torch.cuda.CUDAGraph"):
+    """``torch.cuda.graph(graph)`` with Python's garbage collector held off while the stream
+    records: a collected object that owns pinned host memory, an event or another graph makes
+    runtime calls in its destructor that a recording stream does not allow, and the process
+    aborts.  Garbage is collected once before the recording starts."""
+    gc.collect()
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if was_on:
+            gc.enable()
 
 
 def rope_inv_freq(cfg: ModelConfig) -> torch.Tensor:
@@ -224,10 +243,12 @@ class ShardModel:
         else:
             ops.quantized_matmul(bf.n, L.router, out=bf.router_logits)
         k = c.num_experts_per_tok
-        if R == 1 and c.num_experts <= 256 and k <= 16:
-            # one sequence: the gate/up launch routes by itself (first wave of every workgroup),
-            # one launch fewer per layer: Qwen3-30B 543 -> 574 tok/s.  (Batch 4: 1277 -> 1261,
-            # the routing then delays 1536 workgroups in two rounds - separate launch kept.)
+        if gemv and c.num_experts <= 256 and k <= 16:
+            # decode: the gate/up launch routes by itself (every wave repeats the top-k of its
+            # token from the logits), one launch fewer per layer.  Qwen3-30B, separate top-k
+            # launch -> routing inside: batch 1 543 -> 574 tok/s on the build that introduced
+            # it; 2 rows 973 -> 1025, 4 rows 1399 -> 1455, 8 rows 2115 -> 2178, 16 rows
+            # 2987 -> 3050 on the current one.
             idx, sc, _ = ops.route_gather_qmv_swiglu(
                 bf.h, bf.router_logits, k, c.norm_topk_prob, L.gate, L.up, out=bf.act,
                 norm_weight=L.post_norm, eps=c.rms_norm_eps)
@@ -395,7 +416,7 @@ class ShardModel:
                 if sampler is not None:
                     sampler.restore(saved_sampler)
                 g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
+                with capture_graph(g):
                     body()
                 cache.pos.copy_(saved)
                 self._graphs[key] = (g, cache, sampler)
