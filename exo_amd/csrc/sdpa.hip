@@ -833,6 +833,9 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
       for (int e = 0; e < 8; ++e) sincosf(fpos * p.inv_freq[(sl * 8 + e) % (D / 2)], &sn[e], &cs[e]);
     }
     const bf16_t* row = p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
+#if (EXO_SDPA_ABL & 8)  // timing only: no table, no rotation
+    for (int e = 0; e < 8; ++e) cs[e] = 1.f, sn[e] = 0.f;
+#endif
     for (int g = wave * 4 + sub; g < G; g += 4 * kWaves)  // a 16-lane group per head
       *reinterpret_cast<uint4*>(&q_lds[g * D + sl * 8]) =
           head_slice<D, true>(row + (size_t)(h0 + g) * D, sl, p.qn, p.eps, cs, sn);
@@ -874,6 +877,10 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
     __builtin_amdgcn_wave_barrier();
     EXO_LOAD_TILE(k0 + TK)
 
+#if (EXO_SDPA_ABL & 4)  // timing only: tiles travel to LDS, nothing is computed
+    o[0][0] += bf2f(k_t[lane]) + bf2f(v_t[lane]);
+    continue;
+#endif
     floatx16 sc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) sc[e] = 0.f;
@@ -1001,6 +1008,10 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
       acc += red[w][g][e] * scw;
       lsum += red[w][g][D + 1] * scw;
     }
+#if (EXO_SDPA_ABL & 2)  // timing only: no hand-over, every split writes its own result
+    p.out[qrow + (size_t)(h0 + g) * D + e] = f2bf(acc / lsum);
+    continue;
+#endif
     float* dst = p.ws + ((size_t)(b * p.Hq + h0 + g) * p.splits + blockIdx.x) * (D + 2);
     st_dev(dst + e, acc);
     if (e == 0) {
@@ -1008,6 +1019,9 @@ __global__ __launch_bounds__(kThreads, 2) void sdpa_decode_mfma_kernel(const Sdp
       st_dev(dst + D + 1, lsum);
     }
   }
+#if (EXO_SDPA_ABL & 2)
+  return;
+#endif
   // the last workgroup of this (sequence, kv head) merges the splits (see sdpa_kernel)
   wait_own_stores_done();
   __syncthreads();

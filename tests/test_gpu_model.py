@@ -240,6 +240,44 @@ def test_decode_step_first_replay_matches_call(ckpt, device):
     assert got_toks == want_toks
 
 
+def test_graph_capture_keeps_the_garbage_collector_out(device):
+    """Recording a step into a graph with garbage waiting to be collected - cycles that own
+    pinned host memory and events, as a finished batch engine leaves behind: nothing is
+    collected while the stream records (a collection there aborted the process), the
+    collector is back afterwards, and the replays give the eager result."""
+    import gc
+    from exo_amd.model import capture_graph
+
+    class Node:
+        pass
+
+    def litter():
+        for _ in range(50):
+            a, b = Node(), Node()
+            a.other, b.other = b, a
+            a.buf = torch.empty(1024, dtype=torch.int32).pin_memory()
+            a.ev = torch.cuda.Event()
+            a.buf.copy_(torch.zeros(1024, dtype=torch.int32, device=device), non_blocking=True)
+            a.ev.record()
+    assert gc.isenabled()
+    x = torch.arange(4096, dtype=torch.float32, device=device)
+    y = torch.empty_like(x)
+    litter()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with capture_graph(g):
+        assert not gc.isenabled()
+        litter_in_capture = [dict(k=i) for i in range(5000)]  # allocations that would trigger a collection
+        torch.mul(x, 2.0, out=y)
+        del litter_in_capture
+    assert gc.isenabled()
+    for rep in range(3):
+        y.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, x * 2.0), rep
+
+
 def test_decode_step_recaptures_when_the_context_regime_changes(ckpt, device):
     """The attention launch of a decode step is laid out per context regime (the host's count
     of the longest sequence against ATTN_LONG_KEYS): graph replays across the threshold give
