@@ -738,8 +738,10 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     uint4 raw[ITERS][4], nwv[ITERS][4];
-    // without a norm the weight words are loaded from the activations and not used: a
-    // branch per load would split the requests over basic blocks
+    // routing instance: without a norm the weight words are loaded from the activations and
+    // not used - a branch per load would split the requests over basic blocks, and the wait
+    // for the logits must not cover them.  (The plain instance keeps the branch: the extra
+    // loads cost the o projection, which has no norm, 0.26 of its 4.65 us.)
     const bf16_t* nw_src = p.norm_w ? p.norm_w : xin;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j)
@@ -747,7 +749,7 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
       for (int t = 0; t < 4; ++t) {
         const int wi = 4 * chunk_of<BITS, ITERS>(j, lane) + t;
         raw[j][t] = load_word_x<BITS>(xin, wi);
-        nwv[j][t] = load_word_x<BITS>(nw_src, wi);
+        if (ROUTE || p.norm_w) nwv[j][t] = load_word_x<BITS>(nw_src, wi);
       }
     // (the routing waits for its logits only: the activation loads above go out before that wait)
     if (ROUTE) __builtin_amdgcn_sched_barrier(0);
