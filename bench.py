@@ -76,6 +76,21 @@ def measure_kernels(model, torch, reps: int = 20):
         return "qmv_rows_kernel<%d,1,%d,%d,false>" % (c.bits, nmat, K * c.bits // 8 // 1024)
 
     nw, eps = torch.ones(H, **bf), c.rms_norm_eps
+
+    def timed_rounds(graph, launches, rounds=5):
+        """Average launch duration in us: `rounds` timed regions of `reps` replays each,
+        the median region (the first one after a capture runs 2-3 % slow)."""
+        avg = []
+        for _ in range(rounds):
+            st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            st.record()
+            for _ in range(reps):
+                graph.replay()
+            en.record()
+            torch.cuda.synchronize()
+            avg.append(st.elapsed_time(en) * 1e3 / (reps * launches))
+        return sorted(avg)[len(avg) // 2]
+
     groups = {
         "norm_gate_up_swiglu": (lambda L: ops.qmv_swiglu(xh, L.gate, L.up, out=y_i, norm_weight=nw, eps=eps),
                                 2 * qbytes(I, H, c.bits) + 2 * (2 * H + I), kernel_name(2, H)),
@@ -98,13 +113,7 @@ def measure_kernels(model, torch, reps: int = 20):
                 fn(L)
         g.replay()
         torch.cuda.synchronize()
-        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        st.record()
-        for _ in range(reps):
-            g.replay()
-        en.record()
-        torch.cuda.synchronize()
-        us = st.elapsed_time(en) * 1e3 / (reps * len(model.layers))
+        us = timed_rounds(g, len(model.layers))
         out.append(dict(name=name, kernel=kname, launches_per_token=len(model.layers),
                         bytes_per_launch=nbytes, avg_us=us, GBps=nbytes / us * 1e-3))
     # lm_head: once per token, with 4 GB of layer weights streamed since its last use, so
@@ -124,13 +133,7 @@ def measure_kernels(model, torch, reps: int = 20):
             ops.quantized_matmul(xh, q, out=y_v, norm_weight=nw, eps=eps)
     g.replay()
     torch.cuda.synchronize()
-    st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    st.record()
-    for _ in range(reps):
-        g.replay()
-    en.record()
-    torch.cuda.synchronize()
-    us = st.elapsed_time(en) * 1e3 / (reps * len(heads))
+    us = timed_rounds(g, len(heads))
     del heads
     nbytes = qbytes(c.vocab_size, H, c.bits) + 2 * (2 * H + c.vocab_size)
     out.append(dict(name="norm_lm_head", kernel=kernel_name(1, H), launches_per_token=1,
