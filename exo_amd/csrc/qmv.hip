@@ -1200,7 +1200,7 @@ int launch_ksplit(const QmvParams& p, hipStream_t st) {
 //   out[t,n] = bf16( bf16( sum_j bf16( bf16(W[e_j][n,:] . x[t,j,:]) * score[t,j] ) ) + res[t,n] )
 // - the same rounding points as exo_gather_qmv followed by exo_moe_combine.
 // blockIdx.y = token; a workgroup has one wave per expert slot.  Wave j stages ITS
-// activation row x[t,j,:], multiplies kDownRW (1 or 2) sets of 64/LPR rows of expert e_j (all its
+// activation row x[t,j,:], multiplies kDownRW (1, 2 or 4) sets of 64/LPR rows of expert e_j (all its
 // loads in flight from the start) and leaves bf16(bf16(dot) * score_j) in LDS; the first
 // wave adds the k contributions in slot order.  The launch is latency-bound, hence the
 // many short waves.
@@ -2037,11 +2037,16 @@ extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, cons
   p.lpr_log2 = pl.lpr_log2;
   p.iters = pl.iters;
   const int rpwi = 64 >> pl.lpr_log2;
-  // two row sets per wave only while that leaves 512 workgroups per token: the launch is
-  // latency-bound and wants a wide grid (Qwen3-30B, 2048 outputs in sets of 8: one set,
-  // 256 workgroups, 482 -> 509 tok/s; Qwen3-235B, 4096 outputs in sets of 2: two sets, 1024
-  // workgroups - one set per wave loses 5 % there, four lose 6 %)
-  const int rw = exo_ceil_div(N, 2 * rpwi) >= 512 ? 2 : 1;
+  // as many row sets per wave (4, 2 or 1) as leave 512 workgroups per token: every wave stages
+  // its slot's activation row, which more rows amortise, but the launch is latency-bound and
+  // wants a wide grid (Qwen3-30B, 2048 outputs in sets of 8: one set, 256 workgroups, 482 ->
+  // 509 tok/s over two; Qwen3-235B, 4096 outputs in sets of 2, whole step: one set 457 tok/s,
+  // two 478, four - 512 workgroups - 490, eight 481)
+#ifdef EXO_DOWN_RW
+  const int rw = EXO_DOWN_RW;
+#else
+  const int rw = exo_ceil_div(N, 4 * rpwi) >= 512 ? 4 : (exo_ceil_div(N, 2 * rpwi) >= 512 ? 2 : 1);
+#endif
   const dim3 grid(exo_ceil_div(N, rw * rpwi), T);
   const size_t lds = (size_t)topk * ((size_t)p.wpr * 16 + (size_t)(p.wpr / 4) * 8);
   exo_note_variant("moe_down_combine<%d,%d,%d> grid=%dx%d", bits, rw, pl.iters, (int)grid.x, (int)grid.y);
@@ -2054,6 +2059,8 @@ extern "C" int exo_gather_qmv_combine(const uint16_t* x, const uint32_t* w, cons
   EXO_DOWN_ITERS(4, 2)
   EXO_DOWN_ITERS(8, 1)
   EXO_DOWN_ITERS(8, 2)
+  EXO_DOWN_ITERS(4, 4)
+  EXO_DOWN_ITERS(8, 4)
 #undef EXO_DOWN_ITERS
 #undef EXO_DOWN_CASE
   EXO_CHECK_LAUNCH("exo_gather_qmv_combine");
