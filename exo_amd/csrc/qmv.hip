@@ -829,242 +829,6 @@ __global__ __launch_bounds__(kThreads) void qmv_rows_kernel(const QmvParams p) {
 }
 
 
-// The single-round kernel: EXO_QMV_ONCE_GRID workgroups (one per CU) of up to
-// EXO_QMV_ONCE_MAXW waves, each wave at most RW rows and at most 16 KiB of codes.
-// (off: in the whole decode step the single-round kernel loses - Llama-3.1-8B 1.533 against
-// 1.501 ms per token on one box, repeatedly - although a graph of its launches alone is level
-// or ahead of the row kernel's: 16.0 against 16.5 us for the gate/up pair, 6.0 against 6.4)
-#ifndef EXO_QMV_ONCE
-#define EXO_QMV_ONCE 0
-#endif
-#ifndef EXO_QMV_ONCE_GRID
-#define EXO_QMV_ONCE_GRID 256
-#endif
-#ifndef EXO_QMV_ONCE_MAXW
-#define EXO_QMV_ONCE_MAXW 16
-#endif
-#ifndef EXO_QMV_ONCE_MINRW
-#define EXO_QMV_ONCE_MINRW 1
-#endif
-// rows requested before the first product (0: all).  Measured on the 14336x4096 gate/up pair
-// with the fused norm (4 rows per wave): all four 20.4 us, two 17.3, one 16.0 - the more
-// loads a wave queues in front of the ones it needs first, the later those arrive.
-#ifndef EXO_QMV_ONCE_AHEAD
-#define EXO_QMV_ONCE_AHEAD 1
-#endif
-#ifndef EXO_QMV_ONCE_XBARRIER
-#define EXO_QMV_ONCE_XBARRIER 1
-#endif
-// ---------------------------------------------------------------------------
-// One activation row against a matrix (or the gate/up pair) small enough that ONE round of
-// workgroups - gridDim.x of them, blockDim.x / 64 waves each, all resident at once - covers
-// it with at most RW rows per wave: every wave requests ALL of its weights, scales and
-// biases (and the residual values of its rows) right behind the activation loads, before
-// anything is waited for.  The whole matrix is then in flight from the first microsecond
-// and streams at the memory's rate while the workgroup normalises and stages the
-// activations ONCE; a wave consumes its rows in the order they were requested (the waits are
-// static counts).  No refill loop, no second round of workgroups whose activation loads
-// would queue behind their neighbours' weight loads.
-template <int BITS, int NMAT, int ITERS, int RW>
-__global__ __launch_bounds__(1024) void qmv_once_kernel(const QmvParams p) {
-  extern __shared__ uint4 smem[];
-  constexpr int GSHIFT = (BITS == 4) ? 1 : 2;
-  constexpr int UG = 64 >> GSHIFT;  // scale elements per unit
-  constexpr int CPR = 64 * ITERS, WPR = 256 * ITERS;
-  constexpr int UW = RW * ITERS;  // units per wave and matrix
-  uint4* xs = smem;                                       // [WPR]
-  float2* sx = reinterpret_cast<float2*>(smem + WPR);     // [CPR]
-  __shared__ float s_red[16];
-
-  const int tid = threadIdx.x, nthreads = blockDim.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nw = nthreads >> 6;
-  const int G = p.K >> 6;
-
-  // balanced contiguous row range of this wave (at most RW rows: the launcher's rule)
-  const int nwaves = gridDim.x * nw;
-  const int gw = blockIdx.x * nw + wave;
-  const int base = p.N / nwaves, rem = p.N - base * nwaves;
-  const int r0 = gw * base + min(gw, rem);
-  const int nrows = base + (gw < rem ? 1 : 0);
-  const int r1 = r0 + nrows;
-
-  // 1. the activations (and norm weights) of this thread's words (at most XW: the launcher
-  // gives a workgroup WPR / XW threads or more)
-  constexpr int XW = ITERS <= 2 ? ITERS : 2;
-  uint4 xraw[XW], nwv[XW];
-#pragma unroll
-  for (int it = 0; it < XW; ++it) {
-    const int wi = tid + it * nthreads;
-    xraw[it] = make_uint4(0, 0, 0, 0);
-    nwv[it] = make_uint4(0, 0, 0, 0);
-    if (wi < WPR) {
-      xraw[it] = load_word_x<BITS>(p.x, wi);
-      if (p.norm_w) nwv[it] = load_word_x<BITS>(p.norm_w, wi);
-    }
-  }
-
-  // every wave's activation loads are in the memory pipeline before any weight load: a
-  // late wave's activations would otherwise queue behind its neighbours' weights, and the
-  // whole workgroup waits for them
-#if EXO_QMV_ONCE_XBARRIER
-  __syncthreads();
-#endif
-
-  // 2. what this wave will multiply by: the first AHEAD rows now, the others as rows finish
-  uint4 wv[NMAT][UW];
-  uint32_t sv[NMAT][UW], bv[NMAT][UW];
-  bf16_t res = 0;
-  const int rl = max(r1 - 1, 0);  // rows past the range re-read its last row (dropped later)
-  if (NMAT == 1 && p.residual && lane < RW) res = p.residual[min(r0 + lane, rl)];
-  auto issue_row = [&](int r) {
-#pragma unroll
-    for (int j = 0; j < ITERS; ++j) {
-      const int i = r * ITERS + j;
-      const int row = min(r0 + r, rl);
-      const bool paired = !((ITERS & 1) && j == ITERS - 1);
-      const size_t wofs = (size_t)row * (ITERS * 1024) + chunk_of<BITS, ITERS>(j, lane) * 16;
-#pragma unroll
-      for (int a = 0; a < NMAT; ++a) {
-        wv[a][i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p.w[a]) + wofs);
-        if (paired) {
-          if ((j & 1) == 0) {
-            const size_t sofs = ((size_t)row * G + UG * j) * 2 + (lane >> GSHIFT) * 4;
-            sv[a][i] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(p.s[a]) + sofs);
-            bv[a][i] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(p.b[a]) + sofs);
-          }
-        } else {
-          const size_t sofs = ((size_t)row * G + UG * j + (lane >> GSHIFT)) * 2;
-          sv[a][i] = *reinterpret_cast<const bf16_t*>(reinterpret_cast<const char*>(p.s[a]) + sofs);
-          bv[a][i] = *reinterpret_cast<const bf16_t*>(reinterpret_cast<const char*>(p.b[a]) + sofs);
-        }
-      }
-    }
-  };
-  constexpr int AHEAD = (EXO_QMV_ONCE_AHEAD > 0 && EXO_QMV_ONCE_AHEAD < RW) ? EXO_QMV_ONCE_AHEAD : RW;
-#pragma unroll
-  for (int r = 0; r < AHEAD; ++r) issue_row(r);
-
-  // 3. normalise (optional) and stage the activations in dot2 register order
-  if (p.norm_w) {
-    float ss = 0.f;
-#pragma unroll
-    for (int it = 0; it < XW; ++it) ss += sumsq_word<BITS>(xraw[it]);
-    ss = wave_sum(ss);
-    if (lane == 0) s_red[wave] = ss;
-    __syncthreads();
-    // (a wave reduction over the per-wave sums: a loop over them made the compiler shuffle the
-    // registers that the weight loads are landing in, i.e. wait for those loads here)
-    float tot = lane < nw ? s_red[lane] : 0.f;
-    tot = wave_sum_to_lane63(tot);
-    tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, tot), 63));
-    const float inv = rsqrtf(tot / (float)p.K + p.eps);
-#pragma unroll
-    for (int it = 0; it < XW; ++it) norm_word<BITS>(xraw[it], nwv[it], inv);
-  }
-#pragma unroll
-  for (int it = 0; it < XW; ++it) {
-    const int wi = tid + it * nthreads;
-    const int c = wi >> 2, t = wi & 3;
-    int j, sl;
-    unit_lane_of<BITS, ITERS>(c, j, sl);
-    float stored, truesum;
-    const uint4 o = permute_word<BITS>(xraw[it], stored, truesum);
-    stored += __shfl_xor(stored, 1, 64);
-    truesum += __shfl_xor(truesum, 1, 64);
-    stored += __shfl_xor(stored, 2, 64);
-    truesum += __shfl_xor(truesum, 2, 64);
-    if (wi < WPR) {
-      xs[((j << 2) + t) * 64 + sl] = o;
-      if (t == 0) sx[j * 64 + sl] = make_float2(128.f * stored, truesum);
-    }
-  }
-  __syncthreads();
-  if (nrows <= 0) return;
-
-  // 4. short rows: the activations of the lane move into registers once
-  constexpr bool X_IN_REGS = ITERS <= 2;
-  uint4 xr[X_IN_REGS ? ITERS : 1][4];
-  float2 sxr[X_IN_REGS ? ITERS : 1];
-  if (X_IN_REGS) {
-#pragma unroll
-    for (int j = 0; j < ITERS; ++j) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) xr[X_IN_REGS ? j : 0][t] = xs[(j * 4 + t) * 64 + lane];
-      sxr[X_IN_REGS ? j : 0] = sx[j * 64 + lane];
-    }
-  }
-  uint32_t kmask = 0x000F000Fu, kmagic = 0x43004300u;
-  asm volatile("" : "+s"(kmask));
-  asm volatile("" : "+v"(kmagic));
-
-  // 5. the rows, in the order their loads were requested
-#pragma unroll
-  for (int r = 0; r < RW; ++r) {
-    const int row = r0 + r;
-    if (row < r1) {
-      float acc[NMAT];
-#pragma unroll
-      for (int a = 0; a < NMAT; ++a) acc[a] = 0.f;
-#pragma unroll
-      for (int j = 0; j < ITERS; ++j) {
-        const int i = r * ITERS + j;
-        const float2 sm = X_IN_REGS ? sxr[X_IN_REGS ? j : 0] : sx[j * 64 + lane];
-        float d[NMAT];
-#pragma unroll
-        for (int a = 0; a < NMAT; ++a) d[a] = -sm.x;
-#ifdef EXO_QMV_ONCE_NOMATH  // timing-only build (wrong results): loads consumed, no products
-#pragma unroll
-        for (int a = 0; a < NMAT; ++a)
-          d[a] += __builtin_bit_cast(float, wv[a][i].x ^ wv[a][i].y ^ wv[a][i].z ^ wv[a][i].w);
-#else
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const uint4 xv = X_IN_REGS ? xr[X_IN_REGS ? j : 0][t] : xs[(j * 4 + t) * 64 + lane];
-#pragma unroll
-          for (int a = 0; a < NMAT; ++a) {
-            uint32_t pr[4];
-            unpack_word_r(reinterpret_cast<const uint32_t*>(&wv[a][i])[t], kmask, kmagic, pr);
-            d[a] = dot2_bf16(pr[0], xv.x, d[a]);
-            d[a] = dot2_bf16(pr[1], xv.y, d[a]);
-            d[a] = dot2_bf16(pr[2], xv.z, d[a]);
-            d[a] = dot2_bf16(pr[3], xv.w, d[a]);
-          }
-        }
-#endif
-#pragma unroll
-        for (int a = 0; a < NMAT; ++a) {
-          const bool hi = (j & 1) && !((ITERS & 1) && j == ITERS - 1);
-          const int is = hi ? i - 1 : i;
-          const float sc = hi ? bf_hi(sv[a][is]) : bf_lo(sv[a][is]);
-          const float bi = hi ? bf_hi(bv[a][is]) : bf_lo(bv[a][is]);
-          acc[a] = fmaf(sc, d[a], acc[a]);
-          acc[a] = fmaf(bi, sm.y, acc[a]);
-        }
-      }
-      float rsum[NMAT];
-#pragma unroll
-      for (int a = 0; a < NMAT; ++a) rsum[a] = wave_sum_to_lane63(acc[a]);
-      const float resv = bf2f((bf16_t)__builtin_amdgcn_readlane((int)res, r));
-      if (lane == 63) {
-        float out;
-        if (NMAT == 2) {
-          const float g = bf2f(f2bf(rsum[0])), up = bf2f(f2bf(rsum[NMAT - 1]));
-          out = g / (1.f + __expf(-g)) * up;
-        } else {
-          out = rsum[0];
-          if (p.residual) out = bf2f(f2bf(out)) + resv;
-        }
-        p.y[row] = f2bf(out);
-      }
-    }
-    if (r + AHEAD < RW) {
-      if (r0 + r + AHEAD < r1) issue_row(r + AHEAD);
-    }
-  }
-}
-
 // ---------------------------------------------------------------------------
 // Long rows (4 or more KiB-units per row, one activation row, no fused norm): the NW
 // waves of a workgroup split K.  Wave w owns unit w of every row of the workgroup's row
@@ -1466,86 +1230,8 @@ int launch_rows(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
   return EXO_OK;
 }
 
-// 16-byte weight loads a lane holds at once: 16 where the activations sit in registers beside
-// them (rows of up to two units), 14 for longer rows (16 spill)
-template <int ITERS>
-constexpr int kOnceMaxUnits = ITERS <= 2 ? 16 : 14;
-
-template <int BITS, int NMAT, int ITERS, int RW>
-int launch_once_rw(const QmvParams& p, int nw, hipStream_t st) {
-  if constexpr (RW * ITERS * NMAT <= kOnceMaxUnits<ITERS>) {
-    auto kern = qmv_once_kernel<BITS, NMAT, ITERS, RW>;
-    const size_t lds = (size_t)256 * ITERS * 16 + (size_t)64 * ITERS * 8;
-    static bool attr_done = false;
-    if (!attr_done && lds > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) {
-        exo_set_error("exo_qmv: cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
-        return EXO_ERR_HIP;
-      }
-      attr_done = true;
-    }
-    exo_note_variant("qmv_once<%d,%d,%d,%d> grid=%d waves=%d", BITS, NMAT, ITERS, RW,
-                     EXO_QMV_ONCE_GRID, nw);
-    kern<<<dim3(EXO_QMV_ONCE_GRID), dim3(64 * nw), lds, st>>>(p);
-    return EXO_OK;
-  } else {
-    (void)p; (void)nw; (void)st;
-    exo_set_error("exo_qmv: internal: no single-round instance for %d rows per wave", RW);
-    return EXO_ERR_ARG;
-  }
-}
-
-// rows per wave and waves per workgroup of the single-round kernel, or false: the matrix
-// does not fit one round
-template <int NMAT, int ITERS>
-bool once_shape(int N, int* rw_out, int* nw_out) {
-  if (!EXO_QMV_ONCE) return false;
-  const int rows_wg = (N + EXO_QMV_ONCE_GRID - 1) / EXO_QMV_ONCE_GRID;
-  for (int rw = EXO_QMV_ONCE_MINRW; rw <= 4; rw *= 2) {
-    if (rw * ITERS * NMAT > kOnceMaxUnits<ITERS>) break;
-    int nw = (rows_wg + rw - 1) / rw;
-    // (enough threads to stage the activations with two words each at most)
-    const int stage_w = ITERS <= 2 ? 4 : 2 * ITERS;
-    if (nw < stage_w) nw = stage_w;
-    if (nw <= EXO_QMV_ONCE_MAXW) {
-      *rw_out = rw;
-      *nw_out = nw;
-      return true;
-    }
-  }
-  return false;
-}
-
-template <int BITS, int NMAT, int ITERS>
-int launch_once(const QmvParams& p, int rw, int nw, hipStream_t st) {
-  switch (rw) {
-    case 1: return launch_once_rw<BITS, NMAT, ITERS, 1>(p, nw, st);
-    case 2: return launch_once_rw<BITS, NMAT, ITERS, 2>(p, nw, st);
-    default: return launch_once_rw<BITS, NMAT, ITERS, 4>(p, nw, st);
-  }
-}
-
 template <int BITS, int MT, int NMAT>
 int launch_one(const QmvParams& p, const Plan& pl, int pairs, hipStream_t st) {
-  if constexpr (MT == 1) {
-   // (launches with the fused RMSNorm: the norm and the staging happen once per CU instead of
-   // once per short-lived workgroup - the gate/up pair 16.5 -> 16.0 us, 6144x4096 6.46 -> 6.01;
-   // without a norm the row kernel below is level or ahead)
-   if (p.M == 1 && pairs == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.idx && !p.each_row && !p.route &&
-       p.norm_w) {
-    int rw, nw;
-    switch (pl.iters) {
-      case 1: if (once_shape<NMAT, 1>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 1>(p, rw, nw, st); break;
-      case 2: if (once_shape<NMAT, 2>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 2>(p, rw, nw, st); break;
-      case 4: if (once_shape<NMAT, 4>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 4>(p, rw, nw, st); break;
-      case 7: if (once_shape<NMAT, 7>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 7>(p, rw, nw, st); break;
-      case 8: if (once_shape<NMAT, 8>(p.N, &rw, &nw)) return launch_once<BITS, NMAT, 8>(p, rw, nw, st); break;
-      default: break;  // (14 units per row: more registers than a single round leaves)
-    }
-   }
-  }
   if (MT == 1 && NMAT == 1 && pl.lpr_log2 == 6 && !pl.ragged && !p.norm_w && !p.idx && !p.each_row &&
       !p.route && p.M == 1) {
     // measured against the row kernel: ahead at 14 units per row (8-bit, K = 14336: 17.0
