@@ -274,7 +274,7 @@ def test_qmm_split_k(device, bits, M, N, K):
     over workgroups and the float32 partial tiles are added by a second launch.  Against
     the oracle, against the
     unsplit kernel (same products, another summation order: a few bf16 ulps at most),
-    with the residual, and twice in a row (the counters return to zero).  The last three
+    with the residual, and three times in a row with identical bits.  The last three
     shapes have K ranges of 1024 and take the wide tile with eight waves (two teams on the
     halves of a range)."""
     trip = rand_quantized(N, K, bits, seed=M + N)
@@ -282,9 +282,12 @@ def test_qmm_split_k(device, bits, M, N, K):
     r = rand_bf16((M, N), seed=M + 5)
     qw, xt, rt = t_qw(trip, bits, device), t_bf16(x, device), t_bf16(r, device)
     want = affine.qmm(x, *trip, 64, bits)
-    for _ in range(2):
+    first = None
+    for _ in range(3):
         got = ops.quantized_matmul(xt, qw)
         assert_close(n_f32(got), want, what=f"qmm split-K {M}x{N}x{K} b{bits}")
+        first = got.clone() if first is None else first
+        assert torch.equal(got.view(torch.int16), first.view(torch.int16))
     unsplit = ops.qmm(xt, qw)
     assert_close(n_f32(got), n_f32(unsplit), rtol=1e-2, what="split vs unsplit")
     got_r = n_f32(ops.quantized_matmul(xt, qw, residual=rt))
